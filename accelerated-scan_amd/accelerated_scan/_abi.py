@@ -1,0 +1,132 @@
+"""ctypes binding of the HIP scan library (C ABI in ``include/ascan.h``).
+
+This is the only place that touches the shared library.  There is no fallback:
+if ``libascan.so`` is missing, ``load()`` raises, and so does every operator
+built on it.  The library is searched for next to this file, or at the path in
+the ``ASCAN_LIBRARY`` environment variable.
+"""
+
+import ctypes
+import os
+from pathlib import Path
+
+import torch
+
+ABI_VERSION = 1
+
+# ascan_dtype codes of include/ascan.h
+F32, BF16, F16, C64 = 0, 1, 2, 3
+
+DTYPE_CODES = {
+    torch.float32: F32,
+    torch.bfloat16: BF16,
+    torch.float16: F16,
+    torch.complex64: C64,
+}
+
+_SIGNATURES = {
+    # name: (restype, argtypes)
+    "ascan_forward": (
+        ctypes.c_int,
+        [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p,
+         ctypes.c_int64, ctypes.c_int64, ctypes.c_int, ctypes.c_int, ctypes.c_void_p],
+    ),
+    "ascan_backward": (
+        ctypes.c_int,
+        [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p,
+         ctypes.c_int64, ctypes.c_int64, ctypes.c_int, ctypes.c_void_p],
+    ),
+    "ascan_status_string": (ctypes.c_char_p, [ctypes.c_int]),
+    "ascan_last_hip_error": (ctypes.c_int, []),
+    "ascan_abi_version": (ctypes.c_int, []),
+}
+
+_lib = None
+
+
+def library_path() -> Path:
+    override = os.environ.get("ASCAN_LIBRARY")
+    if override:
+        return Path(override)
+    return Path(__file__).resolve().parent / "libascan.so"
+
+
+def load() -> ctypes.CDLL:
+    """Load the shared library once and declare its prototypes."""
+    global _lib
+    if _lib is not None:
+        return _lib
+    path = library_path()
+    if not path.exists():
+        raise ImportError(
+            f"accelerated_scan: HIP library not found at {path}; build it with "
+            f"`make -C {Path(__file__).resolve().parent.parent}` (needs hipcc, targets gfx950)"
+        )
+    lib = ctypes.CDLL(str(path))
+    for name, (restype, argtypes) in _SIGNATURES.items():
+        fn = getattr(lib, name)
+        fn.restype = restype
+        fn.argtypes = argtypes
+    version = lib.ascan_abi_version()
+    if version != ABI_VERSION:
+        raise ImportError(f"accelerated_scan: {path} has ABI version {version}, expected {ABI_VERSION}")
+    _lib = lib
+    return lib
+
+
+def exported_symbols():
+    """Names the binding expects the library to export."""
+    return tuple(_SIGNATURES)
+
+
+def check(status: int) -> None:
+    """Turn a non-zero ascan_status into RuntimeError (the reference raises
+    RuntimeError through TORCH_CHECK, accelerated_scan/warp.cuh:379,391,396-421)."""
+    if status == 0:
+        return
+    lib = load()
+    text = lib.ascan_status_string(status).decode()
+    if status == 5:
+        text += f" (hipError_t {lib.ascan_last_hip_error()})"
+    raise RuntimeError(f"accelerated_scan: {text}")
+
+
+def dtype_code(dtype: torch.dtype) -> int:
+    try:
+        return DTYPE_CODES[dtype]
+    except KeyError:
+        raise RuntimeError(
+            f"accelerated_scan: unsupported tensor dtype {dtype}: "
+            "expecting bfloat16, float16, float32 or complex64"
+        ) from None
+
+
+def _stream_handle(device: torch.device) -> int:
+    return torch.cuda.current_stream(device).cuda_stream
+
+
+def forward(gates, tokens, out, reverse: bool) -> None:
+    """Enqueue ascan_forward on the current stream of the tensors' device."""
+    lib = load()
+    rows = tokens.numel() // tokens.shape[-1] if tokens.shape[-1] else 0
+    with torch.cuda.device(tokens.device):
+        status = lib.ascan_forward(
+            gates.data_ptr(), tokens.data_ptr(), out.data_ptr(),
+            rows, tokens.shape[-1], dtype_code(tokens.dtype), int(bool(reverse)),
+            _stream_handle(tokens.device),
+        )
+    check(status)
+
+
+def backward(gates, states, grad_out, d_gates, d_tokens) -> None:
+    """Enqueue ascan_backward on the current stream of the tensors' device."""
+    lib = load()
+    rows = gates.numel() // gates.shape[-1] if gates.shape[-1] else 0
+    with torch.cuda.device(gates.device):
+        status = lib.ascan_backward(
+            gates.data_ptr(), states.data_ptr(), grad_out.data_ptr(),
+            d_gates.data_ptr(), d_tokens.data_ptr(),
+            rows, gates.shape[-1], dtype_code(gates.dtype),
+            _stream_handle(gates.device),
+        )
+    check(status)

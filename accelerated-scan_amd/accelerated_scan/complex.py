@@ -1,0 +1,85 @@
+"""Complex64 scan on the HIP backend (operator of accelerated_scan/complex.py:157-239).
+
+``forget`` must be complex; ``inputs`` may be complex or real (a real tensor
+is read as having zero imaginary part and receives a real gradient).  The
+backward pass follows complex.py:79-92: with g the adjoint of the states,
+``g[t] = d_output[t] + conj(forget[t+1]) * g[t+1]``, ``d_inputs = g`` and
+``d_forget[t] = g[t] * conj(states[t-1])``.
+"""
+
+import torch
+
+from . import _abi
+
+
+def _require(cond: bool, what: str) -> None:
+    if not cond:
+        raise RuntimeError(f"accelerated_scan: expected {what}")
+
+
+def _launch_forward(forget, inputs, states):
+    for t, name in ((forget, "forget"), (inputs, "inputs"), (states, "states")):
+        _require(t.is_cuda, f"{name} to be a device tensor")
+        _require(t.dtype == torch.complex64, f"{name} to be complex64")
+        _require(t.device == forget.device, f"{name} to be on the device of forget")
+    _abi.forward(forget, inputs, states, False)
+
+
+def _launch_backward(forget, states, d_output, d_forget, d_inputs):
+    for t, name in ((forget, "forget"), (states, "states"), (d_output, "d_output")):
+        _require(t.is_cuda, f"{name} to be a device tensor")
+        _require(t.dtype == torch.complex64, f"{name} to be complex64")
+        _require(t.shape == forget.shape, f"{name} to have the shape of forget")
+        _require(t.device == forget.device, f"{name} to be on the device of forget")
+    _abi.backward(forget, states, d_output, d_forget, d_inputs)
+
+
+class Scan(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, forget, inputs):
+        if not torch.is_complex(forget):
+            raise TypeError("forget must be a complex tensor")
+        real_inputs = not torch.is_complex(inputs)
+        B, C, T = forget.shape
+        assert inputs.shape == (B, C, T)
+        assert forget.is_contiguous()
+        assert inputs.is_contiguous()
+
+        if real_inputs:
+            inputs = torch.complex(inputs, torch.zeros_like(inputs))
+
+        states = torch.empty_like(inputs)
+        _launch_forward(forget, inputs, states)
+
+        ctx.save_for_backward(forget, states)
+        ctx.real_inputs = real_inputs
+        return states
+
+    @staticmethod
+    def backward(ctx, d_output):
+        forget, states = ctx.saved_tensors
+
+        d_output = d_output.contiguous()
+        assert forget.is_contiguous()
+        assert states.is_contiguous()
+
+        d_forget = torch.empty_like(forget)
+        d_inputs = torch.empty_like(states)
+        _launch_backward(forget, states, d_output, d_forget, d_inputs)
+
+        if ctx.real_inputs:
+            d_inputs = d_inputs.real
+        return d_forget, d_inputs
+
+
+def scan(forget, inputs):
+    """Solve ``x[t] = forget[t] * x[t-1] + inputs[t]`` over complex numbers.
+
+    Arguments:
+        forget (torch.Tensor): shape (B, C, T), complex64, contiguous.
+        inputs (torch.Tensor): shape (B, C, T), complex64 or float32, contiguous.
+
+    Returns:
+        (torch.Tensor): complex64 states of shape (B, C, T).
+    """
+    return Scan.apply(forget, inputs)

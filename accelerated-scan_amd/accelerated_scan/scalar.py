@@ -1,0 +1,44 @@
+"""Any-length real scan with the argument names of accelerated_scan/scalar.py.
+
+The reference implements this module with Triton kernels (scalar.py:16-86);
+here it is the same HIP backend as ``warp``, which already accepts every
+sequence length.  ``Scan`` saves ``(forget, states)`` and returns
+``(d_forget, d_inputs)`` exactly as scalar.py:89-126 does.
+"""
+
+import torch
+
+from . import warp
+
+
+class Scan(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, forget, inputs):
+        B, C, T = forget.shape
+        assert inputs.shape == (B, C, T)
+        assert forget.is_contiguous()
+        assert inputs.is_contiguous()
+
+        states = torch.empty_like(inputs)
+        warp.warpscan_forward(forget, inputs, states, False)
+
+        ctx.save_for_backward(forget, states)
+        return states
+
+    @staticmethod
+    def backward(ctx, d_output):
+        forget, states = ctx.saved_tensors
+
+        d_output = d_output.contiguous()
+        assert forget.is_contiguous()
+        assert states.is_contiguous()
+
+        d_forget = torch.empty_like(forget)
+        d_inputs = torch.empty_like(states)
+        warp.warpscan_backward(forget, states, d_output, d_forget, d_inputs)
+        return d_forget, d_inputs
+
+
+def scan(forget, inputs):
+    """Solve ``x[t] = forget[t] * x[t-1] + inputs[t]`` for (B, C, T) tensors of any T."""
+    return Scan.apply(forget, inputs)

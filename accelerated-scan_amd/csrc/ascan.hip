@@ -1,0 +1,876 @@
+// First-order linear recurrence (scan) kernels for gfx950 (MI355X) and the
+// C ABI declared in include/ascan.h.
+//
+//   forward :  x[t] = gate[t] * x[t-1] + token[t]
+//   backward:  g[t] = grad_out[t] + conj(gate[t+1]) * g[t+1]
+//              d_tokens = g,  d_gates[t] = g[t] * conj(x[t-1])
+//
+// Behaviour follows the reference operator (accelerated_scan/warp.cuh:49-223
+// for the real dtypes, accelerated_scan/complex.py:20-154 for complex64); the
+// decomposition below is specific to CDNA wave64 hardware:
+//
+//   * A row is cut into tiles; inside a tile every wave owns a contiguous
+//     sub-tile of U*64 16-byte vectors.  Lane l of the wave loads vector
+//     j*64+l of the sub-tile (j = 0..U-1), so each load instruction of the
+//     wave covers one contiguous KiB.
+//   * Each lane folds its vector into one (A, X) pair, A = product of gates,
+//     X = local scan end value.  The 64 pairs are scanned with 6 DPP steps
+//     (row_shr 1,2,4,8, row_bcast 15, row_bcast 31): no LDS, no barrier.
+//   * The carry entering a block is a wave-uniform value; it is chained over
+//     the U blocks and over the tiles of the row in registers.  When several
+//     waves share a row (few rows, long T) their sub-tile totals go through a
+//     double-buffered LDS slot array, one barrier per tile.
+//   * Every output element is then recomputed by the plain recurrence from the
+//     state entering its lane, so the per-element arithmetic is the sequential
+//     one and only the lane-entry state depends on the tree order.
+//   * Reverse-time kernels mirror the lane mapping (lane l takes vector
+//     63-l, elements in descending order) so the same ascending-lane scan
+//     applies.  The backward pass gets gate[t+1] and x[t-1] from the vectors
+//     it already holds plus one-lane DPP shifts; only the two elements just
+//     outside a wave's sub-tile are loaded separately.
+//
+// All arithmetic is fp32 with fused multiply-add.
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+#include <stdlib.h>
+
+#include "ascan.h"
+
+#ifndef ASCAN_USE_DPP
+#define ASCAN_USE_DPP 1
+#endif
+
+namespace {
+
+// ---------------------------------------------------------------------------
+// Value algebra: float for the real dtypes, cfloat for complex64.
+// ---------------------------------------------------------------------------
+struct cfloat {
+    float re, im;
+};
+
+__device__ __forceinline__ float vmul(float a, float b) { return a * b; }
+__device__ __forceinline__ float vfma(float a, float b, float c) { return __builtin_fmaf(a, b, c); }
+__device__ __forceinline__ float vconj(float a) { return a; }
+
+__device__ __forceinline__ cfloat vmul(cfloat a, cfloat b) {
+    cfloat r;
+    r.re = __builtin_fmaf(a.re, b.re, -(a.im * b.im));
+    r.im = __builtin_fmaf(a.re, b.im, a.im * b.re);
+    return r;
+}
+// a * b + c
+__device__ __forceinline__ cfloat vfma(cfloat a, cfloat b, cfloat c) {
+    cfloat r;
+    r.re = __builtin_fmaf(a.re, b.re, __builtin_fmaf(-a.im, b.im, c.re));
+    r.im = __builtin_fmaf(a.re, b.im, __builtin_fmaf(a.im, b.re, c.im));
+    return r;
+}
+__device__ __forceinline__ cfloat vconj(cfloat a) {
+    cfloat r;
+    r.re = a.re;
+    r.im = -a.im;
+    return r;
+}
+
+template <class V> __device__ __forceinline__ V vone();
+template <class V> __device__ __forceinline__ V vzero();
+template <> __device__ __forceinline__ float vone<float>() { return 1.0f; }
+template <> __device__ __forceinline__ float vzero<float>() { return 0.0f; }
+template <> __device__ __forceinline__ cfloat vone<cfloat>() { return cfloat{1.0f, 0.0f}; }
+template <> __device__ __forceinline__ cfloat vzero<cfloat>() { return cfloat{0.0f, 0.0f}; }
+
+__device__ __forceinline__ float vselect(bool c, float a, float b) { return c ? a : b; }
+__device__ __forceinline__ cfloat vselect(bool c, cfloat a, cfloat b) {
+    cfloat r;
+    r.re = c ? a.re : b.re;
+    r.im = c ? a.im : b.im;
+    return r;
+}
+
+// ---------------------------------------------------------------------------
+// Cross-lane primitives for one wave64.
+// ---------------------------------------------------------------------------
+__device__ __forceinline__ int f2i(float x) { return __builtin_bit_cast(int, x); }
+__device__ __forceinline__ float i2f(int x) { return __builtin_bit_cast(float, x); }
+
+#if ASCAN_USE_DPP
+// DPP control words (GFX9 encoding).
+constexpr int kRowShr1 = 0x111, kRowShr2 = 0x112, kRowShr4 = 0x114, kRowShr8 = 0x118;
+constexpr int kWaveShl1 = 0x130, kWaveShr1 = 0x138;
+constexpr int kRowBcast15 = 0x142, kRowBcast31 = 0x143;
+
+// Lanes that have no source lane, or whose row is masked off, receive `old`.
+template <int CTRL, int ROW_MASK>
+__device__ __forceinline__ float dpp_move(float old, float src) {
+    return i2f(__builtin_amdgcn_update_dpp(f2i(old), f2i(src), CTRL, ROW_MASK, 0xF, false));
+}
+template <int CTRL, int ROW_MASK>
+__device__ __forceinline__ cfloat dpp_move(cfloat old, cfloat src) {
+    cfloat r;
+    r.re = dpp_move<CTRL, ROW_MASK>(old.re, src.re);
+    r.im = dpp_move<CTRL, ROW_MASK>(old.im, src.im);
+    return r;
+}
+
+// One Kogge-Stone step of the pair scan: (Ap, Xp) o (A, X) = (Ap*A, Xp*A + X).
+template <int CTRL, int ROW_MASK, class V>
+__device__ __forceinline__ void scan_step(V& A, V& X) {
+    const V Ap = dpp_move<CTRL, ROW_MASK>(vone<V>(), A);
+    const V Xp = dpp_move<CTRL, ROW_MASK>(vzero<V>(), X);
+    X = vfma(Xp, A, X);
+    A = vmul(Ap, A);
+}
+
+// Inclusive scan of the 64 (A, X) pairs of a wave, ascending lane order.
+template <class V>
+__device__ __forceinline__ void wave_scan_inclusive(V& A, V& X) {
+    scan_step<kRowShr1, 0xF>(A, X);
+    scan_step<kRowShr2, 0xF>(A, X);
+    scan_step<kRowShr4, 0xF>(A, X);
+    scan_step<kRowShr8, 0xF>(A, X);
+    scan_step<kRowBcast15, 0xA>(A, X);  // lane 15 of rows 0,2 -> rows 1,3
+    scan_step<kRowBcast31, 0xC>(A, X);  // lane 31 -> rows 2,3
+}
+
+// Lane l receives v of lane l-1; lane 0 receives `edge`.
+template <class V>
+__device__ __forceinline__ V shift_up1(V v, V edge) {
+    return dpp_move<kWaveShr1, 0xF>(edge, v);
+}
+// Lane l receives v of lane l+1; lane 63 receives `edge`.
+template <class V>
+__device__ __forceinline__ V shift_down1(V v, V edge) {
+    return dpp_move<kWaveShl1, 0xF>(edge, v);
+}
+#else
+// Portable variant of the same primitives through ds_bpermute.
+__device__ __forceinline__ float shfl_up_f(float v, int d) { return __shfl_up(v, d, 64); }
+__device__ __forceinline__ cfloat shfl_up_f(cfloat v, int d) {
+    cfloat r;
+    r.re = __shfl_up(v.re, d, 64);
+    r.im = __shfl_up(v.im, d, 64);
+    return r;
+}
+__device__ __forceinline__ float shfl_down_f(float v, int d) { return __shfl_down(v, d, 64); }
+__device__ __forceinline__ cfloat shfl_down_f(cfloat v, int d) {
+    cfloat r;
+    r.re = __shfl_down(v.re, d, 64);
+    r.im = __shfl_down(v.im, d, 64);
+    return r;
+}
+template <class V>
+__device__ __forceinline__ void wave_scan_inclusive(V& A, V& X) {
+    const int lane = threadIdx.x & 63;
+#pragma unroll
+    for (int d = 1; d < 64; d *= 2) {
+        V Ap = shfl_up_f(A, d);
+        V Xp = shfl_up_f(X, d);
+        Ap = vselect(lane >= d, Ap, vone<V>());
+        Xp = vselect(lane >= d, Xp, vzero<V>());
+        X = vfma(Xp, A, X);
+        A = vmul(Ap, A);
+    }
+}
+template <class V>
+__device__ __forceinline__ V shift_up1(V v, V edge) {
+    const int lane = threadIdx.x & 63;
+    return vselect(lane >= 1, shfl_up_f(v, 1), edge);
+}
+template <class V>
+__device__ __forceinline__ V shift_down1(V v, V edge) {
+    const int lane = threadIdx.x & 63;
+    return vselect(lane < 63, shfl_down_f(v, 1), edge);
+}
+#endif
+
+template <int LANE>
+__device__ __forceinline__ float read_lane(float v) {
+    return i2f(__builtin_amdgcn_readlane(f2i(v), LANE));
+}
+template <int LANE>
+__device__ __forceinline__ cfloat read_lane(cfloat v) {
+    cfloat r;
+    r.re = read_lane<LANE>(v.re);
+    r.im = read_lane<LANE>(v.im);
+    return r;
+}
+
+// ---------------------------------------------------------------------------
+// Storage traits: S = element type in memory, V = arithmetic type,
+// EPV = elements per 16-byte vector.
+// ---------------------------------------------------------------------------
+typedef float floatx2_t __attribute__((ext_vector_type(2)));
+typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
+typedef _Float16 halfx2_t __attribute__((ext_vector_type(2)));
+
+struct TraitsF32 {
+    using S = float;
+    using V = float;
+    static constexpr int EPV = 4;
+    static __device__ __forceinline__ void unpack(const uint4& r, V (&d)[EPV]) {
+        d[0] = i2f(r.x);
+        d[1] = i2f(r.y);
+        d[2] = i2f(r.z);
+        d[3] = i2f(r.w);
+    }
+    static __device__ __forceinline__ uint4 pack(const V (&s)[EPV]) {
+        uint4 r;
+        r.x = f2i(s[0]);
+        r.y = f2i(s[1]);
+        r.z = f2i(s[2]);
+        r.w = f2i(s[3]);
+        return r;
+    }
+    static __device__ __forceinline__ V load1(const S* p) { return *p; }
+    static __device__ __forceinline__ void store1(S* p, V v) { *p = v; }
+};
+
+struct TraitsBF16 {
+    using S = uint16_t;
+    using V = float;
+    static constexpr int EPV = 8;
+    static __device__ __forceinline__ uint32_t pack2(float lo, float hi) {
+        floatx2_t f;
+        f.x = lo;
+        f.y = hi;
+        const bf16x2_t h = __builtin_convertvector(f, bf16x2_t);  // round to nearest even
+        return __builtin_bit_cast(uint32_t, h);
+    }
+    static __device__ __forceinline__ void unpack(const uint4& r, V (&d)[EPV]) {
+        const uint32_t w[4] = {r.x, r.y, r.z, r.w};
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            d[2 * i] = i2f((int)(w[i] << 16));
+            d[2 * i + 1] = i2f((int)(w[i] & 0xffff0000u));
+        }
+    }
+    static __device__ __forceinline__ uint4 pack(const V (&s)[EPV]) {
+        uint4 r;
+        r.x = pack2(s[0], s[1]);
+        r.y = pack2(s[2], s[3]);
+        r.z = pack2(s[4], s[5]);
+        r.w = pack2(s[6], s[7]);
+        return r;
+    }
+    static __device__ __forceinline__ V load1(const S* p) { return i2f((int)((uint32_t)(*p) << 16)); }
+    static __device__ __forceinline__ void store1(S* p, V v) { *p = (uint16_t)(pack2(v, 0.0f) & 0xffffu); }
+};
+
+struct TraitsF16 {
+    using S = uint16_t;
+    using V = float;
+    static constexpr int EPV = 8;
+    static __device__ __forceinline__ uint32_t pack2(float lo, float hi) {
+        floatx2_t f;
+        f.x = lo;
+        f.y = hi;
+        const halfx2_t h = __builtin_convertvector(f, halfx2_t);  // round to nearest even
+        return __builtin_bit_cast(uint32_t, h);
+    }
+    static __device__ __forceinline__ void unpack(const uint4& r, V (&d)[EPV]) {
+        const uint32_t w[4] = {r.x, r.y, r.z, r.w};
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const halfx2_t h = __builtin_bit_cast(halfx2_t, w[i]);
+            const floatx2_t f = __builtin_convertvector(h, floatx2_t);
+            d[2 * i] = f.x;
+            d[2 * i + 1] = f.y;
+        }
+    }
+    static __device__ __forceinline__ uint4 pack(const V (&s)[EPV]) {
+        uint4 r;
+        r.x = pack2(s[0], s[1]);
+        r.y = pack2(s[2], s[3]);
+        r.z = pack2(s[4], s[5]);
+        r.w = pack2(s[6], s[7]);
+        return r;
+    }
+    static __device__ __forceinline__ V load1(const S* p) {
+        return (float)__builtin_bit_cast(_Float16, *p);
+    }
+    static __device__ __forceinline__ void store1(S* p, V v) {
+        *p = __builtin_bit_cast(uint16_t, (_Float16)v);
+    }
+};
+
+struct TraitsC64 {
+    using S = cfloat;  // 8 bytes, interleaved (re, im)
+    using V = cfloat;
+    static constexpr int EPV = 2;
+    static __device__ __forceinline__ void unpack(const uint4& r, V (&d)[EPV]) {
+        d[0].re = i2f(r.x);
+        d[0].im = i2f(r.y);
+        d[1].re = i2f(r.z);
+        d[1].im = i2f(r.w);
+    }
+    static __device__ __forceinline__ uint4 pack(const V (&s)[EPV]) {
+        uint4 r;
+        r.x = f2i(s[0].re);
+        r.y = f2i(s[0].im);
+        r.z = f2i(s[1].re);
+        r.w = f2i(s[1].im);
+        return r;
+    }
+    static __device__ __forceinline__ V load1(const S* p) {
+        const float2 v = *reinterpret_cast<const float2*>(p);
+        cfloat r;
+        r.re = v.x;
+        r.im = v.y;
+        return r;
+    }
+    static __device__ __forceinline__ void store1(S* p, V v) {
+        float2 o;
+        o.x = v.re;
+        o.y = v.im;
+        *reinterpret_cast<float2*>(p) = o;
+    }
+};
+
+// ---------------------------------------------------------------------------
+// Vector access.  `pos` is the element index inside the row of the first
+// element of the vector.  FULL: the whole vector is known to lie inside the
+// row.  ALIGNED: rowp + pos is 16-byte aligned and T is a multiple of EPV, so
+// a vector is either entirely inside the row or entirely outside.
+// ---------------------------------------------------------------------------
+template <class Tr, bool ALIGNED, bool FULL>
+__device__ __forceinline__ void load_vec(const typename Tr::S* __restrict__ rowp, int64_t pos, int64_t T,
+                                         typename Tr::V fill, typename Tr::V (&dst)[Tr::EPV]) {
+    if constexpr (ALIGNED) {
+        if (FULL || pos < T) {
+            const uint4 raw = *reinterpret_cast<const uint4*>(rowp + pos);
+            Tr::unpack(raw, dst);
+        } else {
+#pragma unroll
+            for (int e = 0; e < Tr::EPV; ++e) dst[e] = fill;
+        }
+    } else {
+#pragma unroll
+        for (int e = 0; e < Tr::EPV; ++e) {
+            if (FULL || pos + e < T) {
+                dst[e] = Tr::load1(rowp + pos + e);
+            } else {
+                dst[e] = fill;
+            }
+        }
+    }
+}
+
+template <class Tr, bool ALIGNED, bool FULL>
+__device__ __forceinline__ void store_vec(typename Tr::S* __restrict__ rowp, int64_t pos, int64_t T,
+                                          const typename Tr::V (&src)[Tr::EPV]) {
+    if constexpr (ALIGNED) {
+        if (FULL || pos < T) {
+            *reinterpret_cast<uint4*>(rowp + pos) = Tr::pack(src);
+        }
+    } else {
+#pragma unroll
+        for (int e = 0; e < Tr::EPV; ++e) {
+            if (FULL || pos + e < T) Tr::store1(rowp + pos + e, src[e]);
+        }
+    }
+}
+
+// Element index (inside the sub-tile) of the vector that lane `lane` owns in
+// scan-order block j.  Reverse-time kernels mirror the mapping.
+template <int U, int EPV, bool REV>
+__device__ __forceinline__ int vec_offset(int j, int lane) {
+    const int q = j * 64 + lane;
+    return (REV ? (U * 64 - 1 - q) : q) * EPV;
+}
+
+// Carry bookkeeping shared by the forward and the backward kernel.
+//
+// Input : totA/totX[j]   inclusive total of block j of this wave (wave-uniform)
+//         carry          state entering the tile (wave-uniform, same in all waves)
+// Output: c              state entering block 0 of this wave
+//         carry          state entering the next tile
+// With W > 1 the waves of the workgroup exchange their sub-tile totals through
+// `slots` (2 buffers x W entries); `parity` selects the buffer.
+template <class V, int W, int U>
+__device__ __forceinline__ void exchange_carries(const V (&totA)[U], const V (&totX)[U], V& carry, V& c,
+                                                 V* slots, int parity, int w, int lane) {
+    if constexpr (W == 1) {
+        c = carry;
+        V n = carry;
+#pragma unroll
+        for (int j = 0; j < U; ++j) n = vfma(totA[j], n, totX[j]);
+        carry = n;
+    } else {
+        V TA = totA[0], TX = totX[0];
+#pragma unroll
+        for (int j = 1; j < U; ++j) {
+            TX = vfma(TX, totA[j], totX[j]);
+            TA = vmul(TA, totA[j]);
+        }
+        V* buf = slots + parity * (2 * W);
+        if (lane == 0) {
+            buf[2 * w] = TA;
+            buf[2 * w + 1] = TX;
+        }
+        __syncthreads();
+        V run = carry;
+        V mine = carry;
+#pragma unroll
+        for (int i = 0; i < W; ++i) {
+            const V Ai = buf[2 * i];
+            const V Xi = buf[2 * i + 1];
+            mine = vselect(i == w, run, mine);
+            run = vfma(Ai, run, Xi);
+        }
+        c = mine;
+        carry = run;
+    }
+}
+
+// ---------------------------------------------------------------------------
+// Forward kernel (REV = false) and plain reverse scan (REV = true).
+// W waves share one row (W == 1: four independent rows per 256-thread block).
+// ---------------------------------------------------------------------------
+template <class Tr, int W, int U, bool REV, bool ALIGNED>
+__global__ void __launch_bounds__(W == 1 ? 256 : 64 * W)
+    scan_forward_kernel(const typename Tr::S* __restrict__ gates, const typename Tr::S* __restrict__ tokens,
+                        typename Tr::S* __restrict__ out, int64_t rows, int64_t T) {
+    using S = typename Tr::S;
+    using V = typename Tr::V;
+    constexpr int EPV = Tr::EPV;
+    constexpr int64_t SUB = (int64_t)U * 64 * EPV;
+    constexpr int64_t TILE = SUB * W;
+
+    const int lane = threadIdx.x & 63;
+    const int wv = threadIdx.x >> 6;
+    int64_t row;
+    int w;
+    if constexpr (W == 1) {
+        row = (int64_t)blockIdx.x * 4 + wv;
+        w = 0;
+        if (row >= rows) return;  // wave-uniform; this configuration has no barrier
+    } else {
+        row = blockIdx.x;
+        w = wv;
+    }
+    __shared__ V slots[W == 1 ? 1 : 4 * W];
+
+    const S* __restrict__ grow = gates + row * T;
+    const S* __restrict__ trow = tokens + row * T;
+    S* __restrict__ orow = out + row * T;
+
+    const int64_t ntiles = (T + TILE - 1) / TILE;
+    V carry = vzero<V>();
+
+    for (int64_t k = 0; k < ntiles; ++k) {
+        const int64_t tile = REV ? (ntiles - 1 - k) : k;
+        const int64_t sub_base = tile * TILE + (int64_t)(REV ? (W - 1 - w) : w) * SUB;
+        const bool full = sub_base + SUB <= T;  // wave-uniform
+
+        V g[U][EPV], t[U][EPV];
+        if (full) {
+#pragma unroll
+            for (int j = 0; j < U; ++j) {
+                const int64_t pos = sub_base + vec_offset<U, EPV, REV>(j, lane);
+                load_vec<Tr, ALIGNED, true>(grow, pos, T, vone<V>(), g[j]);
+                load_vec<Tr, ALIGNED, true>(trow, pos, T, vzero<V>(), t[j]);
+            }
+        } else {
+#pragma unroll
+            for (int j = 0; j < U; ++j) {
+                const int64_t pos = sub_base + vec_offset<U, EPV, REV>(j, lane);
+                load_vec<Tr, ALIGNED, false>(grow, pos, T, vone<V>(), g[j]);
+                load_vec<Tr, ALIGNED, false>(trow, pos, T, vzero<V>(), t[j]);
+            }
+        }
+
+        V totA[U], totX[U], exA[U], exX[U];
+#pragma unroll
+        for (int j = 0; j < U; ++j) {
+            constexpr int e0 = REV ? EPV - 1 : 0;
+            V A = g[j][e0];
+            V X = t[j][e0];
+#pragma unroll
+            for (int i = 1; i < EPV; ++i) {
+                const int e = REV ? EPV - 1 - i : i;
+                X = vfma(g[j][e], X, t[j][e]);
+                A = vmul(A, g[j][e]);
+            }
+            wave_scan_inclusive(A, X);
+            totA[j] = read_lane<63>(A);
+            totX[j] = read_lane<63>(X);
+            exA[j] = shift_up1(A, vone<V>());
+            exX[j] = shift_up1(X, vzero<V>());
+        }
+
+        V c;
+        exchange_carries<V, W, U>(totA, totX, carry, c, slots, (int)(k & 1), w, lane);
+
+#pragma unroll
+        for (int j = 0; j < U; ++j) {
+            V x = vfma(exA[j], c, exX[j]);  // state entering this lane's vector
+            c = vfma(totA[j], c, totX[j]);  // state entering the next block
+            V o[EPV];
+#pragma unroll
+            for (int i = 0; i < EPV; ++i) {
+                const int e = REV ? EPV - 1 - i : i;
+                x = vfma(g[j][e], x, t[j][e]);
+                o[e] = x;
+            }
+            const int64_t pos = sub_base + vec_offset<U, EPV, REV>(j, lane);
+            if (full) {
+                store_vec<Tr, ALIGNED, true>(orow, pos, T, o);
+            } else {
+                store_vec<Tr, ALIGNED, false>(orow, pos, T, o);
+            }
+        }
+    }
+}
+
+// ---------------------------------------------------------------------------
+// Fused backward kernel: reverse-time scan over gate[t+1] producing d_tokens,
+// and d_gates[t] = d_tokens[t] * conj(x[t-1]) in the same pass.
+// ---------------------------------------------------------------------------
+template <class Tr, int W, int U, bool ALIGNED>
+__global__ void __launch_bounds__(W == 1 ? 256 : 64 * W)
+    scan_backward_kernel(const typename Tr::S* __restrict__ gates, const typename Tr::S* __restrict__ states,
+                         const typename Tr::S* __restrict__ grad_out, typename Tr::S* __restrict__ d_gates,
+                         typename Tr::S* __restrict__ d_tokens, int64_t rows, int64_t T) {
+    using S = typename Tr::S;
+    using V = typename Tr::V;
+    constexpr int EPV = Tr::EPV;
+    constexpr int64_t SUB = (int64_t)U * 64 * EPV;
+    constexpr int64_t TILE = SUB * W;
+
+    const int lane = threadIdx.x & 63;
+    const int wv = threadIdx.x >> 6;
+    int64_t row;
+    int w;
+    if constexpr (W == 1) {
+        row = (int64_t)blockIdx.x * 4 + wv;
+        w = 0;
+        if (row >= rows) return;  // wave-uniform; this configuration has no barrier
+    } else {
+        row = blockIdx.x;
+        w = wv;
+    }
+    __shared__ V slots[W == 1 ? 1 : 4 * W];
+
+    const S* __restrict__ arow = gates + row * T;
+    const S* __restrict__ xrow = states + row * T;
+    const S* __restrict__ drow = grad_out + row * T;
+    S* __restrict__ dgrow = d_gates + row * T;
+    S* __restrict__ dtrow = d_tokens + row * T;
+
+    const int64_t ntiles = (T + TILE - 1) / TILE;
+    V carry = vzero<V>();
+
+    for (int64_t k = 0; k < ntiles; ++k) {
+        const int64_t tile = ntiles - 1 - k;
+        const int64_t sub_base = tile * TILE + (int64_t)(W - 1 - w) * SUB;
+        const int64_t sub_end = sub_base + SUB;
+        const bool full = sub_end <= T;  // wave-uniform
+
+        V a[U][EPV], d[U][EPV], x[U][EPV];
+        if (full) {
+#pragma unroll
+            for (int j = 0; j < U; ++j) {
+                const int64_t pos = sub_base + vec_offset<U, EPV, true>(j, lane);
+                load_vec<Tr, ALIGNED, true>(arow, pos, T, vone<V>(), a[j]);
+                load_vec<Tr, ALIGNED, true>(drow, pos, T, vzero<V>(), d[j]);
+                load_vec<Tr, ALIGNED, true>(xrow, pos, T, vzero<V>(), x[j]);
+            }
+        } else {
+#pragma unroll
+            for (int j = 0; j < U; ++j) {
+                const int64_t pos = sub_base + vec_offset<U, EPV, true>(j, lane);
+                load_vec<Tr, ALIGNED, false>(arow, pos, T, vone<V>(), a[j]);
+                load_vec<Tr, ALIGNED, false>(drow, pos, T, vzero<V>(), d[j]);
+                load_vec<Tr, ALIGNED, false>(xrow, pos, T, vzero<V>(), x[j]);
+            }
+        }
+
+        // The two elements just outside the sub-tile: gate[sub_end] and
+        // x[sub_base-1].  Addresses are clamped into the row so the loads are
+        // unconditional; out-of-row positions take the identity values.
+        V a_edge, x_edge;
+        {
+            const int64_t ia = sub_end < T ? sub_end : T - 1;
+            int64_t ix = sub_base - 1;
+            ix = ix < 0 ? 0 : (ix < T ? ix : T - 1);
+            const V av = Tr::load1(arow + ia);
+            const V xv = Tr::load1(xrow + ix);
+            a_edge = vselect(sub_end < T, av, vone<V>());
+            x_edge = vselect(sub_base >= 1 && sub_base - 1 < T, xv, vzero<V>());
+        }
+
+        // Shift gates down by one element (gate[t+1]) and states up by one
+        // (x[t-1]); in scan order the neighbour vector at the next higher
+        // address is lane-1, the one at the next lower address is lane+1.
+        V ga[U][EPV], xs[U][EPV];
+#pragma unroll
+        for (int j = 0; j < U; ++j) {
+            V hi_edge, lo_edge;
+            if (j == 0) {
+                hi_edge = a_edge;
+            } else {
+                hi_edge = read_lane<63>(a[j - 1][0]);
+            }
+            if (j == U - 1) {
+                lo_edge = x_edge;
+            } else {
+                lo_edge = read_lane<0>(x[j + 1][EPV - 1]);
+            }
+            const V a_next = shift_up1(a[j][0], hi_edge);
+            const V x_prev = shift_down1(x[j][EPV - 1], lo_edge);
+#pragma unroll
+            for (int e = 0; e < EPV; ++e) {
+                ga[j][e] = vconj(e < EPV - 1 ? a[j][e + 1] : a_next);
+                xs[j][e] = vconj(e > 0 ? x[j][e - 1] : x_prev);
+            }
+        }
+
+        V totA[U], totX[U], exA[U], exX[U];
+#pragma unroll
+        for (int j = 0; j < U; ++j) {
+            V A = ga[j][EPV - 1];
+            V X = d[j][EPV - 1];
+#pragma unroll
+            for (int e = EPV - 2; e >= 0; --e) {
+                X = vfma(ga[j][e], X, d[j][e]);
+                A = vmul(A, ga[j][e]);
+            }
+            wave_scan_inclusive(A, X);
+            totA[j] = read_lane<63>(A);
+            totX[j] = read_lane<63>(X);
+            exA[j] = shift_up1(A, vone<V>());
+            exX[j] = shift_up1(X, vzero<V>());
+        }
+
+        V c;
+        exchange_carries<V, W, U>(totA, totX, carry, c, slots, (int)(k & 1), w, lane);
+
+#pragma unroll
+        for (int j = 0; j < U; ++j) {
+            V gr = vfma(exA[j], c, exX[j]);  // g entering this lane's vector from above
+            c = vfma(totA[j], c, totX[j]);
+            V dt[EPV], dg[EPV];
+#pragma unroll
+            for (int e = EPV - 1; e >= 0; --e) {
+                gr = vfma(ga[j][e], gr, d[j][e]);
+                dt[e] = gr;
+                dg[e] = vmul(gr, xs[j][e]);
+            }
+            const int64_t pos = sub_base + vec_offset<U, EPV, true>(j, lane);
+            if (full) {
+                store_vec<Tr, ALIGNED, true>(dtrow, pos, T, dt);
+                store_vec<Tr, ALIGNED, true>(dgrow, pos, T, dg);
+            } else {
+                store_vec<Tr, ALIGNED, false>(dtrow, pos, T, dt);
+                store_vec<Tr, ALIGNED, false>(dgrow, pos, T, dg);
+            }
+        }
+    }
+}
+
+// ---------------------------------------------------------------------------
+// Host side.
+// ---------------------------------------------------------------------------
+thread_local int g_last_hip_error = 0;
+
+// Blocks per sub-tile (U) by dtype: 1024 elements per wave per tile for the
+// real dtypes, 512 for complex64.
+template <class Tr> struct Tuning;
+template <> struct Tuning<TraitsF32> { static constexpr int U = 4; };
+template <> struct Tuning<TraitsBF16> { static constexpr int U = 2; };
+template <> struct Tuning<TraitsF16> { static constexpr int U = 2; };
+template <> struct Tuning<TraitsC64> { static constexpr int U = 4; };
+
+// Optional override of the waves-per-row choice (1, 4 or 16), read once.
+int forced_waves_per_row() {
+    static const int v = [] {
+        const char* s = getenv("ASCAN_WAVES_PER_ROW");
+        const int n = s ? atoi(s) : 0;
+        return (n == 1 || n == 4 || n == 16) ? n : 0;
+    }();
+    return v;
+}
+
+// How many waves cooperate on one row.  One wave per row is the cheapest
+// arrangement (no LDS, no barrier) and is used whenever the rows alone give
+// the machine enough waves; few long rows are split over 4 or 16 waves.
+int choose_waves_per_row(int64_t rows, int64_t T, int64_t sub) {
+    const int forced = forced_waves_per_row();
+    int w;
+    if (forced) {
+        w = forced;
+    } else if (rows >= 2048) {
+        w = 1;
+    } else if (rows >= 512) {
+        w = 4;
+    } else {
+        w = 16;
+    }
+    // No point in more waves than sub-tiles in the row.
+    while (w > 1 && (int64_t)(w / 4) * sub >= T) w /= 4;
+    return w;
+}
+
+bool is_aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
+
+int finish_launch() {
+    const hipError_t e = hipGetLastError();
+    if (e != hipSuccess) {
+        g_last_hip_error = (int)e;
+        return ASCAN_ERR_LAUNCH;
+    }
+    return ASCAN_OK;
+}
+
+template <class Tr, int W, bool REV, bool ALIGNED>
+void launch_forward(const void* gates, const void* tokens, void* out, int64_t rows, int64_t T,
+                    hipStream_t stream) {
+    using S = typename Tr::S;
+    constexpr int U = Tuning<Tr>::U;
+    const unsigned blocks = (unsigned)(W == 1 ? (rows + 3) / 4 : rows);
+    const unsigned threads = W == 1 ? 256 : 64 * W;
+    hipLaunchKernelGGL((scan_forward_kernel<Tr, W, U, REV, ALIGNED>), dim3(blocks), dim3(threads), 0, stream,
+                       static_cast<const S*>(gates), static_cast<const S*>(tokens), static_cast<S*>(out), rows,
+                       T);
+}
+
+template <class Tr, int W, bool ALIGNED>
+void launch_backward(const void* gates, const void* states, const void* grad_out, void* d_gates,
+                     void* d_tokens, int64_t rows, int64_t T, hipStream_t stream) {
+    using S = typename Tr::S;
+    constexpr int U = Tuning<Tr>::U;
+    const unsigned blocks = (unsigned)(W == 1 ? (rows + 3) / 4 : rows);
+    const unsigned threads = W == 1 ? 256 : 64 * W;
+    hipLaunchKernelGGL((scan_backward_kernel<Tr, W, U, ALIGNED>), dim3(blocks), dim3(threads), 0, stream,
+                       static_cast<const S*>(gates), static_cast<const S*>(states),
+                       static_cast<const S*>(grad_out), static_cast<S*>(d_gates), static_cast<S*>(d_tokens),
+                       rows, T);
+}
+
+template <class Tr>
+int forward_typed(const void* gates, const void* tokens, void* out, int64_t rows, int64_t T, bool reverse,
+                  hipStream_t stream) {
+    constexpr int EPV = Tr::EPV;
+    constexpr int64_t SUB = (int64_t)Tuning<Tr>::U * 64 * EPV;
+    const bool aligned = is_aligned16(gates) && is_aligned16(tokens) && is_aligned16(out) && (T % EPV == 0);
+    const int W = aligned ? choose_waves_per_row(rows, T, SUB) : 1;
+#define ASCAN_FWD(WV, AL)                                                              \
+    do {                                                                               \
+        if (reverse)                                                                   \
+            launch_forward<Tr, WV, true, AL>(gates, tokens, out, rows, T, stream);     \
+        else                                                                           \
+            launch_forward<Tr, WV, false, AL>(gates, tokens, out, rows, T, stream);    \
+    } while (0)
+    if (!aligned) {
+        ASCAN_FWD(1, false);
+    } else if (W == 1) {
+        ASCAN_FWD(1, true);
+    } else if (W == 4) {
+        ASCAN_FWD(4, true);
+    } else {
+        ASCAN_FWD(16, true);
+    }
+#undef ASCAN_FWD
+    return finish_launch();
+}
+
+template <class Tr>
+int backward_typed(const void* gates, const void* states, const void* grad_out, void* d_gates, void* d_tokens,
+                   int64_t rows, int64_t T, hipStream_t stream) {
+    constexpr int EPV = Tr::EPV;
+    constexpr int64_t SUB = (int64_t)Tuning<Tr>::U * 64 * EPV;
+    const bool aligned = is_aligned16(gates) && is_aligned16(states) && is_aligned16(grad_out) &&
+                         is_aligned16(d_gates) && is_aligned16(d_tokens) && (T % EPV == 0);
+    const int W = aligned ? choose_waves_per_row(rows, T, SUB) : 1;
+    if (!aligned) {
+        launch_backward<Tr, 1, false>(gates, states, grad_out, d_gates, d_tokens, rows, T, stream);
+    } else if (W == 1) {
+        launch_backward<Tr, 1, true>(gates, states, grad_out, d_gates, d_tokens, rows, T, stream);
+    } else if (W == 4) {
+        launch_backward<Tr, 4, true>(gates, states, grad_out, d_gates, d_tokens, rows, T, stream);
+    } else {
+        launch_backward<Tr, 16, true>(gates, states, grad_out, d_gates, d_tokens, rows, T, stream);
+    }
+    return finish_launch();
+}
+
+size_t element_size(int dtype) {
+    switch (dtype) {
+        case ASCAN_F32: return 4;
+        case ASCAN_BF16: return 2;
+        case ASCAN_F16: return 2;
+        case ASCAN_C64: return 8;
+        default: return 0;
+    }
+}
+
+bool element_aligned(const void* p, size_t es) { return (reinterpret_cast<uintptr_t>(p) % es) == 0; }
+
+// Largest row count one launch can address: gridDim.x is limited to 2^31-1.
+constexpr int64_t kMaxBlocks = 2147483647LL;
+
+}  // namespace
+
+extern "C" {
+
+int ascan_forward(const void* gates, const void* tokens, void* out, int64_t rows, int64_t seqlen, int dtype,
+                  int reverse, void* stream) {
+    const size_t es = element_size(dtype);
+    if (es == 0) return ASCAN_ERR_BAD_DTYPE;
+    if (rows < 0 || seqlen < 0 || rows > kMaxBlocks) return ASCAN_ERR_BAD_SHAPE;
+    if (rows == 0 || seqlen == 0) return ASCAN_OK;
+    if (!gates || !tokens || !out) return ASCAN_ERR_NULL_POINTER;
+    if (!element_aligned(gates, es) || !element_aligned(tokens, es) || !element_aligned(out, es))
+        return ASCAN_ERR_MISALIGNED;
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    const bool rev = reverse != 0;
+    switch (dtype) {
+        case ASCAN_F32: return forward_typed<TraitsF32>(gates, tokens, out, rows, seqlen, rev, s);
+        case ASCAN_BF16: return forward_typed<TraitsBF16>(gates, tokens, out, rows, seqlen, rev, s);
+        case ASCAN_F16: return forward_typed<TraitsF16>(gates, tokens, out, rows, seqlen, rev, s);
+        default: return forward_typed<TraitsC64>(gates, tokens, out, rows, seqlen, rev, s);
+    }
+}
+
+int ascan_backward(const void* gates, const void* states, const void* grad_out, void* d_gates, void* d_tokens,
+                   int64_t rows, int64_t seqlen, int dtype, void* stream) {
+    const size_t es = element_size(dtype);
+    if (es == 0) return ASCAN_ERR_BAD_DTYPE;
+    if (rows < 0 || seqlen < 0 || rows > kMaxBlocks) return ASCAN_ERR_BAD_SHAPE;
+    if (rows == 0 || seqlen == 0) return ASCAN_OK;
+    if (!gates || !states || !grad_out || !d_gates || !d_tokens) return ASCAN_ERR_NULL_POINTER;
+    if (!element_aligned(gates, es) || !element_aligned(states, es) || !element_aligned(grad_out, es) ||
+        !element_aligned(d_gates, es) || !element_aligned(d_tokens, es))
+        return ASCAN_ERR_MISALIGNED;
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    switch (dtype) {
+        case ASCAN_F32:
+            return backward_typed<TraitsF32>(gates, states, grad_out, d_gates, d_tokens, rows, seqlen, s);
+        case ASCAN_BF16:
+            return backward_typed<TraitsBF16>(gates, states, grad_out, d_gates, d_tokens, rows, seqlen, s);
+        case ASCAN_F16:
+            return backward_typed<TraitsF16>(gates, states, grad_out, d_gates, d_tokens, rows, seqlen, s);
+        default:
+            return backward_typed<TraitsC64>(gates, states, grad_out, d_gates, d_tokens, rows, seqlen, s);
+    }
+}
+
+const char* ascan_status_string(int status) {
+    switch (status) {
+        case ASCAN_OK: return "ok";
+        case ASCAN_ERR_NULL_POINTER: return "a required buffer pointer is NULL";
+        case ASCAN_ERR_BAD_SHAPE: return "rows or seqlen is negative, or rows exceeds the grid limit";
+        case ASCAN_ERR_BAD_DTYPE: return "unsupported dtype: expecting float32, bfloat16, float16 or complex64";
+        case ASCAN_ERR_MISALIGNED: return "a buffer is not aligned to its element size";
+        case ASCAN_ERR_LAUNCH: return "the HIP runtime reported a launch error";
+        default: return "unknown status";
+    }
+}
+
+int ascan_last_hip_error(void) { return g_last_hip_error; }
+
+int ascan_abi_version(void) { return ASCAN_ABI_VERSION; }
+
+}  // extern "C"

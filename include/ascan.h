@@ -1,0 +1,102 @@
+/*
+ * ascan.h -- C ABI of the MI355X (gfx950) first-order scan library.
+ *
+ * The library solves, independently for every row of a contiguous
+ * (rows, seqlen) matrix (rows = B*D of a (B, D, T) tensor, T innermost):
+ *
+ *     forward :  x[t] = gate[t] * x[t-1] + token[t],      x[-1] = 0
+ *     reverse :  y[t] = gate[t] * y[t+1] + token[t],      y[T]  = 0
+ *     backward:  g[t] = grad_out[t] + conj(gate[t+1]) * g[t+1],   g[T] = 0
+ *                d_tokens[t] = g[t]
+ *                d_gates[t]  = g[t] * conj(x[t-1]),       x[-1] = 0
+ *
+ * (conj is the identity for the real dtypes).
+ *
+ * These entry points stand where the reference binds its compiled extension:
+ *   accelerated_scan/warp.py:29-30   (module.warpscan_forward / warpscan_backward)
+ *   accelerated_scan/warp.cuh:394-424 (the two functions those names resolve to)
+ * and, for ASCAN_C64, where accelerated_scan/complex.py:174-180,205-214 launches
+ * its forward_scan / backward_scan kernels.
+ *
+ * Conventions
+ *   - every buffer is device memory owned by the caller; the library allocates
+ *     nothing, keeps no reference after the call returns and holds no mutable
+ *     global state, so calls are re-entrant from any host thread;
+ *   - work is enqueued on `stream` (a hipStream_t passed as void*, NULL = the
+ *     default stream) and the call returns without synchronising;
+ *   - rows are dense: row r starts at element r*seqlen; 64-bit element offsets
+ *     are used throughout, so rows*seqlen may exceed 2^31;
+ *   - input and output buffers must not overlap;
+ *   - arithmetic is done in fp32 for every dtype (bf16/fp16 are storage
+ *     formats, rounded to nearest-even on store);
+ *   - 16-byte aligned base pointers with seqlen*sizeof(element) a multiple of
+ *     16 take the vectorised kernels; anything else takes an element-wise
+ *     kernel with identical results;
+ *   - errors are reported by return code, never by abort or exception.
+ */
+#ifndef ASCAN_H_
+#define ASCAN_H_
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define ASCAN_ABI_VERSION 1
+
+/* Element types of gates / tokens / outputs (one code for all tensors of a call). */
+enum ascan_dtype {
+    ASCAN_F32  = 0, /* float                                   (warp.cuh:388) */
+    ASCAN_BF16 = 1, /* bfloat16 storage, fp32 arithmetic       (warp.cuh:384) */
+    ASCAN_F16  = 2, /* IEEE half storage, fp32 arithmetic      (warp.cuh:386) */
+    ASCAN_C64  = 3  /* complex64 = interleaved (re, im) floats (complex.py:37-42) */
+};
+
+/* Return codes. */
+enum ascan_status {
+    ASCAN_OK                = 0,
+    ASCAN_ERR_NULL_POINTER  = 1, /* a required buffer is NULL while rows*seqlen > 0 */
+    ASCAN_ERR_BAD_SHAPE     = 2, /* rows < 0, seqlen < 0, or rows too large for one grid */
+    ASCAN_ERR_BAD_DTYPE     = 3, /* dtype is not an ascan_dtype (warp.cuh:390-391) */
+    ASCAN_ERR_MISALIGNED    = 4, /* a pointer is not aligned to its element size */
+    ASCAN_ERR_LAUNCH        = 5  /* the HIP runtime refused the launch (see ascan_last_hip_error) */
+};
+
+/*
+ * Replaces warpscan_forward (accelerated_scan/warp.cuh:394-405; bound at
+ * warp.py:29) and the forward_scan launches at scalar.py:98 and
+ * complex.py:174-180.  out[r, t] receives the inclusive scan of row r.
+ * reverse != 0 runs the recurrence from t = seqlen-1 down to 0 with the
+ * un-shifted gates (the `reverse` argument of warp.cuh:395).
+ */
+int ascan_forward(const void* gates, const void* tokens, void* out,
+                  int64_t rows, int64_t seqlen, int dtype, int reverse,
+                  void* stream);
+
+/*
+ * Replaces warpscan_backward (accelerated_scan/warp.cuh:407-424; bound at
+ * warp.py:30) and the backward_scan launches at scalar.py:116-124 and
+ * complex.py:205-214.  `states` is the forward output, `grad_out` the incoming
+ * gradient; d_gates and d_tokens receive the two gradients.  One fused
+ * reverse-time pass: 3 tensors read, 2 written.
+ */
+int ascan_backward(const void* gates, const void* states, const void* grad_out,
+                   void* d_gates, void* d_tokens,
+                   int64_t rows, int64_t seqlen, int dtype,
+                   void* stream);
+
+/* Static, human-readable text for an ascan_status code. */
+const char* ascan_status_string(int status);
+
+/* hipError_t (as int) recorded by the calling thread's last ASCAN_ERR_LAUNCH. */
+int ascan_last_hip_error(void);
+
+/* ASCAN_ABI_VERSION the library was built with. */
+int ascan_abi_version(void);
+
+#ifdef __cplusplus
+}
+#endif
+
+#endif /* ASCAN_H_ */

@@ -1,0 +1,121 @@
+/*
+ * ORACLE (test infrastructure, not part of the product).
+ *
+ * The recurrences of the scan operator written as the plain sequential loops
+ * that define them, evaluated in double precision from fp32 inputs.  This is
+ * the "truth" both the GPU kernels and the torch tree scan (oracle/ref_scan.py)
+ * are measured against.  Formulas as the reference states them:
+ *   forward            accelerated_scan/warp.py:71-74,  scalar.py:28-45
+ *   reverse            accelerated_scan/ref.py:100-102,116-118 (used at tests/test_eq.py:77-78)
+ *   backward (real)    accelerated_scan/scalar.py:48-86, tests/test_eq.py:77-80
+ *   backward (complex) accelerated_scan/complex.py:79-92,113-115,141-147
+ * Rows are independent; OpenMP runs them in parallel.
+ */
+#include <stdint.h>
+
+/* out[r,t] = g[r,t] * out[r,t-1] + x[r,t]   (reverse: t+1 in place of t-1) */
+void seq_forward_f32(const float* g, const float* x, double* out, int64_t rows, int64_t T, int reverse) {
+#pragma omp parallel for schedule(static)
+    for (int64_t r = 0; r < rows; ++r) {
+        const float* gr = g + r * T;
+        const float* xr = x + r * T;
+        double* o = out + r * T;
+        double s = 0.0;
+        if (!reverse) {
+            for (int64_t t = 0; t < T; ++t) {
+                s = (double)gr[t] * s + (double)xr[t];
+                o[t] = s;
+            }
+        } else {
+            for (int64_t t = T - 1; t >= 0; --t) {
+                s = (double)gr[t] * s + (double)xr[t];
+                o[t] = s;
+            }
+        }
+    }
+}
+
+/*
+ * Adjoint of the forward recurrence for an incoming gradient dout:
+ *   a[t]  = dout[t] + g[t+1] * a[t+1],  a[T] = 0
+ *   dx[t] = a[t]
+ *   dg[t] = a[t] * state[t-1],          state[-1] = 0
+ * `state` is the forward output (fp32, as the product kernel receives it).
+ */
+void seq_backward_f32(const float* g, const float* state, const float* dout, double* dg, double* dx,
+                      int64_t rows, int64_t T) {
+#pragma omp parallel for schedule(static)
+    for (int64_t r = 0; r < rows; ++r) {
+        const float* gr = g + r * T;
+        const float* sr = state + r * T;
+        const float* dr = dout + r * T;
+        double* dgr = dg + r * T;
+        double* dxr = dx + r * T;
+        double a = 0.0;
+        for (int64_t t = T - 1; t >= 0; --t) {
+            const double gnext = (t + 1 < T) ? (double)gr[t + 1] : 1.0;
+            a = (double)dr[t] + gnext * a;
+            dxr[t] = a;
+            dgr[t] = a * ((t > 0) ? (double)sr[t - 1] : 0.0);
+        }
+    }
+}
+
+/* Complex versions; arrays are interleaved (re, im). */
+void seq_forward_c64(const float* g, const float* x, double* out, int64_t rows, int64_t T, int reverse) {
+#pragma omp parallel for schedule(static)
+    for (int64_t r = 0; r < rows; ++r) {
+        const float* gr = g + 2 * r * T;
+        const float* xr = x + 2 * r * T;
+        double* o = out + 2 * r * T;
+        double sr = 0.0, si = 0.0;
+        for (int64_t k = 0; k < T; ++k) {
+            const int64_t t = reverse ? T - 1 - k : k;
+            const double a = gr[2 * t], b = gr[2 * t + 1];
+            const double nr = a * sr - b * si + (double)xr[2 * t];
+            const double ni = a * si + b * sr + (double)xr[2 * t + 1];
+            sr = nr;
+            si = ni;
+            o[2 * t] = sr;
+            o[2 * t + 1] = si;
+        }
+    }
+}
+
+/*
+ *   a[t]  = dout[t] + conj(g[t+1]) * a[t+1]
+ *   dx[t] = a[t]
+ *   dg[t] = a[t] * conj(state[t-1])
+ */
+void seq_backward_c64(const float* g, const float* state, const float* dout, double* dg, double* dx,
+                      int64_t rows, int64_t T) {
+#pragma omp parallel for schedule(static)
+    for (int64_t r = 0; r < rows; ++r) {
+        const float* gr = g + 2 * r * T;
+        const float* sr = state + 2 * r * T;
+        const float* dr = dout + 2 * r * T;
+        double* dgr = dg + 2 * r * T;
+        double* dxr = dx + 2 * r * T;
+        double ar = 0.0, ai = 0.0;
+        for (int64_t t = T - 1; t >= 0; --t) {
+            double cr = 1.0, ci = 0.0; /* conj(g[t+1]) */
+            if (t + 1 < T) {
+                cr = gr[2 * (t + 1)];
+                ci = -(double)gr[2 * (t + 1) + 1];
+            }
+            const double nr = (double)dr[2 * t] + cr * ar - ci * ai;
+            const double ni = (double)dr[2 * t + 1] + cr * ai + ci * ar;
+            ar = nr;
+            ai = ni;
+            dxr[2 * t] = ar;
+            dxr[2 * t + 1] = ai;
+            double pr = 0.0, pi = 0.0; /* conj(state[t-1]) */
+            if (t > 0) {
+                pr = sr[2 * (t - 1)];
+                pi = -(double)sr[2 * (t - 1) + 1];
+            }
+            dgr[2 * t] = ar * pr - ai * pi;
+            dgr[2 * t + 1] = ar * pi + ai * pr;
+        }
+    }
+}

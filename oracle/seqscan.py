@@ -1,0 +1,79 @@
+"""ORACLE (test infrastructure, not part of the product).
+
+numpy-facing loader of oracle/seqscan.c: the sequential fp64 recurrences that
+define the operator.  Inputs are fp32 (or complex64) arrays of shape
+(..., T); results are float64 (complex128).
+"""
+
+import ctypes
+import subprocess
+from pathlib import Path
+
+import numpy as np
+
+_HERE = Path(__file__).resolve().parent
+_LIB_PATH = _HERE / "_build" / "libseqscan.so"
+_lib = None
+
+
+def build() -> Path:
+    subprocess.run(["make", "-C", str(_HERE), "all"], check=True, capture_output=True)
+    return _LIB_PATH
+
+
+def _load():
+    global _lib
+    if _lib is None:
+        if not _LIB_PATH.exists():
+            build()
+        lib = ctypes.CDLL(str(_LIB_PATH))
+        p = ctypes.c_void_p
+        i64 = ctypes.c_int64
+        lib.seq_forward_f32.argtypes = [p, p, p, i64, i64, ctypes.c_int]
+        lib.seq_forward_c64.argtypes = [p, p, p, i64, i64, ctypes.c_int]
+        lib.seq_backward_f32.argtypes = [p, p, p, p, p, i64, i64]
+        lib.seq_backward_c64.argtypes = [p, p, p, p, p, i64, i64]
+        for f in (lib.seq_forward_f32, lib.seq_forward_c64, lib.seq_backward_f32, lib.seq_backward_c64):
+            f.restype = None
+        _lib = lib
+    return _lib
+
+
+def _prep(a, dtype):
+    a = np.ascontiguousarray(a, dtype=dtype)
+    return a, a.ctypes.data_as(ctypes.c_void_p)
+
+
+def forward(gates, tokens, reverse=False):
+    """Sequential scan in fp64.  Real (float32) or complex (complex64) inputs."""
+    lib = _load()
+    cplx = np.iscomplexobj(gates) or np.iscomplexobj(tokens)
+    dt = np.complex64 if cplx else np.float32
+    g, gp = _prep(gates, dt)
+    x, xp = _prep(tokens, dt)
+    assert g.shape == x.shape
+    T = g.shape[-1]
+    rows = g.size // T if T else 0
+    out = np.empty(g.shape, dtype=np.complex128 if cplx else np.float64)
+    fn = lib.seq_forward_c64 if cplx else lib.seq_forward_f32
+    fn(gp, xp, out.ctypes.data_as(ctypes.c_void_p), rows, T, int(bool(reverse)))
+    return out
+
+
+def backward(gates, states, grad_out):
+    """(d_gates, d_tokens) of the scan for an incoming gradient, in fp64."""
+    lib = _load()
+    cplx = np.iscomplexobj(gates) or np.iscomplexobj(states) or np.iscomplexobj(grad_out)
+    dt = np.complex64 if cplx else np.float32
+    g, gp = _prep(gates, dt)
+    s, sp = _prep(states, dt)
+    d, dp = _prep(grad_out, dt)
+    assert g.shape == s.shape == d.shape
+    T = g.shape[-1]
+    rows = g.size // T if T else 0
+    odt = np.complex128 if cplx else np.float64
+    dg = np.empty(g.shape, dtype=odt)
+    dx = np.empty(g.shape, dtype=odt)
+    fn = lib.seq_backward_c64 if cplx else lib.seq_backward_f32
+    fn(gp, sp, dp, dg.ctypes.data_as(ctypes.c_void_p), dx.ctypes.data_as(ctypes.c_void_p), rows, T)
+    return dg, dx

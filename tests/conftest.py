@@ -1,0 +1,22 @@
+import sys
+from pathlib import Path
+
+import pytest
+
+ROOT = Path(__file__).resolve().parent.parent
+for p in (ROOT, ROOT / "accelerated-scan_amd"):
+    if str(p) not in sys.path:
+        sys.path.insert(0, str(p))
+
+
+def pytest_configure(config):
+    config.addinivalue_line("markers", "gpu: needs a HIP device (run on the MI355X box)")
+
+
+@pytest.fixture(scope="session")
+def golden():
+    import numpy as np
+
+    path = Path(__file__).resolve().parent / "golden" / "ref_scan_golden.npz"
+    with np.load(path, allow_pickle=False) as z:
+        return {k: z[k] for k in z.files}

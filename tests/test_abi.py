@@ -1,0 +1,129 @@
+"""CPU tests of the drop-in boundary: the shared library loads, exports every
+symbol include/ascan.h declares, rejects bad arguments by return code before
+touching the GPU, and the Python operators validate like the reference's
+(accelerated_scan/warp.py:41-44, warp.cuh:394-421, complex.py:160-161).
+No kernel is launched here.
+"""
+
+import ctypes
+import re
+from pathlib import Path
+
+import pytest
+import torch
+
+from accelerated_scan import _abi
+
+ROOT = Path(__file__).resolve().parent.parent
+HEADER = ROOT / "include" / "ascan.h"
+
+
+def declared_functions():
+    text = HEADER.read_text()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return re.findall(r"\b(ascan_[a-z0-9_]+)\s*\(", text)
+
+
+def test_library_exports_every_declared_symbol():
+    lib = ctypes.CDLL(str(_abi.library_path()))
+    names = declared_functions()
+    assert set(names) >= {"ascan_forward", "ascan_backward", "ascan_status_string", "ascan_abi_version"}
+    for name in names:
+        assert hasattr(lib, name), name
+    assert set(_abi.exported_symbols()) == set(names)
+
+
+def test_abi_version_and_status_strings():
+    lib = _abi.load()
+    assert lib.ascan_abi_version() == _abi.ABI_VERSION
+    texts = {lib.ascan_status_string(i).decode() for i in range(6)}
+    assert len(texts) == 6 and "ok" in texts
+    assert lib.ascan_status_string(99).decode() == "unknown status"
+
+
+def test_argument_validation_returns_codes():
+    lib = _abi.load()
+    buf = ctypes.create_string_buffer(64)
+    p = ctypes.addressof(buf)
+    # unknown dtype
+    assert lib.ascan_forward(p, p, p, 1, 4, 7, 0, None) == 3
+    assert lib.ascan_backward(p, p, p, p, p, 1, 4, -1, None) == 3
+    # negative sizes, too many rows
+    assert lib.ascan_forward(p, p, p, -1, 4, 0, 0, None) == 2
+    assert lib.ascan_forward(p, p, p, 1, -4, 0, 0, None) == 2
+    assert lib.ascan_forward(p, p, p, 2**31, 4, 0, 0, None) == 2
+    assert lib.ascan_backward(p, p, p, p, p, 1, -1, 0, None) == 2
+    # empty problems succeed without looking at the pointers
+    assert lib.ascan_forward(None, None, None, 0, 4, 0, 0, None) == 0
+    assert lib.ascan_forward(None, None, None, 4, 0, 0, 0, None) == 0
+    assert lib.ascan_backward(None, None, None, None, None, 0, 0, 3, None) == 0
+    # null pointers
+    assert lib.ascan_forward(None, p, p, 1, 4, 0, 0, None) == 1
+    assert lib.ascan_forward(p, p, None, 1, 4, 0, 0, None) == 1
+    assert lib.ascan_backward(p, p, p, p, None, 1, 4, 0, None) == 1
+    # element misalignment
+    assert lib.ascan_forward(p + 2, p, p, 1, 4, 0, 0, None) == 4
+    assert lib.ascan_forward(p + 1, p, p, 1, 4, 1, 0, None) == 4
+    assert lib.ascan_forward(p + 4, p, p, 1, 4, 3, 0, None) == 4
+    assert lib.ascan_backward(p, p, p, p + 2, p, 1, 4, 0, None) == 4
+
+
+def test_status_becomes_runtime_error():
+    with pytest.raises(RuntimeError, match="unsupported dtype"):
+        _abi.check(3)
+    _abi.check(0)
+    with pytest.raises(RuntimeError, match="unsupported tensor dtype"):
+        _abi.dtype_code(torch.float64)
+
+
+def test_missing_library_fails_loudly(monkeypatch, tmp_path):
+    monkeypatch.setenv("ASCAN_LIBRARY", str(tmp_path / "nope.so"))
+    monkeypatch.setattr(_abi, "_lib", None)
+    with pytest.raises(ImportError, match="HIP library not found"):
+        _abi.load()
+
+
+def test_warp_rejects_host_tensors_and_bad_shapes():
+    from accelerated_scan import warp
+
+    g = torch.rand(1, 2, 8)
+    x = torch.rand(1, 2, 8)
+    with pytest.raises(RuntimeError, match="device tensor"):
+        warp.scan(g, x)
+    with pytest.raises(RuntimeError, match="device tensor"):
+        warp.warpscan_backward(g, g, g, g, g)
+    with pytest.raises(AssertionError):
+        warp.scan(g, torch.rand(1, 2, 9))
+    with pytest.raises(AssertionError):
+        warp.scan(torch.rand(2, 1, 8, 2)[..., 0], x.reshape(2, 1, 8))
+    with pytest.raises(AssertionError):
+        warp.scan(g, torch.rand(1, 2, 16)[:, :, ::2])
+
+
+def test_scalar_and_complex_validation():
+    from accelerated_scan import complex as cscan
+    from accelerated_scan import scalar
+
+    g = torch.rand(1, 2, 8)
+    with pytest.raises(RuntimeError, match="device tensor"):
+        scalar.scan(g, g)
+    with pytest.raises(TypeError, match="forget must be a complex tensor"):
+        cscan.scan(g, g)
+    gc = torch.polar(torch.rand(1, 2, 8), torch.rand(1, 2, 8))
+    with pytest.raises(RuntimeError, match="device tensor"):
+        cscan.scan(gc, g)
+    with pytest.raises(AssertionError):
+        cscan.scan(gc, torch.rand(1, 2, 9))
+
+
+def test_module_surface_matches_reference():
+    import accelerated_scan
+    from accelerated_scan import complex as cscan
+    from accelerated_scan import scalar, warp
+
+    assert accelerated_scan.__version__ == "0.3.1"
+    for name in ("scan", "Scan", "scan_forward", "warpscan_forward", "warpscan_backward"):
+        assert hasattr(warp, name)
+    for mod in (scalar, cscan):
+        assert hasattr(mod, "scan") and hasattr(mod, "Scan")
+        assert issubclass(mod.Scan, torch.autograd.Function)

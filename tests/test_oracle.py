@@ -1,0 +1,218 @@
+"""CPU tests that pin the oracle (oracle/ref_scan.py, oracle/seqscan.c).
+
+Three independent anchors:
+  * golden outputs recorded from the reference's own tree scan (bit-exact for
+    the forward values, tight tolerance for autograd gradients);
+  * the sequential recurrence in fp64 (different algorithm, different language);
+  * closed forms that reduce the operator to library routines (cumsum, cumprod,
+    geometric series) and the flip identity for the reverse scan.
+The backward formulas are pinned the way the reference proves them
+(tests/test_eq.py:65-90) and by autograd through an explicit fp64 loop.
+"""
+
+import doctest
+import math
+
+import numpy as np
+import pytest
+import torch
+
+from oracle import ref_scan, seqscan
+
+SEQLENS = [2**i for i in range(5, 13)] + [8000, 16323]
+
+REAL_CASES = ["cfg1_fwd", "pow2_rev", "pad_fwd", "pad_rev", "tiny_T2", "tiny_T3", "long_memory",
+              "grads_fwd", "grads_pow2"]
+
+
+def test_doctests():
+    assert doctest.testmod(ref_scan).failed == 0
+
+
+@pytest.mark.parametrize("name", REAL_CASES)
+def test_tree_scan_bit_exact_vs_reference_golden(golden, name):
+    gates = torch.from_numpy(golden[f"{name}.gates"])
+    tokens = torch.from_numpy(golden[f"{name}.tokens"])
+    reverse = bool(golden[f"{name}.reverse"])
+    out = ref_scan.scan(gates, tokens, reverse=reverse)
+    assert torch.equal(out, torch.from_numpy(golden[f"{name}.out"]))
+
+
+@pytest.mark.parametrize("name", ["grads_fwd", "grads_pow2"])
+def test_tree_scan_gradients_vs_reference_golden(golden, name):
+    gates = torch.from_numpy(golden[f"{name}.gates"]).requires_grad_(True)
+    tokens = torch.from_numpy(golden[f"{name}.tokens"]).requires_grad_(True)
+    grad_out = torch.from_numpy(golden[f"{name}.grad_out"])
+    out = ref_scan.scan(gates, tokens)
+    dg, dt = torch.autograd.grad(out, (gates, tokens), grad_out)
+    # same graph up to the order in which autograd sums a node's contributions
+    torch.testing.assert_close(dg, torch.from_numpy(golden[f"{name}.d_gates"]), atol=1e-6, rtol=1e-6)
+    torch.testing.assert_close(dt, torch.from_numpy(golden[f"{name}.d_tokens"]), atol=1e-6, rtol=1e-6)
+
+
+@pytest.mark.parametrize("name", ["complex_real_tokens", "complex_complex_tokens"])
+def test_tree_scan_complex_vs_reference_golden(golden, name):
+    gates = torch.from_numpy(golden[f"{name}.gates"]).requires_grad_(True)
+    tokens = torch.from_numpy(golden[f"{name}.tokens"]).requires_grad_(True)
+    grad_out = torch.from_numpy(golden[f"{name}.grad_out"])
+    out = ref_scan.scan(gates, tokens)
+    assert torch.equal(out.detach(), torch.from_numpy(golden[f"{name}.out"]))
+    dg, dt = torch.autograd.grad(out, (gates, tokens), grad_out)
+    torch.testing.assert_close(dg, torch.from_numpy(golden[f"{name}.d_gates"]), atol=1e-5, rtol=1e-5)
+    torch.testing.assert_close(dt, torch.from_numpy(golden[f"{name}.d_tokens"]), atol=1e-5, rtol=1e-5)
+
+
+@pytest.mark.parametrize("name", REAL_CASES + ["complex_real_tokens", "complex_complex_tokens"])
+def test_sequential_fp64_vs_reference_golden(golden, name):
+    """The C loops agree with the reference's recorded outputs to fp32 rounding."""
+    gates = golden[f"{name}.gates"]
+    tokens = golden[f"{name}.tokens"]
+    reverse = bool(golden.get(f"{name}.reverse", 0))
+    truth = seqscan.forward(gates, tokens, reverse=reverse)
+    ref = golden[f"{name}.out"]
+    scale = np.abs(truth).max()
+    assert np.abs(truth - ref).max() <= 2e-6 * scale
+    if f"{name}.d_gates" in golden:
+        if np.iscomplexobj(gates) and not np.iscomplexobj(tokens):
+            tokens_c = tokens.astype(np.complex64)
+        states = seqscan.forward(gates, tokens).astype(gates.dtype)
+        dg, dt = seqscan.backward(gates, states, golden[f"{name}.grad_out"])
+        ref_dt = golden[f"{name}.d_tokens"]
+        if not np.iscomplexobj(ref_dt) and np.iscomplexobj(dt):
+            dt = dt.real  # real tokens keep the real part (accelerated_scan/complex.py:217-218)
+        assert np.abs(dt - ref_dt).max() <= 1e-5 * np.abs(dt).max()
+        assert np.abs(dg - golden[f"{name}.d_gates"]).max() <= 1e-5 * np.abs(dg).max()
+
+
+@pytest.mark.parametrize("T", [1, 2, 3, 5, 31, 32, 33, 100, 1024, 1025, 4097])
+@pytest.mark.parametrize("reverse", [False, True])
+def test_tree_scan_vs_sequential_fp64(T, reverse):
+    gen = torch.Generator().manual_seed(T)
+    gates = torch.rand(2, 3, T, generator=gen)
+    tokens = torch.randn(2, 3, T, generator=gen)
+    out = ref_scan.scan(gates, tokens, reverse=reverse).numpy()
+    truth = seqscan.forward(gates.numpy(), tokens.numpy(), reverse=reverse)
+    np.testing.assert_allclose(out, truth, rtol=2e-6, atol=2e-6)
+
+
+def test_closed_forms():
+    gen = torch.Generator().manual_seed(0)
+    T = 777
+    tokens = torch.randn(1, 4, T, generator=gen, dtype=torch.float64)
+    gates = 0.5 + torch.rand(1, 4, T, generator=gen, dtype=torch.float64)
+    ones, zeros = torch.ones_like(tokens), torch.zeros_like(tokens)
+    # gates == 1: running sum
+    torch.testing.assert_close(ref_scan.scan(ones, tokens), torch.cumsum(tokens, -1), rtol=1e-12, atol=1e-12)
+    # gates == 0: the tokens themselves
+    assert torch.equal(ref_scan.scan(zeros, tokens), tokens)
+    # tokens == 0: zero
+    assert torch.equal(ref_scan.scan(gates, zeros), zeros)
+    # impulse at t = 0: running product of gates[1:]
+    impulse = zeros.clone()
+    impulse[..., 0] = 1.0
+    g1 = gates.clone()
+    g1[..., 0] = 1.0
+    torch.testing.assert_close(ref_scan.scan(gates, impulse), torch.cumprod(g1, -1), rtol=1e-12, atol=0)
+    # constant gate a, tokens == 1: (1 - a^(t+1)) / (1 - a)
+    a = 0.9
+    t = torch.arange(T, dtype=torch.float64)
+    closed = (1 - a ** (t + 1)) / (1 - a)
+    got = ref_scan.scan(torch.full_like(tokens, a), ones)
+    torch.testing.assert_close(got, closed.expand_as(got), rtol=1e-12, atol=0)
+    # and the same through the C loop (fp32 inputs)
+    seq = seqscan.forward(np.full((1, T), 0.5, np.float32), np.ones((1, T), np.float32))
+    np.testing.assert_allclose(seq[0], (1 - 0.5 ** (np.arange(T) + 1.0)) / 0.5, rtol=1e-15)
+    seq = seqscan.forward(np.ones((2, T), np.float32), tokens[0, :2].float().numpy())
+    np.testing.assert_allclose(seq, np.cumsum(tokens[0, :2].float().numpy().astype(np.float64), -1), rtol=1e-12)
+
+
+@pytest.mark.parametrize("T", [2, 7, 64, 1000])
+def test_reverse_is_flip_of_forward(T):
+    gen = torch.Generator().manual_seed(T)
+    gates = torch.rand(1, 3, T, generator=gen, dtype=torch.float64)
+    tokens = torch.randn(1, 3, T, generator=gen, dtype=torch.float64)
+    rev = ref_scan.scan(gates, tokens, reverse=True)
+    fwd = ref_scan.scan(gates.flip(-1).contiguous(), tokens.flip(-1).contiguous()).flip(-1)
+    torch.testing.assert_close(rev, fwd, rtol=1e-12, atol=1e-12)
+    truth = seqscan.forward(gates.float().numpy(), tokens.float().numpy(), reverse=True)
+    truth_flip = seqscan.forward(gates.float().numpy()[..., ::-1], tokens.float().numpy()[..., ::-1])[..., ::-1]
+    np.testing.assert_array_equal(truth, truth_flip)
+
+
+@pytest.mark.parametrize("seqlen", SEQLENS)
+def test_backward_is_shifted_reverse_scan(seqlen):
+    """The identity the reference proves at tests/test_eq.py:65-90, same tolerances."""
+    gen = torch.Generator().manual_seed(1)
+    f = torch.randn(1, 1, seqlen, generator=gen, requires_grad=True)
+    x = torch.randn(1, 1, seqlen, generator=gen, requires_grad=True)
+    c = ref_scan.scan(f, x)
+    ones = torch.ones_like(c)
+    f_shift = torch.cat([f, torch.ones_like(f[:, :, :1])], dim=-1)[:, :, 1:].contiguous()
+    dcdx = ref_scan.scan(f_shift, ones, reverse=True)
+    c_shift = torch.cat([torch.zeros_like(c[:, :, :1]), c], dim=-1)[:, :, :-1].contiguous()
+    dcdf = dcdx * c_shift
+    c.sum().backward()
+    torch.testing.assert_close(x.grad, dcdx, atol=1e-5, rtol=1.3e-6)
+    torch.testing.assert_close(f.grad, dcdf, atol=2e-5, rtol=1.3e-6)
+
+
+def _loop_scan(gates, tokens):
+    """The recurrence as an explicit Python loop (autograd-friendly, any dtype)."""
+    state = torch.zeros_like(tokens[..., 0])
+    outs = []
+    for t in range(tokens.shape[-1]):
+        state = gates[..., t] * state + tokens[..., t]
+        outs.append(state)
+    return torch.stack(outs, dim=-1)
+
+
+@pytest.mark.parametrize("T", [1, 2, 9, 130])
+def test_sequential_backward_vs_autograd_of_loop(T):
+    gen = torch.Generator().manual_seed(100 + T)
+    gates = torch.rand(2, 2, T, generator=gen)
+    tokens = torch.randn(2, 2, T, generator=gen)
+    grad_out = torch.randn(2, 2, T, generator=gen)
+    g64 = gates.double().requires_grad_(True)
+    t64 = tokens.double().requires_grad_(True)
+    out = _loop_scan(g64, t64)
+    dg_ref, dt_ref = torch.autograd.grad(out, (g64, t64), grad_out.double())
+    states = seqscan.forward(gates.numpy(), tokens.numpy()).astype(np.float32)
+    dg, dt = seqscan.backward(gates.numpy(), states, grad_out.numpy())
+    np.testing.assert_allclose(dt, dt_ref.numpy(), rtol=1e-12, atol=1e-12)
+    # states were rounded to fp32 before the multiply
+    np.testing.assert_allclose(dg, dg_ref.numpy(), rtol=1e-6, atol=1e-6)
+
+
+@pytest.mark.parametrize("T", [1, 2, 9, 130])
+@pytest.mark.parametrize("real_tokens", [False, True])
+def test_sequential_complex_backward_vs_autograd_of_loop(T, real_tokens):
+    gen = torch.Generator().manual_seed(200 + T)
+    angle = 2 * math.pi * torch.rand(1, 3, T, generator=gen)
+    radius = 0.9 + 0.1 * torch.rand(1, 3, T, generator=gen)
+    gates = torch.polar(radius, angle)
+    if real_tokens:
+        tokens = torch.randn(1, 3, T, generator=gen)
+    else:
+        tokens = torch.complex(torch.randn(1, 3, T, generator=gen), torch.randn(1, 3, T, generator=gen))
+    grad_out = torch.complex(torch.randn(1, 3, T, generator=gen), torch.randn(1, 3, T, generator=gen))
+    g128 = gates.to(torch.complex128).requires_grad_(True)
+    t128 = (tokens.double() if real_tokens else tokens.to(torch.complex128)).requires_grad_(True)
+    out = _loop_scan(g128, t128.to(torch.complex128))
+    dg_ref, dt_ref = torch.autograd.grad(out, (g128, t128), grad_out.to(torch.complex128))
+    fwd = seqscan.forward(gates.numpy(), tokens.numpy().astype(np.complex64))
+    np.testing.assert_allclose(fwd, out.detach().numpy(), rtol=1e-12, atol=1e-12)
+    dg, dt = seqscan.backward(gates.numpy(), fwd.astype(np.complex64), grad_out.numpy())
+    if real_tokens:
+        dt = dt.real
+    np.testing.assert_allclose(dt, dt_ref.numpy(), rtol=1e-12, atol=1e-12)
+    np.testing.assert_allclose(dg, dg_ref.numpy(), rtol=1e-5, atol=1e-5)
+
+
+def test_tree_scan_complex_vs_sequential():
+    gen = torch.Generator().manual_seed(3)
+    T = 1000
+    gates = torch.polar(0.99 + 0.01 * torch.rand(1, 4, T, generator=gen), 2 * math.pi * torch.rand(1, 4, T, generator=gen))
+    tokens = torch.randn(1, 4, T, generator=gen).tanh()
+    out = ref_scan.scan(gates, tokens).numpy()
+    truth = seqscan.forward(gates.numpy(), tokens.numpy().astype(np.complex64))
+    np.testing.assert_allclose(out, truth, rtol=1e-4, atol=1e-5)

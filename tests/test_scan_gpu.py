@@ -1,0 +1,546 @@
+"""GPU parity tests: the HIP path (through the C ABI) against the oracle.
+
+Structure, seeds, shapes, distributions and tolerances follow the reference's
+own differential tests (tests/test_eq.py:9-62, tests/tests_eq_complex.py:7-86);
+the oracle is oracle/ref_scan.py run on the same device tensors (as the
+reference runs its ref.scan), backed by the sequential fp64 loops of
+oracle/seqscan.c where an independent truth is wanted.
+
+Tolerances
+  fp32  vs tree scan : atol 1e-7, rtol 1.3e-6           (tests/test_eq.py:13-14)
+  bf16  vs bf16 tree : atol 1e-1, rtol 1.6e-2           (tests/test_eq.py:13-14)
+  fp16  vs fp16 tree : atol 12e-3, rtol 1e-3            (tests/test_eq.py:13-14)
+  bf16 / fp16 vs the fp32 tree scan of the same (up-cast) inputs, possible here
+  because the kernels accumulate in fp32: one storage ulp (2^-8 / 2^-11
+  relative) plus 1e-5 of the largest reference magnitude; twice that for
+  d_gates, which multiplies by states that were themselves rounded once.
+  complex64          : atol 1e-5, rtol 1e-4             (tests/tests_eq_complex.py:23)
+  long-memory fp32   : 1e-5 relative to the largest magnitude of the row set,
+                       against the fp64 recurrence.
+"""
+
+import ctypes
+import math
+
+import numpy as np
+import pytest
+import torch
+
+from oracle import ref_scan, seqscan
+
+pytestmark = pytest.mark.gpu
+
+DEVICE = "cuda"
+
+seeds = [3407, 4, 42, 57]
+seqlens = [2**i for i in range(5, 17)] + [16323, 8000, 33753, 127323]
+dtypes = [torch.float32, torch.bfloat16, torch.float16]
+atol = {torch.float32: 1e-7, torch.bfloat16: 1e-1, torch.float16: 12e-3}
+rtol = {torch.float32: 1.3e-6, torch.bfloat16: 1.6e-2, torch.float16: 1e-3}
+storage_ulp = {torch.bfloat16: 2.0**-8, torch.float16: 2.0**-11}
+
+
+@pytest.fixture(scope="module", autouse=True)
+def _need_gpu_and_library():
+    assert torch.cuda.is_available(), "these tests need the MI355X"
+    from accelerated_scan import _abi
+
+    _abi.load()  # raises if the HIP library is missing: no fallback exists
+
+
+def scan_warp(*a):
+    from accelerated_scan.warp import scan
+
+    return scan(*a)
+
+
+def scan_scalar(*a):
+    from accelerated_scan.scalar import scan
+
+    return scan(*a)
+
+
+def init(seed, batch_size=1, dim=512, seqlen=32, requires_grad=False, dtype=torch.float32):
+    torch.manual_seed(seed)
+    gates = torch.rand(batch_size, dim, seqlen, requires_grad=requires_grad, dtype=dtype, device=DEVICE)
+    tokens = torch.rand(batch_size, dim, seqlen, requires_grad=requires_grad, dtype=dtype, device=DEVICE)
+    return gates, tokens
+
+
+def assert_close_storage(got, ref32, dtype, factor=1.0):
+    """Reduced-precision result against an fp32 reference of the same inputs."""
+    scale = ref32.abs().max().item()
+    torch.testing.assert_close(
+        got.float(), ref32, atol=factor * 1e-5 * scale + 1e-30, rtol=factor * storage_ulp[dtype]
+    )
+
+
+# ---------------------------------------------------------------------------
+# The reference's test matrix (tests/test_eq.py:26-62)
+# ---------------------------------------------------------------------------
+@pytest.mark.parametrize("scan", [scan_warp, scan_scalar], ids=["warp", "scalar"])
+@pytest.mark.parametrize("seed", seeds)
+@pytest.mark.parametrize("seqlen", seqlens)
+@pytest.mark.parametrize("dtype", dtypes, ids=["fp32", "bf16", "fp16"])
+@torch.inference_mode()
+def test_eq_forward(scan, seed, seqlen, dtype):
+    if scan is scan_scalar and seed != seeds[0]:
+        pytest.skip("scalar shares the backend; one seed is enough")
+    gates, tokens = init(seed, seqlen=seqlen, dtype=dtype)
+    out = scan(gates, tokens)
+    assert out.dtype == dtype and out.shape == tokens.shape
+    out_ref = ref_scan.scan(gates, tokens)
+    torch.testing.assert_close(out, out_ref, atol=atol[dtype], rtol=rtol[dtype])
+    if dtype != torch.float32:
+        assert_close_storage(out, ref_scan.scan(gates.float(), tokens.float()), dtype)
+
+
+@pytest.mark.parametrize("seed", seeds)
+@pytest.mark.parametrize("seqlen", seqlens)
+@pytest.mark.parametrize("dtype", dtypes, ids=["fp32", "bf16", "fp16"])
+def test_eq_backward(seed, seqlen, dtype):
+    gates, tokens = init(seed, seqlen=seqlen, requires_grad=True, dtype=dtype)
+    scan_warp(gates, tokens).mean(dim=-1).sum().backward()
+    gates_grad, tokens_grad = gates.grad, tokens.grad
+    assert gates_grad.dtype == dtype and tokens_grad.dtype == dtype
+
+    gates_ref, tokens_ref = init(seed, seqlen=seqlen, requires_grad=True, dtype=dtype)
+    ref_scan.scan(gates_ref, tokens_ref).mean(dim=-1).sum().backward()
+    torch.testing.assert_close(gates_grad, gates_ref.grad, atol=atol[dtype], rtol=rtol[dtype])
+    torch.testing.assert_close(tokens_grad, tokens_ref.grad, atol=atol[dtype], rtol=rtol[dtype])
+
+    if dtype != torch.float32:
+        g32 = gates.detach().float().requires_grad_(True)
+        t32 = tokens.detach().float().requires_grad_(True)
+        ref_scan.scan(g32, t32).mean(dim=-1).sum().backward()
+        # the incoming gradient 1/T is itself rounded to the storage dtype by autograd
+        assert_close_storage(tokens_grad, t32.grad, dtype, factor=2.0)
+        assert_close_storage(gates_grad, g32.grad, dtype, factor=3.0)
+
+
+# ---------------------------------------------------------------------------
+# Every small T against the fp64 recurrence: tile, wave and vector boundaries,
+# aligned and unaligned rows, all dtypes, forward / reverse / backward.
+# ---------------------------------------------------------------------------
+def _truth_inputs(rows, T, dtype, seed):
+    gen = torch.Generator().manual_seed(seed)
+    if dtype == torch.complex64:
+        gates = torch.polar(0.5 + 0.5 * torch.rand(rows, T, generator=gen), 2 * math.pi * torch.rand(rows, T, generator=gen))
+        mk = lambda: torch.complex(torch.randn(rows, T, generator=gen), torch.randn(rows, T, generator=gen))
+        return gates, mk(), mk()
+    gates = torch.rand(rows, T, generator=gen).to(dtype)
+    tokens = torch.randn(rows, T, generator=gen).to(dtype)
+    grad_out = torch.randn(rows, T, generator=gen).to(dtype)
+    return gates, tokens, grad_out
+
+
+def _np32(t):
+    return t.numpy() if t.dtype == torch.complex64 else t.float().numpy()
+
+
+def _check_against_truth(gates, tokens, grad_out, dtype, what=""):
+    """Runs forward, reverse and backward on the GPU for (rows, T) host tensors."""
+    from accelerated_scan import _abi
+
+    rows, T = gates.shape
+    g, x, d = (t.to(DEVICE).reshape(1, rows, T) for t in (gates, tokens, grad_out))
+    out = torch.empty_like(x)
+    rev = torch.empty_like(x)
+    _abi.forward(g, x, out, False)
+    _abi.forward(g, x, rev, True)
+    dg = torch.empty_like(x)
+    dx = torch.empty_like(x)
+    _abi.backward(g, out, d, dg, dx)
+    torch.cuda.synchronize()
+
+    if dtype == torch.complex64 or dtype == torch.float32:
+        tol = dict(rtol=2e-5, atol=2e-5)
+    else:
+        tol = dict(rtol=2 * storage_ulp[dtype], atol=2 * storage_ulp[dtype])
+    t_out = seqscan.forward(_np32(gates), _np32(tokens))
+    t_rev = seqscan.forward(_np32(gates), _np32(tokens), reverse=True)
+    # backward consumes the states the GPU produced (already rounded to storage)
+    states = out.reshape(rows, T).cpu()
+    t_dg, t_dx = seqscan.backward(_np32(gates), _np32(states), _np32(grad_out))
+    for name, got, want in (("out", out, t_out), ("rev", rev, t_rev), ("d_tokens", dx, t_dx), ("d_gates", dg, t_dg)):
+        got = _np32(got.reshape(rows, T).cpu())
+        scale = max(1.0, float(np.abs(want).max()))
+        np.testing.assert_allclose(
+            got, want, rtol=tol["rtol"], atol=tol["atol"] * scale, err_msg=f"{what} {name} rows={rows} T={T} {dtype}"
+        )
+
+
+ALL_DTYPES = [torch.float32, torch.bfloat16, torch.float16, torch.complex64]
+ALL_IDS = ["fp32", "bf16", "fp16", "c64"]
+
+
+@pytest.mark.parametrize("dtype", ALL_DTYPES, ids=ALL_IDS)
+def test_every_small_T(dtype):
+    for T in list(range(1, 70)) + list(range(120, 136)) + list(range(250, 262)) + [511, 512, 513, 520]:
+        gates, tokens, grad_out = _truth_inputs(5, T, dtype, seed=T)
+        _check_against_truth(gates, tokens, grad_out, dtype, what="small")
+
+
+@pytest.mark.parametrize("dtype", ALL_DTYPES, ids=ALL_IDS)
+@pytest.mark.parametrize("T", [1016, 1024, 1032, 2040, 2048, 2056, 4088, 4096, 4104, 5000, 8192 + 8, 16384 - 8])
+def test_tile_boundaries_one_wave_per_row(dtype, T):
+    # rows >= 2048 selects one wave per row
+    gates, tokens, grad_out = _truth_inputs(2050, T, dtype, seed=T)
+    _check_against_truth(gates, tokens, grad_out, dtype, what="W1")
+
+
+@pytest.mark.parametrize("dtype", ALL_DTYPES, ids=ALL_IDS)
+@pytest.mark.parametrize("rows,T", [(600, 4096), (600, 4104), (513, 20000), (700, 1032), (1024, 3000)])
+def test_four_waves_per_row(dtype, rows, T):
+    gates, tokens, grad_out = _truth_inputs(rows, T, dtype, seed=T + rows)
+    _check_against_truth(gates, tokens, grad_out, dtype, what="W4")
+
+
+@pytest.mark.parametrize("dtype", ALL_DTYPES, ids=ALL_IDS)
+@pytest.mark.parametrize("rows,T", [(3, 16384), (7, 16392), (2, 65536 + 64), (5, 4104), (1, 40000), (9, 131072)])
+def test_sixteen_waves_per_row(dtype, rows, T):
+    gates, tokens, grad_out = _truth_inputs(rows, T, dtype, seed=T + rows)
+    _check_against_truth(gates, tokens, grad_out, dtype, what="W16")
+
+
+@pytest.mark.parametrize("dtype", ALL_DTYPES, ids=ALL_IDS)
+@pytest.mark.parametrize("rows,T", [(3, 1000), (2050, 1031), (5, 4099), (600, 5001), (2, 33753)])
+def test_unaligned_rows(dtype, rows, T):
+    """T not a multiple of the vector width: rows start at unaligned addresses."""
+    gates, tokens, grad_out = _truth_inputs(rows, T, dtype, seed=T + rows)
+    _check_against_truth(gates, tokens, grad_out, dtype, what="unaligned")
+
+
+@pytest.mark.parametrize("dtype", ALL_DTYPES, ids=ALL_IDS)
+def test_unaligned_base_pointer(dtype):
+    """Views with a storage offset: base pointers off the 16-byte grid."""
+    from accelerated_scan import _abi
+
+    rows, T = 6, 2048
+    gates, tokens, grad_out = _truth_inputs(rows, T, dtype, seed=9)
+
+    def offset_copy(t):
+        flat = torch.empty(rows * T + 1, dtype=t.dtype, device=DEVICE)
+        view = flat[1:].view(1, rows, T)
+        view.copy_(t.reshape(1, rows, T))
+        assert view.data_ptr() % 16 != 0 and view.is_contiguous()
+        return view
+
+    g, x = offset_copy(gates), offset_copy(tokens)
+    out = offset_copy(torch.zeros_like(tokens))
+    _abi.forward(g, x, out, False)
+    ref = torch.empty(1, rows, T, dtype=dtype, device=DEVICE)
+    _abi.forward(gates.to(DEVICE).view(1, rows, T), tokens.to(DEVICE).view(1, rows, T), ref, False)
+    assert torch.equal(torch.view_as_real(out) if dtype == torch.complex64 else out,
+                       torch.view_as_real(ref) if dtype == torch.complex64 else ref)
+    d = offset_copy(grad_out)
+    dg, dx = offset_copy(torch.zeros_like(tokens)), offset_copy(torch.zeros_like(tokens))
+    _abi.backward(g, out, d, dg, dx)
+    rdg, rdx = torch.empty_like(ref), torch.empty_like(ref)
+    _abi.backward(gates.to(DEVICE).view(1, rows, T), ref, grad_out.to(DEVICE).view(1, rows, T), rdg, rdx)
+    for a, b in ((dg, rdg), (dx, rdx)):
+        if dtype == torch.complex64:
+            a, b = torch.view_as_real(a), torch.view_as_real(b)
+        assert torch.equal(a, b)
+
+
+# ---------------------------------------------------------------------------
+# BASELINE configurations
+# ---------------------------------------------------------------------------
+def test_config1_cpu_plumbing(golden):
+    """fp32 (1, 64, 1024), U(0,1): GPU against the CPU tree scan and the recorded reference output."""
+    gen = torch.Generator().manual_seed(3407)
+    gates = torch.rand(1, 64, 1024, generator=gen)
+    tokens = torch.rand(1, 64, 1024, generator=gen)
+    cpu = ref_scan.scan(gates, tokens)
+    out = scan_warp(gates.to(DEVICE), tokens.to(DEVICE)).cpu()
+    torch.testing.assert_close(out, cpu, atol=1e-7, rtol=1.3e-6)
+    # and on the exact inputs / outputs recorded from the reference implementation
+    g = torch.from_numpy(golden["cfg1_fwd.gates"]).to(DEVICE)
+    x = torch.from_numpy(golden["cfg1_fwd.tokens"]).to(DEVICE)
+    torch.testing.assert_close(scan_warp(g, x).cpu(), torch.from_numpy(golden["cfg1_fwd.out"]), atol=1e-7, rtol=1.3e-6)
+
+
+def _long_memory(shape, seed):
+    gen = torch.Generator().manual_seed(seed)
+    gates = 0.999 + 0.001 * torch.rand(*shape, generator=gen)
+    tokens = torch.rand(*shape, generator=gen)
+    grad_out = torch.randn(*shape, generator=gen)
+    return gates, tokens, grad_out
+
+
+def _rel_err(got, want):
+    want = torch.as_tensor(want)
+    return ((got.double().cpu() - want).abs().max() / want.abs().max()).item()
+
+
+def test_config2_forward_fp32_long_memory():
+    """fp32 (8, 1536, 4096), gates = 0.999 + 0.001 U: forward only."""
+    gates, tokens, _ = _long_memory((8, 1536, 4096), 3407)
+    out = scan_warp(gates.to(DEVICE), tokens.to(DEVICE))
+    truth = seqscan.forward(gates.numpy(), tokens.numpy())
+    tree = ref_scan.scan(gates.to(DEVICE), tokens.to(DEVICE))
+    e_gpu, e_tree = _rel_err(out, truth), _rel_err(tree, truth)
+    print(f"config2 rel err vs fp64: hip {e_gpu:.3e}, tree scan {e_tree:.3e}")
+    assert e_gpu <= 1e-5
+    torch.testing.assert_close(out, tree, rtol=1e-5, atol=1e-5 * tree.abs().max().item())
+
+
+def test_config3_bf16_forward_backward():
+    """bf16 storage (8, 1536, 16384), U(0,1) inputs, N(0,1) upstream gradient."""
+    gen = torch.Generator().manual_seed(3407)
+    shape = (8, 1536, 16384)
+    gates = torch.rand(*shape, generator=gen).bfloat16().to(DEVICE).requires_grad_(True)
+    tokens = torch.rand(*shape, generator=gen).bfloat16().to(DEVICE).requires_grad_(True)
+    grad_out = torch.randn(*shape, generator=gen).bfloat16().to(DEVICE)
+    out = scan_warp(gates, tokens)
+    dg, dx = torch.autograd.grad(out, (gates, tokens), grad_out)
+    assert out.dtype == dg.dtype == dx.dtype == torch.bfloat16
+
+    # fp64 truth on a slice of rows (every 97th), from the same bf16 values
+    rows = slice(0, 1536, 97)
+    g32 = gates.detach()[:, rows].float().cpu().numpy()
+    x32 = tokens.detach()[:, rows].float().cpu().numpy()
+    d32 = grad_out[:, rows].float().cpu().numpy()
+    t_out = seqscan.forward(g32, x32)
+    t_dg, t_dx = seqscan.backward(g32, out.detach()[:, rows].float().cpu().numpy(), d32)
+    for name, got, want in (("out", out, t_out), ("d_tokens", dx, t_dx), ("d_gates", dg, t_dg)):
+        got = got.detach()[:, rows].float().cpu().numpy()
+        np.testing.assert_allclose(got, want, rtol=2.0**-8, atol=1e-5 * np.abs(want).max(), err_msg=name)
+
+    # the whole tensor against the fp32 tree scan run on the device
+    g_ref = gates.detach().float().requires_grad_(True)
+    x_ref = tokens.detach().float().requires_grad_(True)
+    ref = ref_scan.scan(g_ref, x_ref)
+    rdg, rdx = torch.autograd.grad(ref, (g_ref, x_ref), grad_out.float())
+    assert_close_storage(out.detach(), ref.detach(), torch.bfloat16)
+    assert_close_storage(dx, rdx, torch.bfloat16)
+    assert_close_storage(dg, rdg, torch.bfloat16, factor=2.0)
+
+
+def test_config4_long_sequence_fp32():
+    """fp32 (1, 512, 131072): more than one tile per row, carry along T, fwd + bwd."""
+    gates, tokens, grad_out = _long_memory((1, 512, 131072), 3407)
+    g = gates.to(DEVICE).requires_grad_(True)
+    x = tokens.to(DEVICE).requires_grad_(True)
+    out = scan_warp(g, x)
+    dg, dx = torch.autograd.grad(out, (g, x), grad_out.to(DEVICE))
+    t_out = seqscan.forward(gates.numpy(), tokens.numpy())
+    t_dg, t_dx = seqscan.backward(gates.numpy(), out.detach().cpu().numpy(), grad_out.numpy())
+    errs = {"out": _rel_err(out.detach(), t_out), "d_tokens": _rel_err(dx, t_dx), "d_gates": _rel_err(dg, t_dg)}
+    print("config4 rel err vs fp64:", errs)
+    assert max(errs.values()) <= 1e-5
+    # against the tree scan and its autograd, as the reference's tests compare
+    g_ref = gates.to(DEVICE).requires_grad_(True)
+    x_ref = tokens.to(DEVICE).requires_grad_(True)
+    ref = ref_scan.scan(g_ref, x_ref)
+    rdg, rdx = torch.autograd.grad(ref, (g_ref, x_ref), grad_out.to(DEVICE))
+    for got, want in ((out.detach(), ref.detach()), (dx, rdx), (dg, rdg)):
+        torch.testing.assert_close(got, want, rtol=1e-5, atol=1e-5 * want.abs().max().item())
+
+
+def test_config5_complex64_forward_backward():
+    """complex64 (4, 1024, 8192): gates r e^{i theta}, r ~ U(0.9, 1), theta ~ U(-pi, pi)."""
+    from accelerated_scan.complex import scan as scan_complex
+
+    gen = torch.Generator().manual_seed(3407)
+    shape = (4, 1024, 8192)
+    radius = 0.9 + 0.1 * torch.rand(*shape, generator=gen)
+    theta = (2 * torch.rand(*shape, generator=gen) - 1) * math.pi
+    gates = torch.polar(radius, theta)
+    tokens = torch.complex(torch.randn(*shape, generator=gen), torch.randn(*shape, generator=gen))
+    grad_out = torch.complex(torch.randn(*shape, generator=gen), torch.randn(*shape, generator=gen))
+
+    g = gates.to(DEVICE).requires_grad_(True)
+    x = tokens.to(DEVICE).requires_grad_(True)
+    out = scan_complex(g, x)
+    dg, dx = torch.autograd.grad(out, (g, x), grad_out.to(DEVICE))
+
+    g_ref = gates.to(DEVICE).requires_grad_(True)
+    x_ref = tokens.to(DEVICE).requires_grad_(True)
+    ref = ref_scan.scan(g_ref, x_ref)
+    rdg, rdx = torch.autograd.grad(ref, (g_ref, x_ref), grad_out.to(DEVICE))
+    torch.testing.assert_close(out.detach(), ref.detach(), atol=1e-5, rtol=1e-4)
+    torch.testing.assert_close(dx, rdx, atol=1e-5 * rdx.abs().max().item(), rtol=1e-4)
+    torch.testing.assert_close(dg, rdg, atol=1e-5 * rdg.abs().max().item(), rtol=1e-4)
+
+    rows = slice(0, 1024, 61)
+    t_out = seqscan.forward(gates[:, rows].numpy(), tokens[:, rows].numpy())
+    t_dg, t_dx = seqscan.backward(gates[:, rows].numpy(), out.detach()[:, rows].cpu().numpy(), grad_out[:, rows].numpy())
+    assert _rel_err(out.detach()[:, rows], t_out) <= 1e-5
+    assert _rel_err(dx[:, rows], t_dx) <= 1e-5
+    assert _rel_err(dg[:, rows], t_dg) <= 1e-5
+
+
+def test_target_shape_fp32_properties():
+    """(8, 1536, 65536) fp32, forward + backward, checked without a full-size oracle:
+    sampled rows against the fp64 recurrence and the adjoint identity
+    <grad_out, scan(g, x)> = <d_tokens, x> (the scan is linear in the tokens)."""
+    shape = (8, 1536, 65536)
+    torch.manual_seed(12312323)
+    gates = 0.999 + 0.001 * torch.rand(*shape, device=DEVICE)
+    tokens = torch.rand(*shape, device=DEVICE)
+    grad_out = torch.randn(*shape, device=DEVICE)
+    gates.requires_grad_(True)
+    tokens.requires_grad_(True)
+    out = scan_warp(gates, tokens)
+    dg, dx = torch.autograd.grad(out, (gates, tokens), grad_out)
+    out = out.detach()
+
+    lhs = (grad_out.double() * out.double()).sum().item()
+    rhs = (dx.double() * tokens.detach().double()).sum().item()
+    assert abs(lhs - rhs) <= 1e-6 * max(abs(lhs), abs(rhs)), (lhs, rhs)
+
+    b, rows = 5, slice(7, 1536, 211)
+    g_np = gates.detach()[b, rows].cpu().numpy()
+    x_np = tokens.detach()[b, rows].cpu().numpy()
+    t_out = seqscan.forward(g_np, x_np)
+    t_dg, t_dx = seqscan.backward(g_np, out[b, rows].cpu().numpy(), grad_out[b, rows].cpu().numpy())
+    errs = {"out": _rel_err(out[b, rows], t_out), "d_tokens": _rel_err(dx[b, rows], t_dx), "d_gates": _rel_err(dg[b, rows], t_dg)}
+    print("target shape rel err vs fp64:", errs)
+    assert max(errs.values()) <= 1e-5
+    # first and last row of the tensor too (grid edges)
+    for bb, rr in ((0, 0), (7, 1535)):
+        t = seqscan.forward(gates.detach()[bb, rr][None].cpu().numpy(), tokens.detach()[bb, rr][None].cpu().numpy())
+        assert _rel_err(out[bb, rr][None], t) <= 1e-5
+
+
+# ---------------------------------------------------------------------------
+# Complex operator: the reference's matrix (tests/tests_eq_complex.py)
+# ---------------------------------------------------------------------------
+def loss_real_mean(out):
+    return out.real.mean()
+
+
+def loss_last_sum(out):
+    return out[:, :, -1].real.sum() + out[:, :, -1].imag.sum()
+
+
+def loss_abs_sq_mean(out):
+    return out.abs().square().mean()
+
+
+complex_seqlens = [2**i for i in range(12, 18)] + [16323, 8000, 33753, 127323]
+
+
+def init_complex(seed, batch_size=1, dim=512, seqlen=32, requires_grad=False, hard_mode=True):
+    torch.manual_seed(seed)
+    angle = 2 * torch.pi * torch.rand(batch_size, dim, seqlen, dtype=torch.float32, device=DEVICE)
+    if hard_mode:
+        radius = 0.99 + 0.01 * torch.rand_like(angle)
+    else:
+        radius = 0.4 + 0.6 * torch.rand_like(angle)
+    forget = torch.polar(radius, angle).to(torch.complex64).requires_grad_(requires_grad)
+    inputs = torch.randn(batch_size, dim, seqlen, requires_grad=requires_grad, device=DEVICE).tanh()
+    if requires_grad:
+        inputs = inputs.detach().requires_grad_(True)
+    return forget, inputs
+
+
+@pytest.mark.parametrize("seed", [1, 11, 22])
+@pytest.mark.parametrize("seqlen", complex_seqlens)
+@pytest.mark.parametrize("hard_mode", [False, True])
+@torch.inference_mode()
+def test_complex_forward(seed, seqlen, hard_mode):
+    from accelerated_scan.complex import scan as scan_complex
+
+    forget, inputs = init_complex(seed, seqlen=seqlen, hard_mode=hard_mode)
+    out = scan_complex(forget, inputs)
+    out_ref = ref_scan.scan(forget, inputs)
+    torch.testing.assert_close(out, out_ref, atol=1e-5, rtol=1e-4)
+
+
+@pytest.mark.parametrize("seed", [1, 11, 22])
+@pytest.mark.parametrize("seqlen", complex_seqlens)
+@pytest.mark.parametrize("hard_mode", [False, True])
+@pytest.mark.parametrize("loss_fn", [loss_real_mean, loss_last_sum, loss_abs_sq_mean])
+def test_complex_backward(seed, seqlen, hard_mode, loss_fn):
+    from accelerated_scan.complex import scan as scan_complex
+
+    forget, inputs = init_complex(seed, seqlen=seqlen, requires_grad=True, hard_mode=hard_mode)
+    loss_fn(scan_complex(forget, inputs)).backward()
+    forget_grad, inputs_grad = forget.grad, inputs.grad
+    assert not torch.is_complex(inputs_grad)
+
+    forget_ref, inputs_ref = init_complex(seed, seqlen=seqlen, requires_grad=True, hard_mode=hard_mode)
+    loss_fn(ref_scan.scan(forget_ref, inputs_ref)).backward()
+    torch.testing.assert_close(forget_grad, forget_ref.grad, atol=1e-5, rtol=1e-4)
+    torch.testing.assert_close(inputs_grad, inputs_ref.grad, atol=1e-5, rtol=1e-4)
+
+
+# ---------------------------------------------------------------------------
+# Boundary behaviour on the device
+# ---------------------------------------------------------------------------
+def test_reverse_scan_forward():
+    from accelerated_scan.warp import scan_forward
+
+    gates, tokens = init(4, dim=37, seqlen=5000)
+    rev = scan_forward(gates, tokens, reverse=True)
+    torch.testing.assert_close(rev, ref_scan.scan(gates, tokens, reverse=True), atol=1e-7, rtol=1.3e-6)
+    flipped = scan_forward(gates.flip(-1).contiguous(), tokens.flip(-1).contiguous()).flip(-1)
+    torch.testing.assert_close(rev, flipped, atol=1e-6, rtol=1e-6)
+
+
+def test_backward_accepts_non_contiguous_grad_and_saves_states():
+    gates, tokens = init(42, dim=33, seqlen=777, requires_grad=True)
+    out = scan_warp(gates, tokens)
+    weight = torch.randn(777, 33, device=DEVICE).t()  # non-contiguous upstream gradient
+    (out * weight).sum().backward()
+    g_ref, x_ref = init(42, dim=33, seqlen=777, requires_grad=True)
+    (ref_scan.scan(g_ref, x_ref) * weight).sum().backward()
+    torch.testing.assert_close(gates.grad, g_ref.grad, atol=1e-5, rtol=1e-5)
+    torch.testing.assert_close(tokens.grad, x_ref.grad, atol=1e-5, rtol=1e-5)
+
+
+def test_device_side_validation():
+    from accelerated_scan import warp
+
+    g = torch.rand(1, 4, 64, device=DEVICE)
+    with pytest.raises(RuntimeError, match="one dtype"):
+        warp.warpscan_forward(g, g.half(), torch.empty_like(g), False)
+    with pytest.raises(RuntimeError, match="unsupported tensor dtype"):
+        warp.scan(g.double(), g.double())
+    with pytest.raises(RuntimeError, match="device tensor"):
+        warp.warpscan_forward(g, g.cpu(), torch.empty_like(g), False)
+    empty = torch.empty(2, 3, 0, device=DEVICE)
+    assert warp.scan(empty, empty).shape == (2, 3, 0)
+    none = torch.empty(0, 3, 8, device=DEVICE)
+    assert warp.scan(none, none).shape == (0, 3, 8)
+
+
+def test_raw_c_abi_on_a_side_stream():
+    """Plain pointers and sizes through ctypes, on a non-default stream."""
+    from accelerated_scan import _abi
+
+    lib = _abi.load()
+    rows, T = 300, 3000
+    gates, tokens, grad_out = _truth_inputs(rows, T, torch.float32, seed=5)
+    g, x, d = (t.to(DEVICE) for t in (gates, tokens, grad_out))
+    out, dg, dx = (torch.empty_like(x) for _ in range(3))
+    stream = torch.cuda.Stream()
+    stream.wait_stream(torch.cuda.current_stream())
+    assert lib.ascan_forward(g.data_ptr(), x.data_ptr(), out.data_ptr(), rows, T, 0, 0, stream.cuda_stream) == 0
+    assert lib.ascan_backward(g.data_ptr(), out.data_ptr(), d.data_ptr(), dg.data_ptr(), dx.data_ptr(), rows, T, 0,
+                              stream.cuda_stream) == 0
+    stream.synchronize()
+    t_out = seqscan.forward(gates.numpy(), tokens.numpy())
+    t_dg, t_dx = seqscan.backward(gates.numpy(), out.cpu().numpy(), grad_out.numpy())
+    np.testing.assert_allclose(out.cpu().numpy(), t_out, rtol=2e-5, atol=2e-5)
+    np.testing.assert_allclose(dx.cpu().numpy(), t_dx, rtol=2e-5, atol=2e-5)
+    np.testing.assert_allclose(dg.cpu().numpy(), t_dg, rtol=2e-5, atol=2e-5 * np.abs(t_dg).max())
+
+
+def test_linearity_and_concatenation():
+    """Size-independent properties: linear in tokens; a scan restarted from the
+    state at a cut equals the uncut scan."""
+    gates, tokens = init(57, dim=40, seqlen=20000)
+    other = torch.randn_like(tokens)
+    a = scan_warp(gates, tokens)
+    b = scan_warp(gates, other)
+    ab = scan_warp(gates, 2.0 * tokens - 3.0 * other)
+    torch.testing.assert_close(ab, 2.0 * a - 3.0 * b, atol=2e-5, rtol=2e-5)
+    cut = 7777
+    tail_tokens = tokens[:, :, cut:].clone()
+    tail_tokens[:, :, 0] += gates[:, :, cut] * a[:, :, cut - 1]
+    tail = scan_warp(gates[:, :, cut:].contiguous(), tail_tokens.contiguous())
+    torch.testing.assert_close(tail, a[:, :, cut:], atol=1e-6, rtol=1e-6)
