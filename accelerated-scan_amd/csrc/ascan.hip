@@ -40,6 +40,31 @@
 #ifndef ASCAN_USE_DPP
 #define ASCAN_USE_DPP 1
 #endif
+// Build-time tuning knobs (defaults are the measured best).
+#ifndef ASCAN_NT_LOAD
+#define ASCAN_NT_LOAD 1
+#endif
+#ifndef ASCAN_NT_STORE
+#define ASCAN_NT_STORE 1
+#endif
+#ifndef ASCAN_U_BWD_F32
+#define ASCAN_U_BWD_F32 ASCAN_U_F32
+#endif
+#ifndef ASCAN_U_F32
+#define ASCAN_U_F32 4
+#endif
+#ifndef ASCAN_U_16BIT
+#define ASCAN_U_16BIT 4
+#endif
+#ifndef ASCAN_U_BWD_16BIT
+#define ASCAN_U_BWD_16BIT 2
+#endif
+#ifndef ASCAN_U_C64
+#define ASCAN_U_C64 4
+#endif
+#ifndef ASCAN_U_BWD_C64
+#define ASCAN_U_BWD_C64 2
+#endif
 
 namespace {
 
@@ -201,6 +226,7 @@ __device__ __forceinline__ cfloat read_lane(cfloat v) {
 // Storage traits: S = element type in memory, V = arithmetic type,
 // EPV = elements per 16-byte vector.
 // ---------------------------------------------------------------------------
+typedef unsigned int u32x4_t __attribute__((ext_vector_type(4)));  // one 16-byte vector
 typedef float floatx2_t __attribute__((ext_vector_type(2)));
 typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
 typedef _Float16 halfx2_t __attribute__((ext_vector_type(2)));
@@ -209,14 +235,14 @@ struct TraitsF32 {
     using S = float;
     using V = float;
     static constexpr int EPV = 4;
-    static __device__ __forceinline__ void unpack(const uint4& r, V (&d)[EPV]) {
+    static __device__ __forceinline__ void unpack(const u32x4_t& r, V (&d)[EPV]) {
         d[0] = i2f(r.x);
         d[1] = i2f(r.y);
         d[2] = i2f(r.z);
         d[3] = i2f(r.w);
     }
-    static __device__ __forceinline__ uint4 pack(const V (&s)[EPV]) {
-        uint4 r;
+    static __device__ __forceinline__ u32x4_t pack(const V (&s)[EPV]) {
+        u32x4_t r;
         r.x = f2i(s[0]);
         r.y = f2i(s[1]);
         r.z = f2i(s[2]);
@@ -238,7 +264,7 @@ struct TraitsBF16 {
         const bf16x2_t h = __builtin_convertvector(f, bf16x2_t);  // round to nearest even
         return __builtin_bit_cast(uint32_t, h);
     }
-    static __device__ __forceinline__ void unpack(const uint4& r, V (&d)[EPV]) {
+    static __device__ __forceinline__ void unpack(const u32x4_t& r, V (&d)[EPV]) {
         const uint32_t w[4] = {r.x, r.y, r.z, r.w};
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
@@ -246,8 +272,8 @@ struct TraitsBF16 {
             d[2 * i + 1] = i2f((int)(w[i] & 0xffff0000u));
         }
     }
-    static __device__ __forceinline__ uint4 pack(const V (&s)[EPV]) {
-        uint4 r;
+    static __device__ __forceinline__ u32x4_t pack(const V (&s)[EPV]) {
+        u32x4_t r;
         r.x = pack2(s[0], s[1]);
         r.y = pack2(s[2], s[3]);
         r.z = pack2(s[4], s[5]);
@@ -269,7 +295,7 @@ struct TraitsF16 {
         const halfx2_t h = __builtin_convertvector(f, halfx2_t);  // round to nearest even
         return __builtin_bit_cast(uint32_t, h);
     }
-    static __device__ __forceinline__ void unpack(const uint4& r, V (&d)[EPV]) {
+    static __device__ __forceinline__ void unpack(const u32x4_t& r, V (&d)[EPV]) {
         const uint32_t w[4] = {r.x, r.y, r.z, r.w};
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
@@ -279,8 +305,8 @@ struct TraitsF16 {
             d[2 * i + 1] = f.y;
         }
     }
-    static __device__ __forceinline__ uint4 pack(const V (&s)[EPV]) {
-        uint4 r;
+    static __device__ __forceinline__ u32x4_t pack(const V (&s)[EPV]) {
+        u32x4_t r;
         r.x = pack2(s[0], s[1]);
         r.y = pack2(s[2], s[3]);
         r.z = pack2(s[4], s[5]);
@@ -299,14 +325,14 @@ struct TraitsC64 {
     using S = cfloat;  // 8 bytes, interleaved (re, im)
     using V = cfloat;
     static constexpr int EPV = 2;
-    static __device__ __forceinline__ void unpack(const uint4& r, V (&d)[EPV]) {
+    static __device__ __forceinline__ void unpack(const u32x4_t& r, V (&d)[EPV]) {
         d[0].re = i2f(r.x);
         d[0].im = i2f(r.y);
         d[1].re = i2f(r.z);
         d[1].im = i2f(r.w);
     }
-    static __device__ __forceinline__ uint4 pack(const V (&s)[EPV]) {
-        uint4 r;
+    static __device__ __forceinline__ u32x4_t pack(const V (&s)[EPV]) {
+        u32x4_t r;
         r.x = f2i(s[0].re);
         r.y = f2i(s[0].im);
         r.z = f2i(s[1].re);
@@ -339,7 +365,11 @@ __device__ __forceinline__ void load_vec(const typename Tr::S* __restrict__ rowp
                                          typename Tr::V fill, typename Tr::V (&dst)[Tr::EPV]) {
     if constexpr (ALIGNED) {
         if (FULL || pos < T) {
-            const uint4 raw = *reinterpret_cast<const uint4*>(rowp + pos);
+#if ASCAN_NT_LOAD
+            const u32x4_t raw = __builtin_nontemporal_load(reinterpret_cast<const u32x4_t*>(rowp + pos));
+#else
+            const u32x4_t raw = *reinterpret_cast<const u32x4_t*>(rowp + pos);
+#endif
             Tr::unpack(raw, dst);
         } else {
 #pragma unroll
@@ -362,7 +392,11 @@ __device__ __forceinline__ void store_vec(typename Tr::S* __restrict__ rowp, int
                                           const typename Tr::V (&src)[Tr::EPV]) {
     if constexpr (ALIGNED) {
         if (FULL || pos < T) {
-            *reinterpret_cast<uint4*>(rowp + pos) = Tr::pack(src);
+#if ASCAN_NT_STORE
+            __builtin_nontemporal_store(Tr::pack(src), reinterpret_cast<u32x4_t*>(rowp + pos));
+#else
+            *reinterpret_cast<u32x4_t*>(rowp + pos) = Tr::pack(src);
+#endif
         }
     } else {
 #pragma unroll
@@ -380,14 +414,36 @@ __device__ __forceinline__ int vec_offset(int j, int lane) {
     return (REV ? (U * 64 - 1 - q) : q) * EPV;
 }
 
+// A workgroup has at most 16 waves: R rows x W waves per row.
+constexpr int kMaxWavesPerBlock = 16;
+constexpr int kSlotsPerBuffer = 2 * kMaxWavesPerBlock;  // one (A, X) pair per wave
+
+// Maps the wave to its row and its position in the row.  Returns false for a
+// wave whose row is past the end: it only keeps the workgroup's barriers
+// company (one per tile) and touches no memory.
+template <int W>
+__device__ __forceinline__ bool locate_wave(int64_t rows, int64_t ntiles, int64_t& row, int& w, int& slot_base) {
+    const int wv = threadIdx.x >> 6;
+    const int rows_per_block = (int)(blockDim.x >> 6) / W;
+    const int rib = wv / W;  // row inside the block
+    w = wv - rib * W;
+    slot_base = 2 * rib * W;
+    row = (int64_t)blockIdx.x * rows_per_block + rib;
+    if (row < rows) return true;
+    if constexpr (W > 1) {
+        for (int64_t k = 0; k < ntiles; ++k) __syncthreads();
+    }
+    return false;
+}
+
 // Carry bookkeeping shared by the forward and the backward kernel.
 //
 // Input : totA/totX[j]   inclusive total of block j of this wave (wave-uniform)
 //         carry          state entering the tile (wave-uniform, same in all waves)
 // Output: c              state entering block 0 of this wave
 //         carry          state entering the next tile
-// With W > 1 the waves of the workgroup exchange their sub-tile totals through
-// `slots` (2 buffers x W entries); `parity` selects the buffer.
+// With W > 1 the W waves of a row exchange their sub-tile totals through
+// `slots`, the row's W entries of one of two buffers selected by `parity`.
 template <class V, int W, int U>
 __device__ __forceinline__ void exchange_carries(const V (&totA)[U], const V (&totX)[U], V& carry, V& c,
                                                  V* slots, int parity, int w, int lane) {
@@ -404,7 +460,7 @@ __device__ __forceinline__ void exchange_carries(const V (&totA)[U], const V (&t
             TX = vfma(TX, totA[j], totX[j]);
             TA = vmul(TA, totA[j]);
         }
-        V* buf = slots + parity * (2 * W);
+        V* buf = slots + parity * kSlotsPerBuffer;
         if (lane == 0) {
             buf[2 * w] = TA;
             buf[2 * w + 1] = TX;
@@ -426,10 +482,12 @@ __device__ __forceinline__ void exchange_carries(const V (&totA)[U], const V (&t
 
 // ---------------------------------------------------------------------------
 // Forward kernel (REV = false) and plain reverse scan (REV = true).
-// W waves share one row (W == 1: four independent rows per 256-thread block).
+// A workgroup holds R rows x W waves per row (R = blockDim.x / 64 / W); the
+// rows of a workgroup are adjacent in memory, so with W*R = 16 one tile step
+// of the workgroup covers one contiguous span of 16 sub-tiles.
 // ---------------------------------------------------------------------------
 template <class Tr, int W, int U, bool REV, bool ALIGNED>
-__global__ void __launch_bounds__(W == 1 ? 256 : 64 * W)
+__global__ void __launch_bounds__(64 * kMaxWavesPerBlock)
     scan_forward_kernel(const typename Tr::S* __restrict__ gates, const typename Tr::S* __restrict__ tokens,
                         typename Tr::S* __restrict__ out, int64_t rows, int64_t T) {
     using S = typename Tr::S;
@@ -439,24 +497,17 @@ __global__ void __launch_bounds__(W == 1 ? 256 : 64 * W)
     constexpr int64_t TILE = SUB * W;
 
     const int lane = threadIdx.x & 63;
-    const int wv = threadIdx.x >> 6;
+    const int64_t ntiles = (T + TILE - 1) / TILE;
+    __shared__ V slots_all[W == 1 ? 1 : 2 * kSlotsPerBuffer];
     int64_t row;
-    int w;
-    if constexpr (W == 1) {
-        row = (int64_t)blockIdx.x * 4 + wv;
-        w = 0;
-        if (row >= rows) return;  // wave-uniform; this configuration has no barrier
-    } else {
-        row = blockIdx.x;
-        w = wv;
-    }
-    __shared__ V slots[W == 1 ? 1 : 4 * W];
+    int w, slot_base;
+    if (!locate_wave<W>(rows, ntiles, row, w, slot_base)) return;  // wave-uniform
+    V* slots = slots_all + (W == 1 ? 0 : slot_base);
 
     const S* __restrict__ grow = gates + row * T;
     const S* __restrict__ trow = tokens + row * T;
     S* __restrict__ orow = out + row * T;
 
-    const int64_t ntiles = (T + TILE - 1) / TILE;
     V carry = vzero<V>();
 
     for (int64_t k = 0; k < ntiles; ++k) {
@@ -529,7 +580,7 @@ __global__ void __launch_bounds__(W == 1 ? 256 : 64 * W)
 // and d_gates[t] = d_tokens[t] * conj(x[t-1]) in the same pass.
 // ---------------------------------------------------------------------------
 template <class Tr, int W, int U, bool ALIGNED>
-__global__ void __launch_bounds__(W == 1 ? 256 : 64 * W)
+__global__ void __launch_bounds__(64 * kMaxWavesPerBlock)
     scan_backward_kernel(const typename Tr::S* __restrict__ gates, const typename Tr::S* __restrict__ states,
                          const typename Tr::S* __restrict__ grad_out, typename Tr::S* __restrict__ d_gates,
                          typename Tr::S* __restrict__ d_tokens, int64_t rows, int64_t T) {
@@ -540,18 +591,12 @@ __global__ void __launch_bounds__(W == 1 ? 256 : 64 * W)
     constexpr int64_t TILE = SUB * W;
 
     const int lane = threadIdx.x & 63;
-    const int wv = threadIdx.x >> 6;
+    const int64_t ntiles = (T + TILE - 1) / TILE;
+    __shared__ V slots_all[W == 1 ? 1 : 2 * kSlotsPerBuffer];
     int64_t row;
-    int w;
-    if constexpr (W == 1) {
-        row = (int64_t)blockIdx.x * 4 + wv;
-        w = 0;
-        if (row >= rows) return;  // wave-uniform; this configuration has no barrier
-    } else {
-        row = blockIdx.x;
-        w = wv;
-    }
-    __shared__ V slots[W == 1 ? 1 : 4 * W];
+    int w, slot_base;
+    if (!locate_wave<W>(rows, ntiles, row, w, slot_base)) return;  // wave-uniform
+    V* slots = slots_all + (W == 1 ? 0 : slot_base);
 
     const S* __restrict__ arow = gates + row * T;
     const S* __restrict__ xrow = states + row * T;
@@ -559,7 +604,6 @@ __global__ void __launch_bounds__(W == 1 ? 256 : 64 * W)
     S* __restrict__ dgrow = d_gates + row * T;
     S* __restrict__ dtrow = d_tokens + row * T;
 
-    const int64_t ntiles = (T + TILE - 1) / TILE;
     V carry = vzero<V>();
 
     for (int64_t k = 0; k < ntiles; ++k) {
@@ -675,42 +719,53 @@ __global__ void __launch_bounds__(W == 1 ? 256 : 64 * W)
 // ---------------------------------------------------------------------------
 thread_local int g_last_hip_error = 0;
 
-// Blocks per sub-tile (U) by dtype: 1024 elements per wave per tile for the
-// real dtypes, 512 for complex64.
+// Blocks per sub-tile by dtype, forward (U) and backward (UB).  Forward
+// sub-tiles are 4 KiB of each tensor; the backward kernel holds three input
+// tensors in registers and takes half of that where 4 KiB would spill.
 template <class Tr> struct Tuning;
-template <> struct Tuning<TraitsF32> { static constexpr int U = 4; };
-template <> struct Tuning<TraitsBF16> { static constexpr int U = 2; };
-template <> struct Tuning<TraitsF16> { static constexpr int U = 2; };
-template <> struct Tuning<TraitsC64> { static constexpr int U = 4; };
+template <> struct Tuning<TraitsF32> { static constexpr int U = ASCAN_U_F32, UB = ASCAN_U_BWD_F32; };
+template <> struct Tuning<TraitsBF16> { static constexpr int U = ASCAN_U_16BIT, UB = ASCAN_U_BWD_16BIT; };
+template <> struct Tuning<TraitsF16> { static constexpr int U = ASCAN_U_16BIT, UB = ASCAN_U_BWD_16BIT; };
+template <> struct Tuning<TraitsC64> { static constexpr int U = ASCAN_U_C64, UB = ASCAN_U_BWD_C64; };
 
-// Optional override of the waves-per-row choice (1, 4 or 16), read once.
-int forced_waves_per_row() {
-    static const int v = [] {
-        const char* s = getenv("ASCAN_WAVES_PER_ROW");
-        const int n = s ? atoi(s) : 0;
-        return (n == 1 || n == 4 || n == 16) ? n : 0;
-    }();
-    return v;
+// Launch geometry: W waves per row, R rows per workgroup (W*R <= 16).
+struct Plan {
+    int waves_per_row;
+    int rows_per_block;
+};
+
+int env_int(const char* name) {
+    const char* s = getenv(name);
+    return s ? atoi(s) : 0;
 }
 
-// How many waves cooperate on one row.  One wave per row is the cheapest
-// arrangement (no LDS, no barrier) and is used whenever the rows alone give
-// the machine enough waves; few long rows are split over 4 or 16 waves.
-int choose_waves_per_row(int64_t rows, int64_t T, int64_t sub) {
-    const int forced = forced_waves_per_row();
-    int w;
-    if (forced) {
-        w = forced;
-    } else if (rows >= 2048) {
-        w = 1;
-    } else if (rows >= 512) {
-        w = 4;
-    } else {
-        w = 16;
-    }
-    // No point in more waves than sub-tiles in the row.
-    while (w > 1 && (int64_t)(w / 4) * sub >= T) w /= 4;
-    return w;
+// Optional overrides for tuning runs, read once per process:
+// ASCAN_WAVES_PER_ROW in {1,2,4,8,16}, ASCAN_ROWS_PER_BLOCK in {1,2,4,8,16}.
+const Plan& forced_plan() {
+    static const Plan p = [] {
+        auto pow2 = [](int n) { return (n == 1 || n == 2 || n == 4 || n == 8 || n == 16) ? n : 0; };
+        return Plan{pow2(env_int("ASCAN_WAVES_PER_ROW")), pow2(env_int("ASCAN_ROWS_PER_BLOCK"))};
+    }();
+    return p;
+}
+
+// Measured on MI355X: what counts is how few rows are being streamed at any
+// one time.  With every wave on its own row the memory system sees thousands
+// of concurrent streams and tops out near 5.0 TB/s; with 16 waves marching
+// along one row it reaches the 5.7-6.1 TB/s of a plain linear sweep.  So a row
+// gets as many waves as it has sub-tiles (up to 16).  Short rows keep small
+// workgroups (256 threads, several rows each): packing more short rows into
+// one large workgroup measured slower.
+Plan choose_plan(int64_t T, int64_t sub, int64_t element_bytes) {
+    const Plan& forced = forced_plan();
+    // one wave per 4 KiB of row, but never more waves than sub-tiles
+    int w = 1;
+    while (w < kMaxWavesPerBlock && (int64_t)w * 4096 < T * element_bytes && (int64_t)w * sub < T) w *= 2;
+    if (forced.waves_per_row) w = forced.waves_per_row;
+    int r = w >= 4 ? 1 : 4 / w;
+    if (forced.rows_per_block) r = forced.rows_per_block;
+    if (w * r > kMaxWavesPerBlock) r = kMaxWavesPerBlock / w;
+    return Plan{w, r};
 }
 
 bool is_aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
@@ -725,12 +780,12 @@ int finish_launch() {
 }
 
 template <class Tr, int W, bool REV, bool ALIGNED>
-void launch_forward(const void* gates, const void* tokens, void* out, int64_t rows, int64_t T,
+void launch_forward(const void* gates, const void* tokens, void* out, int64_t rows, int64_t T, int rows_per_block,
                     hipStream_t stream) {
     using S = typename Tr::S;
     constexpr int U = Tuning<Tr>::U;
-    const unsigned blocks = (unsigned)(W == 1 ? (rows + 3) / 4 : rows);
-    const unsigned threads = W == 1 ? 256 : 64 * W;
+    const unsigned blocks = (unsigned)((rows + rows_per_block - 1) / rows_per_block);
+    const unsigned threads = 64u * W * rows_per_block;
     hipLaunchKernelGGL((scan_forward_kernel<Tr, W, U, REV, ALIGNED>), dim3(blocks), dim3(threads), 0, stream,
                        static_cast<const S*>(gates), static_cast<const S*>(tokens), static_cast<S*>(out), rows,
                        T);
@@ -738,11 +793,11 @@ void launch_forward(const void* gates, const void* tokens, void* out, int64_t ro
 
 template <class Tr, int W, bool ALIGNED>
 void launch_backward(const void* gates, const void* states, const void* grad_out, void* d_gates,
-                     void* d_tokens, int64_t rows, int64_t T, hipStream_t stream) {
+                     void* d_tokens, int64_t rows, int64_t T, int rows_per_block, hipStream_t stream) {
     using S = typename Tr::S;
-    constexpr int U = Tuning<Tr>::U;
-    const unsigned blocks = (unsigned)(W == 1 ? (rows + 3) / 4 : rows);
-    const unsigned threads = W == 1 ? 256 : 64 * W;
+    constexpr int U = Tuning<Tr>::UB;
+    const unsigned blocks = (unsigned)((rows + rows_per_block - 1) / rows_per_block);
+    const unsigned threads = 64u * W * rows_per_block;
     hipLaunchKernelGGL((scan_backward_kernel<Tr, W, U, ALIGNED>), dim3(blocks), dim3(threads), 0, stream,
                        static_cast<const S*>(gates), static_cast<const S*>(states),
                        static_cast<const S*>(grad_out), static_cast<S*>(d_gates), static_cast<S*>(d_tokens),
@@ -755,22 +810,25 @@ int forward_typed(const void* gates, const void* tokens, void* out, int64_t rows
     constexpr int EPV = Tr::EPV;
     constexpr int64_t SUB = (int64_t)Tuning<Tr>::U * 64 * EPV;
     const bool aligned = is_aligned16(gates) && is_aligned16(tokens) && is_aligned16(out) && (T % EPV == 0);
-    const int W = aligned ? choose_waves_per_row(rows, T, SUB) : 1;
-#define ASCAN_FWD(WV, AL)                                                              \
-    do {                                                                               \
-        if (reverse)                                                                   \
-            launch_forward<Tr, WV, true, AL>(gates, tokens, out, rows, T, stream);     \
-        else                                                                           \
-            launch_forward<Tr, WV, false, AL>(gates, tokens, out, rows, T, stream);    \
+    const Plan plan = choose_plan(T, SUB, (int64_t)sizeof(typename Tr::S));
+    const int R = plan.rows_per_block;
+#define ASCAN_FWD(WV, AL, RPB)                                                              \
+    do {                                                                                    \
+        if (reverse)                                                                        \
+            launch_forward<Tr, WV, true, AL>(gates, tokens, out, rows, T, RPB, stream);     \
+        else                                                                                \
+            launch_forward<Tr, WV, false, AL>(gates, tokens, out, rows, T, RPB, stream);    \
     } while (0)
     if (!aligned) {
-        ASCAN_FWD(1, false);
-    } else if (W == 1) {
-        ASCAN_FWD(1, true);
-    } else if (W == 4) {
-        ASCAN_FWD(4, true);
+        ASCAN_FWD(1, false, 4);  // element-wise kernel: one wave per row
     } else {
-        ASCAN_FWD(16, true);
+        switch (plan.waves_per_row) {
+            case 1: ASCAN_FWD(1, true, R); break;
+            case 2: ASCAN_FWD(2, true, R); break;
+            case 4: ASCAN_FWD(4, true, R); break;
+            case 8: ASCAN_FWD(8, true, R); break;
+            default: ASCAN_FWD(16, true, R); break;
+        }
     }
 #undef ASCAN_FWD
     return finish_launch();
@@ -780,19 +838,25 @@ template <class Tr>
 int backward_typed(const void* gates, const void* states, const void* grad_out, void* d_gates, void* d_tokens,
                    int64_t rows, int64_t T, hipStream_t stream) {
     constexpr int EPV = Tr::EPV;
-    constexpr int64_t SUB = (int64_t)Tuning<Tr>::U * 64 * EPV;
+    constexpr int64_t SUB = (int64_t)Tuning<Tr>::UB * 64 * EPV;
     const bool aligned = is_aligned16(gates) && is_aligned16(states) && is_aligned16(grad_out) &&
                          is_aligned16(d_gates) && is_aligned16(d_tokens) && (T % EPV == 0);
-    const int W = aligned ? choose_waves_per_row(rows, T, SUB) : 1;
+    const Plan plan = choose_plan(T, SUB, (int64_t)sizeof(typename Tr::S));
+    const int R = plan.rows_per_block;
+#define ASCAN_BWD(WV, AL, RPB) \
+    launch_backward<Tr, WV, AL>(gates, states, grad_out, d_gates, d_tokens, rows, T, RPB, stream)
     if (!aligned) {
-        launch_backward<Tr, 1, false>(gates, states, grad_out, d_gates, d_tokens, rows, T, stream);
-    } else if (W == 1) {
-        launch_backward<Tr, 1, true>(gates, states, grad_out, d_gates, d_tokens, rows, T, stream);
-    } else if (W == 4) {
-        launch_backward<Tr, 4, true>(gates, states, grad_out, d_gates, d_tokens, rows, T, stream);
+        ASCAN_BWD(1, false, 4);  // element-wise kernel: one wave per row
     } else {
-        launch_backward<Tr, 16, true>(gates, states, grad_out, d_gates, d_tokens, rows, T, stream);
+        switch (plan.waves_per_row) {
+            case 1: ASCAN_BWD(1, true, R); break;
+            case 2: ASCAN_BWD(2, true, R); break;
+            case 4: ASCAN_BWD(4, true, R); break;
+            case 8: ASCAN_BWD(8, true, R); break;
+            default: ASCAN_BWD(16, true, R); break;
+        }
     }
+#undef ASCAN_BWD
     return finish_launch();
 }
 

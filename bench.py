@@ -1,0 +1,248 @@
+"""Benchmark of the scan hot path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W]
+
+One step = one forward scan plus one fused backward scan over the same
+synthetic batch, both through the C ABI with every buffer already resident in
+HBM.  The default workload is the headline configuration: fp32, shape
+(8, 1536, 65536), inputs drawn as the reference's benchmark draws them
+(tests/bench.py:6-11 of the reference: seed 12312323, gates
+0.999 + 0.001 U rounded through fp16, tokens U(0,1)), upstream gradient N(0,1).
+
+Prints ONE JSON line.  `value` is algorithmic bytes per second for the whole
+step (forward 3 tensors + backward 5 tensors = 8*B*D*T*sizeof(dtype) bytes).
+`roofline` describes the dominant kernel (the backward scan) from HIP-event
+timings taken inside the timed region; `cpu_baseline` times the torch tree
+scan (oracle/ref_scan.py, the restatement of the reference's ref.scan) on the
+host cores on a bounded sample of the same workload.
+
+Other workloads: --dtype {fp32,bf16,fp16,c64} --shape B D T; --sweep runs the
+(8, 1536, T) sweep, T = 4096..65536, fp32 and bf16, and writes one JSON line
+per point to the file given (the single summary line is still printed).
+"""
+
+import argparse
+import json
+import os
+import sys
+import time
+from pathlib import Path
+
+ROOT = Path(__file__).resolve().parent
+for _p in (ROOT, ROOT / "accelerated-scan_amd"):
+    if str(_p) not in sys.path:
+        sys.path.insert(0, str(_p))
+
+HBM_PEAK_GBPS = 8000.0  # MI355X HBM3E, published peak
+
+# HBM bytes per launch of the backward kernel, from two rocprofv3 --pmc runs
+# (FETCH_SIZE x 2.000 + WRITE_SIZE x 1.000 KiB, factors from a plain copy of
+# known size; summary in profiles/scan_f32_8x1536x65536_fwd_bwd.md).
+MEASURED_TRAFFIC_BYTES = {
+    ((8, 1536, 65536), "fp32"): (4756376 * 2 + 6315309) * 1024,
+}
+
+
+def parse_args():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--dtype", choices=["fp32", "bf16", "fp16", "c64"], default="fp32")
+    ap.add_argument("--shape", type=int, nargs=3, default=[8, 1536, 65536], metavar=("B", "D", "T"))
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--pmc-calibration", action="store_true",
+                    help="for rocprofv3 --pmc runs: 3 plain copies of 1 GiB (torch copy_), then 3 steps "
+                         "of the workload, no timing; the copy's known traffic scales the counters")
+    ap.add_argument("--sweep", type=str, default=None, metavar="FILE",
+                    help="also run the (8,1536,T) fp32/bf16 sweep and write JSON lines to FILE")
+    return ap.parse_args()
+
+
+def make_inputs(shape, dtype_name, device):
+    import torch
+
+    torch.manual_seed(12312323)
+    if dtype_name == "c64":
+        angle = 2 * torch.pi * torch.rand(*shape, device=device)
+        radius = 0.9 + 0.1 * torch.rand(*shape, device=device)
+        gates = torch.polar(radius, angle)
+        tokens = torch.complex(torch.randn(*shape, device=device), torch.randn(*shape, device=device))
+        grad_out = torch.complex(torch.randn(*shape, device=device), torch.randn(*shape, device=device))
+        return gates, tokens, grad_out
+    dt = {"fp32": torch.float32, "bf16": torch.bfloat16, "fp16": torch.float16}[dtype_name]
+    gates = (0.999 + 0.001 * torch.rand(*shape, device=device)).half().float()
+    tokens = torch.rand(*shape, device=device)
+    grad_out = torch.randn(*shape, device=device)
+    return gates.to(dt), tokens.to(dt), grad_out.to(dt)
+
+
+def run_workload(shape, dtype_name, steps, warmup):
+    """Times `steps` forward+backward passes; returns a dict of measurements."""
+    import torch
+
+    from accelerated_scan import _abi
+
+    device = torch.device("cuda:0")
+    gates, tokens, grad_out = make_inputs(shape, dtype_name, device)
+    states = torch.empty_like(tokens)
+    d_gates = torch.empty_like(tokens)
+    d_tokens = torch.empty_like(tokens)
+    elems = tokens.numel()
+    esize = tokens.element_size()
+
+    def step(events=None):
+        if events is not None:
+            events[0].record()
+        _abi.forward(gates, tokens, states, False)
+        if events is not None:
+            events[1].record()
+        _abi.backward(gates, states, grad_out, d_gates, d_tokens)
+        if events is not None:
+            events[2].record()
+
+    for _ in range(warmup):
+        step()
+    evs = [[torch.cuda.Event(enable_timing=True) for _ in range(3)] for _ in range(steps)]
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for i in range(steps):
+        step(evs[i])
+    torch.cuda.synchronize()
+    t1 = time.perf_counter()
+
+    fwd_ms = sum(e[0].elapsed_time(e[1]) for e in evs) / steps
+    bwd_ms = sum(e[1].elapsed_time(e[2]) for e in evs) / steps
+    ms_per_step = (t1 - t0) * 1e3 / steps
+    return {
+        "elems": elems,
+        "esize": esize,
+        "ms_per_step": ms_per_step,
+        "fwd_ms": fwd_ms,
+        "bwd_ms": bwd_ms,
+        "gbps": 8 * elems * esize / (ms_per_step * 1e-3) / 1e9,
+        "fwd_gbps": 3 * elems * esize / (fwd_ms * 1e-3) / 1e9,
+        "bwd_gbps": 5 * elems * esize / (bwd_ms * 1e-3) / 1e9,
+    }
+
+
+def cpu_baseline(shape, dtype_name):
+    """Tree scan (the reference's CPU path, restated) forward+backward on the
+    host cores, on a slice of the workload's rows sized to take ~10-30 s."""
+    import torch
+
+    from oracle import ref_scan
+
+    B, D, T = shape
+    rows = max(1, min(B * D, (1 << 27) // T))  # about 134M elements per repetition
+    sample = (1, rows, T)
+    gates, tokens, grad_out = make_inputs(sample, dtype_name, torch.device("cpu"))
+    if dtype_name in ("bf16", "fp16"):
+        gates, tokens, grad_out = gates.float(), tokens.float(), grad_out.float()
+
+    def once():
+        g = gates.clone().requires_grad_(True)
+        x = tokens.clone().requires_grad_(True)
+        t0 = time.perf_counter()
+        out = ref_scan.scan(g, x)
+        torch.autograd.grad(out, (g, x), grad_out)
+        return time.perf_counter() - t0
+
+    once()  # warm-up
+    times = sorted(once() for _ in range(3))
+    median = times[1]
+    esize = 8 if dtype_name == "c64" else 4
+    return {
+        "value": 8 * rows * T * esize / median / 1e9,
+        "unit": "GB/s",
+        "cores": torch.get_num_threads(),
+        "kind": "port",
+        "sample": f"torch tree scan fwd+bwd (autograd), fp32 arithmetic, shape {sample} "
+                  f"= {rows} of {B * D} rows, median of 3: {median * 1e3:.1f} ms; "
+                  f"host has {os.cpu_count()} logical cpus",
+    }
+
+
+def main():
+    args = parse_args()
+    if args.gpus != 1:
+        print(f"bench.py: this build runs on ONE GPU (rows shard without communication); "
+              f"--gpus {args.gpus} is not supported", file=sys.stderr)
+        return 2
+    import torch
+
+    if not torch.cuda.is_available():
+        print("bench.py: no HIP device visible", file=sys.stderr)
+        return 2
+    from accelerated_scan import _abi
+
+    _abi.load()  # no fallback: fail here if the HIP library is missing
+
+    shape = tuple(args.shape)
+    if args.pmc_calibration:
+        src = torch.rand(1 << 28, device="cuda:0")  # 1 GiB of fp32
+        dst = torch.empty_like(src)
+        for _ in range(3):
+            dst.copy_(src)
+        torch.cuda.synchronize()
+        run_workload(shape, args.dtype, 3, 0)
+        print(json.dumps({"calibration_copy_bytes_read": src.numel() * 4, "calibration_copy_bytes_written":
+                          src.numel() * 4, "workload_shape": list(shape), "dtype": args.dtype}))
+        return 0
+    m = run_workload(shape, args.dtype, args.steps, args.warmup)
+
+    if args.sweep:
+        with open(args.sweep, "w") as f:
+            for dt in ("fp32", "bf16"):
+                for T in (4096, 8192, 16384, 32768, 65536):
+                    r = run_workload((8, 1536, T), dt, max(5, args.steps), args.warmup)
+                    r.update({"dtype": dt, "shape": [8, 1536, T]})
+                    f.write(json.dumps(r) + "\n")
+                    f.flush()
+
+    dtype_field = {"fp32": "f32", "bf16": "bf16 storage, f32 arithmetic",
+                   "fp16": "f16 storage, f32 arithmetic", "c64": "complex64 (f32 pairs)"}[args.dtype]
+    bwd_bytes = 5 * m["elems"] * m["esize"]
+    result = {
+        "metric": "fwd+bwd achieved HBM GB/s (algorithmic bytes: 3 tensors forward + 5 backward) "
+                  f"at {shape} {args.dtype}",
+        "value": m["gbps"],
+        "unit": "GB/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": m["ms_per_step"],
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": dtype_field,
+        "data": "synthetic",
+        "config": {
+            "workload": f"scan forward + fused backward, shape {list(shape)}, {args.dtype}, "
+                        "gates 0.999+0.001*U(0,1), tokens U(0,1), grad_out N(0,1)",
+            "fwd_ms": m["fwd_ms"],
+            "bwd_ms": m["bwd_ms"],
+            "fwd_GBps": m["fwd_gbps"],
+            "bwd_GBps": m["bwd_gbps"],
+            "frac_of_hbm_peak": m["gbps"] / HBM_PEAK_GBPS,
+        },
+        "roofline": {
+            "kernel": "scan_backward_kernel",
+            "bound": "hbm",
+            "achieved": m["bwd_gbps"],
+            "peak": HBM_PEAK_GBPS,
+            "unit": "GB/s",
+            "frac": m["bwd_gbps"] / HBM_PEAK_GBPS,
+            "algorithmic_bytes_per_launch": bwd_bytes,
+            "avg_launch_ms": m["bwd_ms"],
+            "traffic": MEASURED_TRAFFIC_BYTES.get((shape, args.dtype)),
+        },
+    }
+    if not args.no_cpu_baseline:
+        result["cpu_baseline"] = cpu_baseline(shape, args.dtype)
+    print(json.dumps(result))
+    return 0
+
+
+if __name__ == "__main__":
+    sys.exit(main())
