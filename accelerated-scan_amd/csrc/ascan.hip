@@ -151,6 +151,9 @@ __device__ __forceinline__ void scan_step(V& A, V& X) {
 // Inclusive scan of the 64 (A, X) pairs of a wave, ascending lane order.
 template <class V>
 __device__ __forceinline__ void wave_scan_inclusive(V& A, V& X) {
+#ifdef ASCAN_EXPERIMENT_NOSCAN
+    return;
+#endif
     scan_step<kRowShr1, 0xF>(A, X);
     scan_step<kRowShr2, 0xF>(A, X);
     scan_step<kRowShr4, 0xF>(A, X);
@@ -355,55 +358,98 @@ struct TraitsC64 {
 };
 
 // ---------------------------------------------------------------------------
-// Vector access.  `pos` is the element index inside the row of the first
-// element of the vector.  FULL: the whole vector is known to lie inside the
-// row.  ALIGNED: rowp + pos is 16-byte aligned and T is a multiple of EPV, so
-// a vector is either entirely inside the row or entirely outside.
+// Vector access.  A row is addressed in "virtual" positions: position 0 is the
+// 16-byte boundary at or just below the row's first element, the row's
+// elements occupy [lo, hi) with 0 <= lo < EPV, and `rowp` points at virtual
+// position 0.  `pos` is the virtual position of the first element of a vector.
+//   ALIGNED: rowp + pos is 16-byte aligned (pos is a multiple of EPV), so
+//            vectors move as one dwordx4.  A vector that straddles a row end
+//            (at most two per row) is read whole and masked, and stored
+//            element by element so a neighbouring row's bytes are never
+//            written.  The !ALIGNED kernels move everything element by element.
+//   FULL   : the whole vector is known to lie inside the row.
 // ---------------------------------------------------------------------------
-template <class Tr, bool ALIGNED, bool FULL>
-__device__ __forceinline__ void load_vec(const typename Tr::S* __restrict__ rowp, int64_t pos, int64_t T,
-                                         typename Tr::V fill, typename Tr::V (&dst)[Tr::EPV]) {
-    if constexpr (ALIGNED) {
-        if (FULL || pos < T) {
-#if ASCAN_NT_LOAD
-            const u32x4_t raw = __builtin_nontemporal_load(reinterpret_cast<const u32x4_t*>(rowp + pos));
-#else
-            const u32x4_t raw = *reinterpret_cast<const u32x4_t*>(rowp + pos);
-#endif
-            Tr::unpack(raw, dst);
+template <class Tr, bool FULL>
+__device__ __forceinline__ void load_elements(const typename Tr::S* __restrict__ rowp, int64_t pos, int64_t lo,
+                                              int64_t hi, typename Tr::V fill, typename Tr::V (&dst)[Tr::EPV]) {
+#pragma unroll
+    for (int e = 0; e < Tr::EPV; ++e) {
+        if (FULL || (pos + e >= lo && pos + e < hi)) {
+            dst[e] = Tr::load1(rowp + pos + e);
         } else {
-#pragma unroll
-            for (int e = 0; e < Tr::EPV; ++e) dst[e] = fill;
-        }
-    } else {
-#pragma unroll
-        for (int e = 0; e < Tr::EPV; ++e) {
-            if (FULL || pos + e < T) {
-                dst[e] = Tr::load1(rowp + pos + e);
-            } else {
-                dst[e] = fill;
-            }
+            dst[e] = fill;
         }
     }
 }
 
 template <class Tr, bool ALIGNED, bool FULL>
-__device__ __forceinline__ void store_vec(typename Tr::S* __restrict__ rowp, int64_t pos, int64_t T,
+__device__ __forceinline__ void load_vec(const typename Tr::S* __restrict__ rowp, int64_t pos, int64_t lo,
+                                         int64_t hi, typename Tr::V fill, typename Tr::V (&dst)[Tr::EPV]) {
+    if constexpr (ALIGNED) {
+        // A vector that straddles a row end is still read whole: an aligned
+        // 16-byte read that overlaps the row cannot leave the row's memory
+        // page, and the bytes of the neighbouring row are discarded below.  A
+        // vector entirely outside the row re-reads the row's first vector
+        // instead, so the load stays unconditional.
+        int64_t p = pos;
+        if (!FULL && !(pos + Tr::EPV > lo && pos < hi)) p = 0;
+#if ASCAN_NT_LOAD
+        const u32x4_t raw = __builtin_nontemporal_load(reinterpret_cast<const u32x4_t*>(rowp + p));
+#else
+        const u32x4_t raw = *reinterpret_cast<const u32x4_t*>(rowp + p);
+#endif
+        Tr::unpack(raw, dst);
+        if (!FULL) {
+#pragma unroll
+            for (int e = 0; e < Tr::EPV; ++e) {
+                dst[e] = vselect(pos + e >= lo && pos + e < hi, dst[e], fill);
+            }
+        }
+    } else {
+        load_elements<Tr, FULL>(rowp, pos, lo, hi, fill, dst);
+    }
+}
+
+template <class Tr, bool FULL>
+__device__ __forceinline__ void store_elements(typename Tr::S* __restrict__ rowp, int64_t pos, int64_t lo,
+                                               int64_t hi, const typename Tr::V (&src)[Tr::EPV]) {
+#pragma unroll
+    for (int e = 0; e < Tr::EPV; ++e) {
+        if (FULL || (pos + e >= lo && pos + e < hi)) Tr::store1(rowp + pos + e, src[e]);
+    }
+}
+
+template <class Tr, bool ALIGNED, bool FULL>
+__device__ __forceinline__ void store_vec(typename Tr::S* __restrict__ rowp, int64_t pos, int64_t lo, int64_t hi,
                                           const typename Tr::V (&src)[Tr::EPV]) {
     if constexpr (ALIGNED) {
-        if (FULL || pos < T) {
+        if (FULL || (pos >= lo && pos + Tr::EPV <= hi)) {
 #if ASCAN_NT_STORE
             __builtin_nontemporal_store(Tr::pack(src), reinterpret_cast<u32x4_t*>(rowp + pos));
 #else
             *reinterpret_cast<u32x4_t*>(rowp + pos) = Tr::pack(src);
 #endif
+        } else {
+            store_elements<Tr, false>(rowp, pos, lo, hi, src);
         }
     } else {
-#pragma unroll
-        for (int e = 0; e < Tr::EPV; ++e) {
-            if (FULL || pos + e < T) Tr::store1(rowp + pos + e, src[e]);
-        }
+        store_elements<Tr, FULL>(rowp, pos, lo, hi, src);
     }
+}
+
+// Number of tiles every wave of the grid iterates over (the barrier count must
+// be the same for all waves of a workgroup).  `head` is the largest misalignment
+// of a row start, in elements, over all rows.
+__device__ __forceinline__ int64_t tiles_per_row(int64_t T, int64_t tile, int head) {
+    return (T + head + tile - 1) / tile;
+}
+
+// Misalignment of the row start in elements (0 <= result < EPV).  All tensors
+// of a call share it: the host checks that their base addresses are congruent
+// modulo 16.
+template <class Tr>
+__device__ __forceinline__ int row_lead(const typename Tr::S* row_start) {
+    return (int)((reinterpret_cast<uintptr_t>(row_start) / sizeof(typename Tr::S)) % Tr::EPV);
 }
 
 // Element index (inside the sub-tile) of the vector that lane `lane` owns in
@@ -497,38 +543,42 @@ __global__ void __launch_bounds__(64 * kMaxWavesPerBlock)
     constexpr int64_t TILE = SUB * W;
 
     const int lane = threadIdx.x & 63;
-    const int64_t ntiles = (T + TILE - 1) / TILE;
+    // rows start at the same misalignment when T is a multiple of the vector width
+    const int head = ALIGNED ? (T % EPV == 0 ? row_lead<Tr>(gates) : EPV - 1) : 0;
+    const int64_t ntiles = tiles_per_row(T, TILE, head);
     __shared__ V slots_all[W == 1 ? 1 : 2 * kSlotsPerBuffer];
     int64_t row;
     int w, slot_base;
     if (!locate_wave<W>(rows, ntiles, row, w, slot_base)) return;  // wave-uniform
     V* slots = slots_all + (W == 1 ? 0 : slot_base);
 
-    const S* __restrict__ grow = gates + row * T;
-    const S* __restrict__ trow = tokens + row * T;
-    S* __restrict__ orow = out + row * T;
+    const int64_t lo = ALIGNED ? row_lead<Tr>(gates + row * T) : 0;
+    const int64_t hi = lo + T;
+    const S* __restrict__ grow = gates + row * T - lo;
+    const S* __restrict__ trow = tokens + row * T - lo;
+    S* __restrict__ orow = out + row * T - lo;
 
     V carry = vzero<V>();
 
     for (int64_t k = 0; k < ntiles; ++k) {
         const int64_t tile = REV ? (ntiles - 1 - k) : k;
         const int64_t sub_base = tile * TILE + (int64_t)(REV ? (W - 1 - w) : w) * SUB;
-        const bool full = sub_base + SUB <= T;  // wave-uniform
+        const bool full = sub_base >= lo && sub_base + SUB <= hi;  // wave-uniform
 
         V g[U][EPV], t[U][EPV];
         if (full) {
 #pragma unroll
             for (int j = 0; j < U; ++j) {
                 const int64_t pos = sub_base + vec_offset<U, EPV, REV>(j, lane);
-                load_vec<Tr, ALIGNED, true>(grow, pos, T, vone<V>(), g[j]);
-                load_vec<Tr, ALIGNED, true>(trow, pos, T, vzero<V>(), t[j]);
+                load_vec<Tr, ALIGNED, true>(grow, pos, lo, hi, vone<V>(), g[j]);
+                load_vec<Tr, ALIGNED, true>(trow, pos, lo, hi, vzero<V>(), t[j]);
             }
         } else {
 #pragma unroll
             for (int j = 0; j < U; ++j) {
                 const int64_t pos = sub_base + vec_offset<U, EPV, REV>(j, lane);
-                load_vec<Tr, ALIGNED, false>(grow, pos, T, vone<V>(), g[j]);
-                load_vec<Tr, ALIGNED, false>(trow, pos, T, vzero<V>(), t[j]);
+                load_vec<Tr, ALIGNED, false>(grow, pos, lo, hi, vone<V>(), g[j]);
+                load_vec<Tr, ALIGNED, false>(trow, pos, lo, hi, vzero<V>(), t[j]);
             }
         }
 
@@ -567,9 +617,9 @@ __global__ void __launch_bounds__(64 * kMaxWavesPerBlock)
             }
             const int64_t pos = sub_base + vec_offset<U, EPV, REV>(j, lane);
             if (full) {
-                store_vec<Tr, ALIGNED, true>(orow, pos, T, o);
+                store_vec<Tr, ALIGNED, true>(orow, pos, lo, hi, o);
             } else {
-                store_vec<Tr, ALIGNED, false>(orow, pos, T, o);
+                store_vec<Tr, ALIGNED, false>(orow, pos, lo, hi, o);
             }
         }
     }
@@ -591,18 +641,22 @@ __global__ void __launch_bounds__(64 * kMaxWavesPerBlock)
     constexpr int64_t TILE = SUB * W;
 
     const int lane = threadIdx.x & 63;
-    const int64_t ntiles = (T + TILE - 1) / TILE;
+    // rows start at the same misalignment when T is a multiple of the vector width
+    const int head = ALIGNED ? (T % EPV == 0 ? row_lead<Tr>(gates) : EPV - 1) : 0;
+    const int64_t ntiles = tiles_per_row(T, TILE, head);
     __shared__ V slots_all[W == 1 ? 1 : 2 * kSlotsPerBuffer];
     int64_t row;
     int w, slot_base;
     if (!locate_wave<W>(rows, ntiles, row, w, slot_base)) return;  // wave-uniform
     V* slots = slots_all + (W == 1 ? 0 : slot_base);
 
-    const S* __restrict__ arow = gates + row * T;
-    const S* __restrict__ xrow = states + row * T;
-    const S* __restrict__ drow = grad_out + row * T;
-    S* __restrict__ dgrow = d_gates + row * T;
-    S* __restrict__ dtrow = d_tokens + row * T;
+    const int64_t lo = ALIGNED ? row_lead<Tr>(gates + row * T) : 0;
+    const int64_t hi = lo + T;
+    const S* __restrict__ arow = gates + row * T - lo;
+    const S* __restrict__ xrow = states + row * T - lo;
+    const S* __restrict__ drow = grad_out + row * T - lo;
+    S* __restrict__ dgrow = d_gates + row * T - lo;
+    S* __restrict__ dtrow = d_tokens + row * T - lo;
 
     V carry = vzero<V>();
 
@@ -610,39 +664,39 @@ __global__ void __launch_bounds__(64 * kMaxWavesPerBlock)
         const int64_t tile = ntiles - 1 - k;
         const int64_t sub_base = tile * TILE + (int64_t)(W - 1 - w) * SUB;
         const int64_t sub_end = sub_base + SUB;
-        const bool full = sub_end <= T;  // wave-uniform
+        const bool full = sub_base >= lo && sub_end <= hi;  // wave-uniform
 
         V a[U][EPV], d[U][EPV], x[U][EPV];
         if (full) {
 #pragma unroll
             for (int j = 0; j < U; ++j) {
                 const int64_t pos = sub_base + vec_offset<U, EPV, true>(j, lane);
-                load_vec<Tr, ALIGNED, true>(arow, pos, T, vone<V>(), a[j]);
-                load_vec<Tr, ALIGNED, true>(drow, pos, T, vzero<V>(), d[j]);
-                load_vec<Tr, ALIGNED, true>(xrow, pos, T, vzero<V>(), x[j]);
+                load_vec<Tr, ALIGNED, true>(arow, pos, lo, hi, vone<V>(), a[j]);
+                load_vec<Tr, ALIGNED, true>(drow, pos, lo, hi, vzero<V>(), d[j]);
+                load_vec<Tr, ALIGNED, true>(xrow, pos, lo, hi, vzero<V>(), x[j]);
             }
         } else {
 #pragma unroll
             for (int j = 0; j < U; ++j) {
                 const int64_t pos = sub_base + vec_offset<U, EPV, true>(j, lane);
-                load_vec<Tr, ALIGNED, false>(arow, pos, T, vone<V>(), a[j]);
-                load_vec<Tr, ALIGNED, false>(drow, pos, T, vzero<V>(), d[j]);
-                load_vec<Tr, ALIGNED, false>(xrow, pos, T, vzero<V>(), x[j]);
+                load_vec<Tr, ALIGNED, false>(arow, pos, lo, hi, vone<V>(), a[j]);
+                load_vec<Tr, ALIGNED, false>(drow, pos, lo, hi, vzero<V>(), d[j]);
+                load_vec<Tr, ALIGNED, false>(xrow, pos, lo, hi, vzero<V>(), x[j]);
             }
         }
 
-        // The two elements just outside the sub-tile: gate[sub_end] and
-        // x[sub_base-1].  Addresses are clamped into the row so the loads are
+        // The two elements just outside the sub-tile: gate at sub_end and x at
+        // sub_base-1.  Addresses are clamped into the row so the loads are
         // unconditional; out-of-row positions take the identity values.
         V a_edge, x_edge;
         {
-            const int64_t ia = sub_end < T ? sub_end : T - 1;
+            const int64_t ia = sub_end < hi ? (sub_end > lo ? sub_end : lo) : hi - 1;
             int64_t ix = sub_base - 1;
-            ix = ix < 0 ? 0 : (ix < T ? ix : T - 1);
+            ix = ix < lo ? lo : (ix < hi ? ix : hi - 1);
             const V av = Tr::load1(arow + ia);
             const V xv = Tr::load1(xrow + ix);
-            a_edge = vselect(sub_end < T, av, vone<V>());
-            x_edge = vselect(sub_base >= 1 && sub_base - 1 < T, xv, vzero<V>());
+            a_edge = vselect(sub_end >= lo && sub_end < hi, av, vone<V>());
+            x_edge = vselect(sub_base - 1 >= lo && sub_base - 1 < hi, xv, vzero<V>());
         }
 
         // Shift gates down by one element (gate[t+1]) and states up by one
@@ -704,11 +758,11 @@ __global__ void __launch_bounds__(64 * kMaxWavesPerBlock)
             }
             const int64_t pos = sub_base + vec_offset<U, EPV, true>(j, lane);
             if (full) {
-                store_vec<Tr, ALIGNED, true>(dtrow, pos, T, dt);
-                store_vec<Tr, ALIGNED, true>(dgrow, pos, T, dg);
+                store_vec<Tr, ALIGNED, true>(dtrow, pos, lo, hi, dt);
+                store_vec<Tr, ALIGNED, true>(dgrow, pos, lo, hi, dg);
             } else {
-                store_vec<Tr, ALIGNED, false>(dtrow, pos, T, dt);
-                store_vec<Tr, ALIGNED, false>(dgrow, pos, T, dg);
+                store_vec<Tr, ALIGNED, false>(dtrow, pos, lo, hi, dt);
+                store_vec<Tr, ALIGNED, false>(dgrow, pos, lo, hi, dg);
             }
         }
     }
@@ -768,7 +822,11 @@ Plan choose_plan(int64_t T, int64_t sub, int64_t element_bytes) {
     return Plan{w, r};
 }
 
-bool is_aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
+// True when both addresses have the same offset inside a 16-byte block, i.e.
+// when 16-byte vectors of the two tensors line up row by row.
+bool same_phase16(const void* p, const void* q) {
+    return ((reinterpret_cast<uintptr_t>(p) ^ reinterpret_cast<uintptr_t>(q)) & 15u) == 0;
+}
 
 int finish_launch() {
     const hipError_t e = hipGetLastError();
@@ -809,7 +867,7 @@ int forward_typed(const void* gates, const void* tokens, void* out, int64_t rows
                   hipStream_t stream) {
     constexpr int EPV = Tr::EPV;
     constexpr int64_t SUB = (int64_t)Tuning<Tr>::U * 64 * EPV;
-    const bool aligned = is_aligned16(gates) && is_aligned16(tokens) && is_aligned16(out) && (T % EPV == 0);
+    const bool aligned = same_phase16(gates, tokens) && same_phase16(gates, out);
     const Plan plan = choose_plan(T, SUB, (int64_t)sizeof(typename Tr::S));
     const int R = plan.rows_per_block;
 #define ASCAN_FWD(WV, AL, RPB)                                                              \
@@ -819,17 +877,20 @@ int forward_typed(const void* gates, const void* tokens, void* out, int64_t rows
         else                                                                                \
             launch_forward<Tr, WV, false, AL>(gates, tokens, out, rows, T, RPB, stream);    \
     } while (0)
-    if (!aligned) {
-        ASCAN_FWD(1, false, 4);  // element-wise kernel: one wave per row
-    } else {
-        switch (plan.waves_per_row) {
-            case 1: ASCAN_FWD(1, true, R); break;
-            case 2: ASCAN_FWD(2, true, R); break;
-            case 4: ASCAN_FWD(4, true, R); break;
-            case 8: ASCAN_FWD(8, true, R); break;
-            default: ASCAN_FWD(16, true, R); break;
-        }
+#define ASCAN_FWD_W(AL)                               \
+    switch (plan.waves_per_row) {                     \
+        case 1: ASCAN_FWD(1, AL, R); break;           \
+        case 2: ASCAN_FWD(2, AL, R); break;           \
+        case 4: ASCAN_FWD(4, AL, R); break;           \
+        case 8: ASCAN_FWD(8, AL, R); break;           \
+        default: ASCAN_FWD(16, AL, R); break;         \
     }
+    if (aligned) {
+        ASCAN_FWD_W(true);
+    } else {
+        ASCAN_FWD_W(false);  // same geometry, element-wise memory access
+    }
+#undef ASCAN_FWD_W
 #undef ASCAN_FWD
     return finish_launch();
 }
@@ -839,23 +900,26 @@ int backward_typed(const void* gates, const void* states, const void* grad_out, 
                    int64_t rows, int64_t T, hipStream_t stream) {
     constexpr int EPV = Tr::EPV;
     constexpr int64_t SUB = (int64_t)Tuning<Tr>::UB * 64 * EPV;
-    const bool aligned = is_aligned16(gates) && is_aligned16(states) && is_aligned16(grad_out) &&
-                         is_aligned16(d_gates) && is_aligned16(d_tokens) && (T % EPV == 0);
+    const bool aligned = same_phase16(gates, states) && same_phase16(gates, grad_out) &&
+                         same_phase16(gates, d_gates) && same_phase16(gates, d_tokens);
     const Plan plan = choose_plan(T, SUB, (int64_t)sizeof(typename Tr::S));
     const int R = plan.rows_per_block;
 #define ASCAN_BWD(WV, AL, RPB) \
     launch_backward<Tr, WV, AL>(gates, states, grad_out, d_gates, d_tokens, rows, T, RPB, stream)
-    if (!aligned) {
-        ASCAN_BWD(1, false, 4);  // element-wise kernel: one wave per row
-    } else {
-        switch (plan.waves_per_row) {
-            case 1: ASCAN_BWD(1, true, R); break;
-            case 2: ASCAN_BWD(2, true, R); break;
-            case 4: ASCAN_BWD(4, true, R); break;
-            case 8: ASCAN_BWD(8, true, R); break;
-            default: ASCAN_BWD(16, true, R); break;
-        }
+#define ASCAN_BWD_W(AL)                               \
+    switch (plan.waves_per_row) {                     \
+        case 1: ASCAN_BWD(1, AL, R); break;           \
+        case 2: ASCAN_BWD(2, AL, R); break;           \
+        case 4: ASCAN_BWD(4, AL, R); break;           \
+        case 8: ASCAN_BWD(8, AL, R); break;           \
+        default: ASCAN_BWD(16, AL, R); break;         \
     }
+    if (aligned) {
+        ASCAN_BWD_W(true);
+    } else {
+        ASCAN_BWD_W(false);  // same geometry, element-wise memory access
+    }
+#undef ASCAN_BWD_W
 #undef ASCAN_BWD
     return finish_launch();
 }

@@ -29,9 +29,10 @@
  *   - input and output buffers must not overlap;
  *   - arithmetic is done in fp32 for every dtype (bf16/fp16 are storage
  *     formats, rounded to nearest-even on store);
- *   - 16-byte aligned base pointers with seqlen*sizeof(element) a multiple of
- *     16 take the vectorised kernels; anything else takes an element-wise
- *     kernel with identical results;
+ *   - buffers whose addresses agree modulo 16 (the usual case: allocator
+ *     blocks, or equal storage offsets) take the vectorised kernels for any
+ *     seqlen; buffers at different offsets inside a 16-byte block take
+ *     element-wise kernels with the same arithmetic;
  *   - errors are reported by return code, never by abort or exception.
  */
 #ifndef ASCAN_H_

@@ -217,36 +217,53 @@ def test_unaligned_rows(dtype, rows, T):
 
 
 @pytest.mark.parametrize("dtype", ALL_DTYPES, ids=ALL_IDS)
-def test_unaligned_base_pointer(dtype):
-    """Views with a storage offset: base pointers off the 16-byte grid."""
+@pytest.mark.parametrize("offsets", [(1, 1, 1), (3, 3, 3), (1, 0, 2)], ids=["same1", "same3", "mixed"])
+@pytest.mark.parametrize("rows,T", [(6, 2048), (3, 40000), (2050, 1031)])
+def test_unaligned_base_pointer(dtype, offsets, rows, T):
+    """Views with a storage offset: base pointers off the 16-byte grid.  Equal
+    offsets keep the vectorised kernels (rows are addressed from the 16-byte
+    boundary below their start); different offsets per tensor take the
+    element-wise kernels."""
     from accelerated_scan import _abi
 
-    rows, T = 6, 2048
     gates, tokens, grad_out = _truth_inputs(rows, T, dtype, seed=9)
 
-    def offset_copy(t):
-        flat = torch.empty(rows * T + 1, dtype=t.dtype, device=DEVICE)
-        view = flat[1:].view(1, rows, T)
+    def offset_copy(t, k):
+        flat = torch.empty(rows * T + 4, dtype=t.dtype, device=DEVICE)
+        view = flat[k:k + rows * T].view(1, rows, T)
         view.copy_(t.reshape(1, rows, T))
-        assert view.data_ptr() % 16 != 0 and view.is_contiguous()
+        assert view.is_contiguous()
         return view
 
-    g, x = offset_copy(gates), offset_copy(tokens)
-    out = offset_copy(torch.zeros_like(tokens))
+    og, ox, oo = offsets
+    g, x, d = offset_copy(gates, og), offset_copy(tokens, ox), offset_copy(grad_out, oo)
+    out, rev = offset_copy(torch.zeros_like(tokens), oo), offset_copy(torch.zeros_like(tokens), og)
+    dg, dx = offset_copy(torch.zeros_like(tokens), ox), offset_copy(torch.zeros_like(tokens), oo)
+    # guard elements just outside the views must stay untouched
+    guards = [t.storage_offset() for t in (out, dg, dx)]
+    for t in (out, rev, dg, dx):
+        t.untyped_storage().fill_(0)
     _abi.forward(g, x, out, False)
-    ref = torch.empty(1, rows, T, dtype=dtype, device=DEVICE)
-    _abi.forward(gates.to(DEVICE).view(1, rows, T), tokens.to(DEVICE).view(1, rows, T), ref, False)
-    assert torch.equal(torch.view_as_real(out) if dtype == torch.complex64 else out,
-                       torch.view_as_real(ref) if dtype == torch.complex64 else ref)
-    d = offset_copy(grad_out)
-    dg, dx = offset_copy(torch.zeros_like(tokens)), offset_copy(torch.zeros_like(tokens))
+    _abi.forward(g, x, rev, True)
     _abi.backward(g, out, d, dg, dx)
-    rdg, rdx = torch.empty_like(ref), torch.empty_like(ref)
-    _abi.backward(gates.to(DEVICE).view(1, rows, T), ref, grad_out.to(DEVICE).view(1, rows, T), rdg, rdx)
-    for a, b in ((dg, rdg), (dx, rdx)):
-        if dtype == torch.complex64:
-            a, b = torch.view_as_real(a), torch.view_as_real(b)
-        assert torch.equal(a, b)
+    torch.cuda.synchronize()
+
+    if dtype == torch.complex64 or dtype == torch.float32:
+        tol = dict(rtol=2e-5, atol=2e-5)
+    else:
+        tol = dict(rtol=2 * storage_ulp[dtype], atol=2 * storage_ulp[dtype])
+    t_out = seqscan.forward(_np32(gates), _np32(tokens))
+    t_rev = seqscan.forward(_np32(gates), _np32(tokens), reverse=True)
+    t_dg, t_dx = seqscan.backward(_np32(gates), _np32(out.reshape(rows, T).cpu()), _np32(grad_out))
+    for name, got, want in (("out", out, t_out), ("rev", rev, t_rev), ("d_tokens", dx, t_dx), ("d_gates", dg, t_dg)):
+        got = _np32(got.reshape(rows, T).cpu())
+        scale = max(1.0, float(np.abs(want).max()))
+        np.testing.assert_allclose(got, want, rtol=tol["rtol"], atol=tol["atol"] * scale, err_msg=name)
+    # nothing was written outside the row range of any output
+    for t in (out, rev, dg, dx):
+        k = t.storage_offset()
+        whole = torch.empty(0, dtype=t.dtype, device=DEVICE).set_(t.untyped_storage())
+        assert whole[:k].abs().sum().item() == 0 and whole[k + rows * T:].abs().sum().item() == 0
 
 
 # ---------------------------------------------------------------------------
