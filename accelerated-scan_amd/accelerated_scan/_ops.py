@@ -1,0 +1,47 @@
+"""The two HIP entry points as ``torch.library`` custom operators.
+
+``torch.compile`` cannot trace a ctypes call; it can trace an opaque custom
+operator that comes with a shape/dtype rule ("fake" implementation).  The
+autograd nodes in ``warp``, ``scalar`` and ``complex`` therefore switch to
+these operators while a graph is being captured and call the C ABI directly
+otherwise (less Python overhead per call).  The reference advertises
+``torch.compile`` for its torch scan only (README.md:36 of the reference).
+"""
+
+from typing import Tuple
+
+import torch
+
+from . import _abi
+
+
+@torch.library.custom_op("accelerated_scan::scan_forward", mutates_args=())
+def scan_forward(gates: torch.Tensor, tokens: torch.Tensor, reverse: bool) -> torch.Tensor:
+    out = torch.empty_like(tokens)
+    _abi.forward(gates, tokens, out, reverse)
+    return out
+
+
+@scan_forward.register_fake
+def _(gates, tokens, reverse):
+    return torch.empty_like(tokens)
+
+
+@torch.library.custom_op("accelerated_scan::scan_backward", mutates_args=())
+def scan_backward(
+    gates: torch.Tensor, states: torch.Tensor, grad_out: torch.Tensor
+) -> Tuple[torch.Tensor, torch.Tensor]:
+    d_gates = torch.empty_like(gates)
+    d_tokens = torch.empty_like(gates)
+    _abi.backward(gates, states, grad_out, d_gates, d_tokens)
+    return d_gates, d_tokens
+
+
+@scan_backward.register_fake
+def _(gates, states, grad_out):
+    return torch.empty_like(gates), torch.empty_like(gates)
+
+
+def capturing() -> bool:
+    """True while torch.compile is tracing the caller."""
+    return torch.compiler.is_compiling()

@@ -9,7 +9,7 @@ backward pass follows complex.py:79-92: with g the adjoint of the states,
 
 import torch
 
-from . import _abi
+from . import _abi, _ops
 
 
 def _require(cond: bool, what: str) -> None:
@@ -48,8 +48,11 @@ class Scan(torch.autograd.Function):
         if real_inputs:
             inputs = torch.complex(inputs, torch.zeros_like(inputs))
 
-        states = torch.empty_like(inputs)
-        _launch_forward(forget, inputs, states)
+        if _ops.capturing():
+            states = _ops.scan_forward(forget, inputs, False)
+        else:
+            states = torch.empty_like(inputs)
+            _launch_forward(forget, inputs, states)
 
         ctx.save_for_backward(forget, states)
         ctx.real_inputs = real_inputs
@@ -63,9 +66,12 @@ class Scan(torch.autograd.Function):
         assert forget.is_contiguous()
         assert states.is_contiguous()
 
-        d_forget = torch.empty_like(forget)
-        d_inputs = torch.empty_like(states)
-        _launch_backward(forget, states, d_output, d_forget, d_inputs)
+        if _ops.capturing():
+            d_forget, d_inputs = _ops.scan_backward(forget, states, d_output)
+        else:
+            d_forget = torch.empty_like(forget)
+            d_inputs = torch.empty_like(states)
+            _launch_backward(forget, states, d_output, d_forget, d_inputs)
 
         if ctx.real_inputs:
             d_inputs = d_inputs.real

@@ -8,7 +8,7 @@ sequence length.  ``Scan`` saves ``(forget, states)`` and returns
 
 import torch
 
-from . import warp
+from . import _ops, warp
 
 
 class Scan(torch.autograd.Function):
@@ -19,8 +19,11 @@ class Scan(torch.autograd.Function):
         assert forget.is_contiguous()
         assert inputs.is_contiguous()
 
-        states = torch.empty_like(inputs)
-        warp.warpscan_forward(forget, inputs, states, False)
+        if _ops.capturing():
+            states = _ops.scan_forward(forget, inputs, False)
+        else:
+            states = torch.empty_like(inputs)
+            warp.warpscan_forward(forget, inputs, states, False)
 
         ctx.save_for_backward(forget, states)
         return states
@@ -33,6 +36,8 @@ class Scan(torch.autograd.Function):
         assert forget.is_contiguous()
         assert states.is_contiguous()
 
+        if _ops.capturing():
+            return _ops.scan_backward(forget, states, d_output)
         d_forget = torch.empty_like(forget)
         d_inputs = torch.empty_like(states)
         warp.warpscan_backward(forget, states, d_output, d_forget, d_inputs)

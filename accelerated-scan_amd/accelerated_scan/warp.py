@@ -10,7 +10,7 @@ output before the kernel runs.
 
 import torch
 
-from . import _abi
+from . import _abi, _ops
 
 _REAL_DTYPES = (torch.float32, torch.bfloat16, torch.float16)
 
@@ -70,6 +70,8 @@ def warpscan_backward(gates, output, outGrad, gateGradOut, tokenGradOut):
 
 def scan_forward(gates, tokens, reverse=False):
     """Forward (or reverse) scan without autograd (accelerated_scan/warp.py:32-35)."""
+    if _ops.capturing():
+        return _ops.scan_forward(gates, tokens, reverse)
     output = torch.empty_like(tokens)
     warpscan_forward(gates, tokens, output, reverse)
     return output
@@ -98,6 +100,8 @@ class Scan(torch.autograd.Function):
         assert states.is_contiguous()
         assert gates.is_contiguous()
 
+        if _ops.capturing():
+            return _ops.scan_backward(gates, states, grad_output)
         d_gates = torch.empty_like(gates)
         d_tokens = torch.empty_like(gates)
         warpscan_backward(gates, states, grad_output, d_gates, d_tokens)
