@@ -101,32 +101,34 @@ def dtype_code(dtype: torch.dtype) -> int:
         ) from None
 
 
-def _stream_handle(device: torch.device) -> int:
-    return torch.cuda.current_stream(device).cuda_stream
+def _launch(device: torch.device, call) -> None:
+    """Run ``call(stream_handle)`` with ``device`` current (kernels launch on the
+    current device) and map the status."""
+    if device.index is None or device.index == torch.cuda.current_device():
+        status = call(torch.cuda.current_stream(device).cuda_stream)
+    else:
+        with torch.cuda.device(device):
+            status = call(torch.cuda.current_stream(device).cuda_stream)
+    if status:
+        check(status)
 
 
 def forward(gates, tokens, out, reverse: bool) -> None:
     """Enqueue ascan_forward on the current stream of the tensors' device."""
-    lib = load()
-    rows = tokens.numel() // tokens.shape[-1] if tokens.shape[-1] else 0
-    with torch.cuda.device(tokens.device):
-        status = lib.ascan_forward(
-            gates.data_ptr(), tokens.data_ptr(), out.data_ptr(),
-            rows, tokens.shape[-1], dtype_code(tokens.dtype), int(bool(reverse)),
-            _stream_handle(tokens.device),
-        )
-    check(status)
+    lib = _lib or load()
+    seqlen = tokens.shape[-1]
+    rows = tokens.numel() // seqlen if seqlen else 0
+    code = dtype_code(tokens.dtype)
+    _launch(tokens.device, lambda stream: lib.ascan_forward(
+        gates.data_ptr(), tokens.data_ptr(), out.data_ptr(), rows, seqlen, code, 1 if reverse else 0, stream))
 
 
 def backward(gates, states, grad_out, d_gates, d_tokens) -> None:
     """Enqueue ascan_backward on the current stream of the tensors' device."""
-    lib = load()
-    rows = gates.numel() // gates.shape[-1] if gates.shape[-1] else 0
-    with torch.cuda.device(gates.device):
-        status = lib.ascan_backward(
-            gates.data_ptr(), states.data_ptr(), grad_out.data_ptr(),
-            d_gates.data_ptr(), d_tokens.data_ptr(),
-            rows, gates.shape[-1], dtype_code(gates.dtype),
-            _stream_handle(gates.device),
-        )
-    check(status)
+    lib = _lib or load()
+    seqlen = gates.shape[-1]
+    rows = gates.numel() // seqlen if seqlen else 0
+    code = dtype_code(gates.dtype)
+    _launch(gates.device, lambda stream: lib.ascan_backward(
+        gates.data_ptr(), states.data_ptr(), grad_out.data_ptr(), d_gates.data_ptr(), d_tokens.data_ptr(),
+        rows, seqlen, code, stream))

@@ -57,7 +57,7 @@
 #define ASCAN_U_16BIT 4
 #endif
 #ifndef ASCAN_U_BWD_16BIT
-#define ASCAN_U_BWD_16BIT 2
+#define ASCAN_U_BWD_16BIT 4
 #endif
 #ifndef ASCAN_U_C64
 #define ASCAN_U_C64 4
@@ -238,6 +238,7 @@ struct TraitsF32 {
     using S = float;
     using V = float;
     static constexpr int EPV = 4;
+    static constexpr bool kNarrow = false;  // unpacked form is no larger than the raw vector
     static __device__ __forceinline__ void unpack(const u32x4_t& r, V (&d)[EPV]) {
         d[0] = i2f(r.x);
         d[1] = i2f(r.y);
@@ -260,6 +261,7 @@ struct TraitsBF16 {
     using S = uint16_t;
     using V = float;
     static constexpr int EPV = 8;
+    static constexpr bool kNarrow = true;
     static __device__ __forceinline__ uint32_t pack2(float lo, float hi) {
         floatx2_t f;
         f.x = lo;
@@ -291,6 +293,7 @@ struct TraitsF16 {
     using S = uint16_t;
     using V = float;
     static constexpr int EPV = 8;
+    static constexpr bool kNarrow = true;
     static __device__ __forceinline__ uint32_t pack2(float lo, float hi) {
         floatx2_t f;
         f.x = lo;
@@ -328,6 +331,7 @@ struct TraitsC64 {
     using S = cfloat;  // 8 bytes, interleaved (re, im)
     using V = cfloat;
     static constexpr int EPV = 2;
+    static constexpr bool kNarrow = false;
     static __device__ __forceinline__ void unpack(const u32x4_t& r, V (&d)[EPV]) {
         d[0].re = i2f(r.x);
         d[0].im = i2f(r.y);
@@ -359,81 +363,116 @@ struct TraitsC64 {
 
 // ---------------------------------------------------------------------------
 // Vector access.  A row is addressed in "virtual" positions: position 0 is the
-// 16-byte boundary at or just below the row's first element, the row's
-// elements occupy [lo, hi) with 0 <= lo < EPV, and `rowp` points at virtual
-// position 0.  `pos` is the virtual position of the first element of a vector.
-//   ALIGNED: rowp + pos is 16-byte aligned (pos is a multiple of EPV), so
-//            vectors move as one dwordx4.  A vector that straddles a row end
-//            (at most two per row) is read whole and masked, and stored
-//            element by element so a neighbouring row's bytes are never
-//            written.  The !ALIGNED kernels move everything element by element.
-//   FULL   : the whole vector is known to lie inside the row.
+// 16-byte boundary at or just below the row's first element and the row's
+// elements occupy [lo, hi) with 0 <= lo < EPV.  Inside the tile loop everything
+// is expressed relative to the wave's sub-tile: `sub` points at the first
+// element of the sub-tile (wave-uniform, 64-bit), `off` is the lane's 32-bit
+// element offset inside it, and a Window holds the row's valid range relative
+// to the sub-tile.  Only `off` is per-lane state.
+//   ALIGNED: sub + off is 16-byte aligned, so vectors move as one dwordx4.  A
+//            vector that straddles a row end (at most two per row) is read
+//            whole and masked, and stored element by element so a neighbouring
+//            row's bytes are never written.  The !ALIGNED kernels move
+//            everything element by element.
+//   FULL   : the whole sub-tile is known to lie inside the row.
 // ---------------------------------------------------------------------------
-template <class Tr, bool FULL>
-__device__ __forceinline__ void load_elements(const typename Tr::S* __restrict__ rowp, int64_t pos, int64_t lo,
-                                              int64_t hi, typename Tr::V fill, typename Tr::V (&dst)[Tr::EPV]) {
-#pragma unroll
-    for (int e = 0; e < Tr::EPV; ++e) {
-        if (FULL || (pos + e >= lo && pos + e < hi)) {
-            dst[e] = Tr::load1(rowp + pos + e);
-        } else {
-            dst[e] = fill;
-        }
-    }
+struct Window {
+    int lo, hi;  // valid element offsets: lo <= off < hi (clamped to +-2^30)
+};
+
+__device__ __forceinline__ Window make_window(int64_t lo, int64_t hi, int64_t sub_base) {
+    constexpr int64_t kClamp = 1 << 30;
+    int64_t l = lo - sub_base, h = hi - sub_base;
+    l = l < -kClamp ? -kClamp : (l > kClamp ? kClamp : l);
+    h = h < -kClamp ? -kClamp : (h > kClamp ? kClamp : h);
+    Window win;
+    win.lo = (int)l;
+    win.hi = (int)h;
+    return win;
 }
 
+__device__ __forceinline__ bool in_window(Window win, int off) { return off >= win.lo && off < win.hi; }
+
+// Returns the vector as raw bits with out-of-row elements replaced by `fill`.
+// The caller guarantees that the sub-tile overlaps the row unless FULL.
 template <class Tr, bool ALIGNED, bool FULL>
-__device__ __forceinline__ void load_vec(const typename Tr::S* __restrict__ rowp, int64_t pos, int64_t lo,
-                                         int64_t hi, typename Tr::V fill, typename Tr::V (&dst)[Tr::EPV]) {
+__device__ __forceinline__ u32x4_t load_raw(const typename Tr::S* __restrict__ sub, int off, Window win,
+                                            typename Tr::V fill) {
+    constexpr int EPV = Tr::EPV;
     if constexpr (ALIGNED) {
         // A vector that straddles a row end is still read whole: an aligned
         // 16-byte read that overlaps the row cannot leave the row's memory
         // page, and the bytes of the neighbouring row are discarded below.  A
-        // vector entirely outside the row re-reads the row's first vector
-        // instead, so the load stays unconditional.
-        int64_t p = pos;
-        if (!FULL && !(pos + Tr::EPV > lo && pos < hi)) p = 0;
-#if ASCAN_NT_LOAD
-        const u32x4_t raw = __builtin_nontemporal_load(reinterpret_cast<const u32x4_t*>(rowp + p));
-#else
-        const u32x4_t raw = *reinterpret_cast<const u32x4_t*>(rowp + p);
-#endif
-        Tr::unpack(raw, dst);
+        // vector entirely outside the row re-reads a vector of this sub-tile
+        // that does overlap it, so the load stays unconditional.
+        int o = off;
         if (!FULL) {
+            const int safe = win.lo > 0 ? (win.lo / EPV) * EPV : 0;
+            o = (off + EPV > win.lo && off < win.hi) ? off : safe;
+        }
+#if ASCAN_NT_LOAD
+        u32x4_t raw = __builtin_nontemporal_load(reinterpret_cast<const u32x4_t*>(sub + o));
+#else
+        u32x4_t raw = *reinterpret_cast<const u32x4_t*>(sub + o);
+#endif
+        if (!FULL) {
+            typename Tr::V v[EPV];
+            Tr::unpack(raw, v);
 #pragma unroll
-            for (int e = 0; e < Tr::EPV; ++e) {
-                dst[e] = vselect(pos + e >= lo && pos + e < hi, dst[e], fill);
+            for (int e = 0; e < EPV; ++e) v[e] = vselect(in_window(win, off + e), v[e], fill);
+            raw = Tr::pack(v);  // exact: every storage value survives the round trip
+        }
+        return raw;
+    } else {
+        typename Tr::V v[EPV];
+#pragma unroll
+        for (int e = 0; e < EPV; ++e) {
+            if (FULL || in_window(win, off + e)) {
+                v[e] = Tr::load1(sub + off + e);
+            } else {
+                v[e] = fill;
             }
         }
-    } else {
-        load_elements<Tr, FULL>(rowp, pos, lo, hi, fill, dst);
+        return Tr::pack(v);
     }
 }
 
-template <class Tr, bool FULL>
-__device__ __forceinline__ void store_elements(typename Tr::S* __restrict__ rowp, int64_t pos, int64_t lo,
-                                               int64_t hi, const typename Tr::V (&src)[Tr::EPV]) {
+// The vector every lane holds when the sub-tile lies entirely outside the row.
+template <class Tr>
+__device__ __forceinline__ u32x4_t fill_raw(typename Tr::V fill) {
+    typename Tr::V v[Tr::EPV];
 #pragma unroll
-    for (int e = 0; e < Tr::EPV; ++e) {
-        if (FULL || (pos + e >= lo && pos + e < hi)) Tr::store1(rowp + pos + e, src[e]);
-    }
+    for (int e = 0; e < Tr::EPV; ++e) v[e] = fill;
+    return Tr::pack(v);
+}
+
+// Makes the compiler forget what it knows about `raw`, so that values unpacked
+// from it before this point are not kept alive for re-use after it.  For the
+// 16-bit formats the raw vector is half the registers of its unpacked form.
+__device__ __forceinline__ void forget_unpacked(u32x4_t& raw) {
+    unsigned x = raw.x, y = raw.y, z = raw.z, w = raw.w;
+    asm volatile("" : "+v"(x), "+v"(y), "+v"(z), "+v"(w));
+    raw.x = x;
+    raw.y = y;
+    raw.z = z;
+    raw.w = w;
 }
 
 template <class Tr, bool ALIGNED, bool FULL>
-__device__ __forceinline__ void store_vec(typename Tr::S* __restrict__ rowp, int64_t pos, int64_t lo, int64_t hi,
+__device__ __forceinline__ void store_vec(typename Tr::S* __restrict__ sub, int off, Window win,
                                           const typename Tr::V (&src)[Tr::EPV]) {
-    if constexpr (ALIGNED) {
-        if (FULL || (pos >= lo && pos + Tr::EPV <= hi)) {
+    constexpr int EPV = Tr::EPV;
+    if (ALIGNED && (FULL || (off >= win.lo && off + EPV <= win.hi))) {
 #if ASCAN_NT_STORE
-            __builtin_nontemporal_store(Tr::pack(src), reinterpret_cast<u32x4_t*>(rowp + pos));
+        __builtin_nontemporal_store(Tr::pack(src), reinterpret_cast<u32x4_t*>(sub + off));
 #else
-            *reinterpret_cast<u32x4_t*>(rowp + pos) = Tr::pack(src);
+        *reinterpret_cast<u32x4_t*>(sub + off) = Tr::pack(src);
 #endif
-        } else {
-            store_elements<Tr, false>(rowp, pos, lo, hi, src);
-        }
     } else {
-        store_elements<Tr, FULL>(rowp, pos, lo, hi, src);
+#pragma unroll
+        for (int e = 0; e < EPV; ++e) {
+            if (FULL || in_window(win, off + e)) Tr::store1(sub + off + e, src[e]);
+        }
     }
 }
 
@@ -532,7 +571,7 @@ __device__ __forceinline__ void exchange_carries(const V (&totA)[U], const V (&t
 // rows of a workgroup are adjacent in memory, so with W*R = 16 one tile step
 // of the workgroup covers one contiguous span of 16 sub-tiles.
 // ---------------------------------------------------------------------------
-template <class Tr, int W, int U, bool REV, bool ALIGNED>
+template <class Tr, int W, int U, bool REV, bool ALIGNED, bool REGULAR>
 __global__ void __launch_bounds__(64 * kMaxWavesPerBlock)
     scan_forward_kernel(const typename Tr::S* __restrict__ gates, const typename Tr::S* __restrict__ tokens,
                         typename Tr::S* __restrict__ out, int64_t rows, int64_t T) {
@@ -544,7 +583,7 @@ __global__ void __launch_bounds__(64 * kMaxWavesPerBlock)
 
     const int lane = threadIdx.x & 63;
     // rows start at the same misalignment when T is a multiple of the vector width
-    const int head = ALIGNED ? (T % EPV == 0 ? row_lead<Tr>(gates) : EPV - 1) : 0;
+    const int head = REGULAR ? 0 : (ALIGNED ? (T % EPV == 0 ? row_lead<Tr>(gates) : EPV - 1) : 0);
     const int64_t ntiles = tiles_per_row(T, TILE, head);
     __shared__ V slots_all[W == 1 ? 1 : 2 * kSlotsPerBuffer];
     int64_t row;
@@ -552,7 +591,7 @@ __global__ void __launch_bounds__(64 * kMaxWavesPerBlock)
     if (!locate_wave<W>(rows, ntiles, row, w, slot_base)) return;  // wave-uniform
     V* slots = slots_all + (W == 1 ? 0 : slot_base);
 
-    const int64_t lo = ALIGNED ? row_lead<Tr>(gates + row * T) : 0;
+    const int64_t lo = (ALIGNED && !REGULAR) ? row_lead<Tr>(gates + row * T) : 0;
     const int64_t hi = lo + T;
     const S* __restrict__ grow = gates + row * T - lo;
     const S* __restrict__ trow = tokens + row * T - lo;
@@ -563,36 +602,54 @@ __global__ void __launch_bounds__(64 * kMaxWavesPerBlock)
     for (int64_t k = 0; k < ntiles; ++k) {
         const int64_t tile = REV ? (ntiles - 1 - k) : k;
         const int64_t sub_base = tile * TILE + (int64_t)(REV ? (W - 1 - w) : w) * SUB;
-        const bool full = sub_base >= lo && sub_base + SUB <= hi;  // wave-uniform
+        const bool full = REGULAR || (sub_base >= lo && sub_base + SUB <= hi);  // wave-uniform
 
-        V g[U][EPV], t[U][EPV];
+        const Window win = make_window(lo, hi, sub_base);
+        const bool touches = win.hi > 0 && win.lo < SUB;  // wave-uniform
+        const S* __restrict__ gsub = grow + sub_base;
+        const S* __restrict__ tsub = trow + sub_base;
+        S* __restrict__ osub = orow + sub_base;
+
+        u32x4_t graw[U], traw[U];
         if (full) {
 #pragma unroll
             for (int j = 0; j < U; ++j) {
-                const int64_t pos = sub_base + vec_offset<U, EPV, REV>(j, lane);
-                load_vec<Tr, ALIGNED, true>(grow, pos, lo, hi, vone<V>(), g[j]);
-                load_vec<Tr, ALIGNED, true>(trow, pos, lo, hi, vzero<V>(), t[j]);
+                const int off = vec_offset<U, EPV, REV>(j, lane);
+                graw[j] = load_raw<Tr, ALIGNED, true>(gsub, off, win, vone<V>());
+                traw[j] = load_raw<Tr, ALIGNED, true>(tsub, off, win, vzero<V>());
             }
-        } else {
+        } else if constexpr (!REGULAR) {
+            if (touches) {
 #pragma unroll
-            for (int j = 0; j < U; ++j) {
-                const int64_t pos = sub_base + vec_offset<U, EPV, REV>(j, lane);
-                load_vec<Tr, ALIGNED, false>(grow, pos, lo, hi, vone<V>(), g[j]);
-                load_vec<Tr, ALIGNED, false>(trow, pos, lo, hi, vzero<V>(), t[j]);
+                for (int j = 0; j < U; ++j) {
+                    const int off = vec_offset<U, EPV, REV>(j, lane);
+                    graw[j] = load_raw<Tr, ALIGNED, false>(gsub, off, win, vone<V>());
+                    traw[j] = load_raw<Tr, ALIGNED, false>(tsub, off, win, vzero<V>());
+                }
+            } else {
+#pragma unroll
+                for (int j = 0; j < U; ++j) {
+                    graw[j] = fill_raw<Tr>(vone<V>());
+                    traw[j] = fill_raw<Tr>(vzero<V>());
+                }
             }
         }
 
+        // Pass 1: fold each vector into one (A, X) pair and scan the pairs.
         V totA[U], totX[U], exA[U], exX[U];
 #pragma unroll
         for (int j = 0; j < U; ++j) {
+            V g[EPV], t[EPV];
+            Tr::unpack(graw[j], g);
+            Tr::unpack(traw[j], t);
             constexpr int e0 = REV ? EPV - 1 : 0;
-            V A = g[j][e0];
-            V X = t[j][e0];
+            V A = g[e0];
+            V X = t[e0];
 #pragma unroll
             for (int i = 1; i < EPV; ++i) {
                 const int e = REV ? EPV - 1 - i : i;
-                X = vfma(g[j][e], X, t[j][e]);
-                A = vmul(A, g[j][e]);
+                X = vfma(g[e], X, t[e]);
+                A = vmul(A, g[e]);
             }
             wave_scan_inclusive(A, X);
             totA[j] = read_lane<63>(A);
@@ -604,22 +661,30 @@ __global__ void __launch_bounds__(64 * kMaxWavesPerBlock)
         V c;
         exchange_carries<V, W, U>(totA, totX, carry, c, slots, (int)(k & 1), w, lane);
 
+        // Pass 2: the plain recurrence from the state entering each lane.
 #pragma unroll
         for (int j = 0; j < U; ++j) {
+            if constexpr (Tr::kNarrow) {
+                forget_unpacked(graw[j]);
+                forget_unpacked(traw[j]);
+            }
+            V g[EPV], t[EPV];
+            Tr::unpack(graw[j], g);
+            Tr::unpack(traw[j], t);
             V x = vfma(exA[j], c, exX[j]);  // state entering this lane's vector
             c = vfma(totA[j], c, totX[j]);  // state entering the next block
             V o[EPV];
 #pragma unroll
             for (int i = 0; i < EPV; ++i) {
                 const int e = REV ? EPV - 1 - i : i;
-                x = vfma(g[j][e], x, t[j][e]);
+                x = vfma(g[e], x, t[e]);
                 o[e] = x;
             }
-            const int64_t pos = sub_base + vec_offset<U, EPV, REV>(j, lane);
+            const int off = vec_offset<U, EPV, REV>(j, lane);
             if (full) {
-                store_vec<Tr, ALIGNED, true>(orow, pos, lo, hi, o);
-            } else {
-                store_vec<Tr, ALIGNED, false>(orow, pos, lo, hi, o);
+                store_vec<Tr, ALIGNED, true>(osub, off, win, o);
+            } else if constexpr (!REGULAR) {
+                if (touches) store_vec<Tr, ALIGNED, false>(osub, off, win, o);
             }
         }
     }
@@ -629,7 +694,7 @@ __global__ void __launch_bounds__(64 * kMaxWavesPerBlock)
 // Fused backward kernel: reverse-time scan over gate[t+1] producing d_tokens,
 // and d_gates[t] = d_tokens[t] * conj(x[t-1]) in the same pass.
 // ---------------------------------------------------------------------------
-template <class Tr, int W, int U, bool ALIGNED>
+template <class Tr, int W, int U, bool ALIGNED, bool REGULAR>
 __global__ void __launch_bounds__(64 * kMaxWavesPerBlock)
     scan_backward_kernel(const typename Tr::S* __restrict__ gates, const typename Tr::S* __restrict__ states,
                          const typename Tr::S* __restrict__ grad_out, typename Tr::S* __restrict__ d_gates,
@@ -642,7 +707,7 @@ __global__ void __launch_bounds__(64 * kMaxWavesPerBlock)
 
     const int lane = threadIdx.x & 63;
     // rows start at the same misalignment when T is a multiple of the vector width
-    const int head = ALIGNED ? (T % EPV == 0 ? row_lead<Tr>(gates) : EPV - 1) : 0;
+    const int head = REGULAR ? 0 : (ALIGNED ? (T % EPV == 0 ? row_lead<Tr>(gates) : EPV - 1) : 0);
     const int64_t ntiles = tiles_per_row(T, TILE, head);
     __shared__ V slots_all[W == 1 ? 1 : 2 * kSlotsPerBuffer];
     int64_t row;
@@ -650,7 +715,7 @@ __global__ void __launch_bounds__(64 * kMaxWavesPerBlock)
     if (!locate_wave<W>(rows, ntiles, row, w, slot_base)) return;  // wave-uniform
     V* slots = slots_all + (W == 1 ? 0 : slot_base);
 
-    const int64_t lo = ALIGNED ? row_lead<Tr>(gates + row * T) : 0;
+    const int64_t lo = (ALIGNED && !REGULAR) ? row_lead<Tr>(gates + row * T) : 0;
     const int64_t hi = lo + T;
     const S* __restrict__ arow = gates + row * T - lo;
     const S* __restrict__ xrow = states + row * T - lo;
@@ -664,24 +729,41 @@ __global__ void __launch_bounds__(64 * kMaxWavesPerBlock)
         const int64_t tile = ntiles - 1 - k;
         const int64_t sub_base = tile * TILE + (int64_t)(W - 1 - w) * SUB;
         const int64_t sub_end = sub_base + SUB;
-        const bool full = sub_base >= lo && sub_end <= hi;  // wave-uniform
+        const bool full = REGULAR || (sub_base >= lo && sub_end <= hi);  // wave-uniform
 
-        V a[U][EPV], d[U][EPV], x[U][EPV];
+        const Window win = make_window(lo, hi, sub_base);
+        const bool touches = win.hi > 0 && win.lo < SUB;  // wave-uniform
+        const S* __restrict__ asub = arow + sub_base;
+        const S* __restrict__ dsub = drow + sub_base;
+        const S* __restrict__ xsub = xrow + sub_base;
+        S* __restrict__ dgsub = dgrow + sub_base;
+        S* __restrict__ dtsub = dtrow + sub_base;
+
+        u32x4_t araw[U], draw[U], xraw[U];
         if (full) {
 #pragma unroll
             for (int j = 0; j < U; ++j) {
-                const int64_t pos = sub_base + vec_offset<U, EPV, true>(j, lane);
-                load_vec<Tr, ALIGNED, true>(arow, pos, lo, hi, vone<V>(), a[j]);
-                load_vec<Tr, ALIGNED, true>(drow, pos, lo, hi, vzero<V>(), d[j]);
-                load_vec<Tr, ALIGNED, true>(xrow, pos, lo, hi, vzero<V>(), x[j]);
+                const int off = vec_offset<U, EPV, true>(j, lane);
+                araw[j] = load_raw<Tr, ALIGNED, true>(asub, off, win, vone<V>());
+                draw[j] = load_raw<Tr, ALIGNED, true>(dsub, off, win, vzero<V>());
+                xraw[j] = load_raw<Tr, ALIGNED, true>(xsub, off, win, vzero<V>());
             }
-        } else {
+        } else if constexpr (!REGULAR) {
+            if (touches) {
 #pragma unroll
-            for (int j = 0; j < U; ++j) {
-                const int64_t pos = sub_base + vec_offset<U, EPV, true>(j, lane);
-                load_vec<Tr, ALIGNED, false>(arow, pos, lo, hi, vone<V>(), a[j]);
-                load_vec<Tr, ALIGNED, false>(drow, pos, lo, hi, vzero<V>(), d[j]);
-                load_vec<Tr, ALIGNED, false>(xrow, pos, lo, hi, vzero<V>(), x[j]);
+                for (int j = 0; j < U; ++j) {
+                    const int off = vec_offset<U, EPV, true>(j, lane);
+                    araw[j] = load_raw<Tr, ALIGNED, false>(asub, off, win, vone<V>());
+                    draw[j] = load_raw<Tr, ALIGNED, false>(dsub, off, win, vzero<V>());
+                    xraw[j] = load_raw<Tr, ALIGNED, false>(xsub, off, win, vzero<V>());
+                }
+            } else {
+#pragma unroll
+                for (int j = 0; j < U; ++j) {
+                    araw[j] = fill_raw<Tr>(vone<V>());
+                    draw[j] = fill_raw<Tr>(vzero<V>());
+                    xraw[j] = fill_raw<Tr>(vzero<V>());
+                }
             }
         }
 
@@ -699,41 +781,45 @@ __global__ void __launch_bounds__(64 * kMaxWavesPerBlock)
             x_edge = vselect(sub_base - 1 >= lo && sub_base - 1 < hi, xv, vzero<V>());
         }
 
-        // Shift gates down by one element (gate[t+1]) and states up by one
-        // (x[t-1]); in scan order the neighbour vector at the next higher
-        // address is lane-1, the one at the next lower address is lane+1.
-        V ga[U][EPV], xs[U][EPV];
+        // Pass 1.  Gates are needed one element later (gate[t+1]) and states one
+        // element earlier (x[t-1]).  In scan order the vector at the next higher
+        // address belongs to lane-1 and the one at the next lower address to
+        // lane+1, so each block needs one value from each neighbour: a_next (the
+        // first gate of the vector above) and x_prev (the last state of the
+        // vector below).
+        V a_next[U], x_prev[U];
+        V totA[U], totX[U], exA[U], exX[U];
 #pragma unroll
         for (int j = 0; j < U; ++j) {
+            V a[EPV], d[EPV], x[EPV];
+            Tr::unpack(araw[j], a);
+            Tr::unpack(draw[j], d);
+            Tr::unpack(xraw[j], x);
             V hi_edge, lo_edge;
             if (j == 0) {
                 hi_edge = a_edge;
             } else {
-                hi_edge = read_lane<63>(a[j - 1][0]);
+                V above[EPV];
+                Tr::unpack(araw[j > 0 ? j - 1 : 0], above);
+                hi_edge = read_lane<63>(above[0]);
             }
             if (j == U - 1) {
                 lo_edge = x_edge;
             } else {
-                lo_edge = read_lane<0>(x[j + 1][EPV - 1]);
+                V below[EPV];
+                Tr::unpack(xraw[j < U - 1 ? j + 1 : j], below);
+                lo_edge = read_lane<0>(below[EPV - 1]);
             }
-            const V a_next = shift_up1(a[j][0], hi_edge);
-            const V x_prev = shift_down1(x[j][EPV - 1], lo_edge);
-#pragma unroll
-            for (int e = 0; e < EPV; ++e) {
-                ga[j][e] = vconj(e < EPV - 1 ? a[j][e + 1] : a_next);
-                xs[j][e] = vconj(e > 0 ? x[j][e - 1] : x_prev);
-            }
-        }
+            a_next[j] = shift_up1(a[0], hi_edge);
+            x_prev[j] = shift_down1(x[EPV - 1], lo_edge);
 
-        V totA[U], totX[U], exA[U], exX[U];
-#pragma unroll
-        for (int j = 0; j < U; ++j) {
-            V A = ga[j][EPV - 1];
-            V X = d[j][EPV - 1];
+            V A = vconj(a_next[j]);
+            V X = d[EPV - 1];
 #pragma unroll
             for (int e = EPV - 2; e >= 0; --e) {
-                X = vfma(ga[j][e], X, d[j][e]);
-                A = vmul(A, ga[j][e]);
+                const V ga = vconj(a[e + 1]);
+                X = vfma(ga, X, d[e]);
+                A = vmul(A, ga);
             }
             wave_scan_inclusive(A, X);
             totA[j] = read_lane<63>(A);
@@ -745,24 +831,38 @@ __global__ void __launch_bounds__(64 * kMaxWavesPerBlock)
         V c;
         exchange_carries<V, W, U>(totA, totX, carry, c, slots, (int)(k & 1), w, lane);
 
+        // Pass 2: the plain reverse recurrence and the gate gradient.
 #pragma unroll
         for (int j = 0; j < U; ++j) {
+            if constexpr (Tr::kNarrow) {
+                forget_unpacked(araw[j]);
+                forget_unpacked(draw[j]);
+                forget_unpacked(xraw[j]);
+            }
+            V a[EPV], d[EPV], x[EPV];
+            Tr::unpack(araw[j], a);
+            Tr::unpack(draw[j], d);
+            Tr::unpack(xraw[j], x);
             V gr = vfma(exA[j], c, exX[j]);  // g entering this lane's vector from above
             c = vfma(totA[j], c, totX[j]);
             V dt[EPV], dg[EPV];
 #pragma unroll
             for (int e = EPV - 1; e >= 0; --e) {
-                gr = vfma(ga[j][e], gr, d[j][e]);
+                const V ga = vconj(e < EPV - 1 ? a[e + 1] : a_next[j]);
+                const V xs = vconj(e > 0 ? x[e - 1] : x_prev[j]);
+                gr = vfma(ga, gr, d[e]);
                 dt[e] = gr;
-                dg[e] = vmul(gr, xs[j][e]);
+                dg[e] = vmul(gr, xs);
             }
-            const int64_t pos = sub_base + vec_offset<U, EPV, true>(j, lane);
+            const int off = vec_offset<U, EPV, true>(j, lane);
             if (full) {
-                store_vec<Tr, ALIGNED, true>(dtrow, pos, lo, hi, dt);
-                store_vec<Tr, ALIGNED, true>(dgrow, pos, lo, hi, dg);
-            } else {
-                store_vec<Tr, ALIGNED, false>(dtrow, pos, lo, hi, dt);
-                store_vec<Tr, ALIGNED, false>(dgrow, pos, lo, hi, dg);
+                store_vec<Tr, ALIGNED, true>(dtsub, off, win, dt);
+                store_vec<Tr, ALIGNED, true>(dgsub, off, win, dg);
+            } else if constexpr (!REGULAR) {
+                if (touches) {
+                    store_vec<Tr, ALIGNED, false>(dtsub, off, win, dt);
+                    store_vec<Tr, ALIGNED, false>(dgsub, off, win, dg);
+                }
             }
         }
     }
@@ -777,10 +877,12 @@ thread_local int g_last_hip_error = 0;
 // sub-tiles are 4 KiB of each tensor; the backward kernel holds three input
 // tensors in registers and takes half of that where 4 KiB would spill.
 template <class Tr> struct Tuning;
-template <> struct Tuning<TraitsF32> { static constexpr int U = ASCAN_U_F32, UB = ASCAN_U_BWD_F32; };
-template <> struct Tuning<TraitsBF16> { static constexpr int U = ASCAN_U_16BIT, UB = ASCAN_U_BWD_16BIT; };
-template <> struct Tuning<TraitsF16> { static constexpr int U = ASCAN_U_16BIT, UB = ASCAN_U_BWD_16BIT; };
-template <> struct Tuning<TraitsC64> { static constexpr int U = ASCAN_U_C64, UB = ASCAN_U_BWD_C64; };
+// UG and UBG are the values for the kernels that carry masking code (rows of
+// arbitrary start and length), which need registers for the masks.
+template <> struct Tuning<TraitsF32> { static constexpr int U = ASCAN_U_F32, UG = ASCAN_U_F32, UB = ASCAN_U_BWD_F32, UBG = 2; };
+template <> struct Tuning<TraitsBF16> { static constexpr int U = ASCAN_U_16BIT, UG = 2, UB = ASCAN_U_BWD_16BIT, UBG = 2; };
+template <> struct Tuning<TraitsF16> { static constexpr int U = ASCAN_U_16BIT, UG = 2, UB = ASCAN_U_BWD_16BIT, UBG = 2; };
+template <> struct Tuning<TraitsC64> { static constexpr int U = ASCAN_U_C64, UG = ASCAN_U_C64, UB = ASCAN_U_BWD_C64, UBG = 2; };
 
 // Launch geometry: W waves per row, R rows per workgroup (W*R <= 16).
 struct Plan {
@@ -837,58 +939,81 @@ int finish_launch() {
     return ASCAN_OK;
 }
 
-template <class Tr, int W, bool REV, bool ALIGNED>
+template <class Tr, int W, bool REV, bool ALIGNED, bool REGULAR>
 void launch_forward(const void* gates, const void* tokens, void* out, int64_t rows, int64_t T, int rows_per_block,
                     hipStream_t stream) {
     using S = typename Tr::S;
-    constexpr int U = Tuning<Tr>::U;
+    constexpr int U = REGULAR ? Tuning<Tr>::U : Tuning<Tr>::UG;
     const unsigned blocks = (unsigned)((rows + rows_per_block - 1) / rows_per_block);
     const unsigned threads = 64u * W * rows_per_block;
-    hipLaunchKernelGGL((scan_forward_kernel<Tr, W, U, REV, ALIGNED>), dim3(blocks), dim3(threads), 0, stream,
+    hipLaunchKernelGGL((scan_forward_kernel<Tr, W, U, REV, ALIGNED, REGULAR>), dim3(blocks), dim3(threads), 0, stream,
                        static_cast<const S*>(gates), static_cast<const S*>(tokens), static_cast<S*>(out), rows,
                        T);
 }
 
-template <class Tr, int W, bool ALIGNED>
+template <class Tr, int W, bool ALIGNED, bool REGULAR>
 void launch_backward(const void* gates, const void* states, const void* grad_out, void* d_gates,
                      void* d_tokens, int64_t rows, int64_t T, int rows_per_block, hipStream_t stream) {
     using S = typename Tr::S;
-    constexpr int U = Tuning<Tr>::UB;
+    constexpr int U = REGULAR ? Tuning<Tr>::UB : Tuning<Tr>::UBG;
     const unsigned blocks = (unsigned)((rows + rows_per_block - 1) / rows_per_block);
     const unsigned threads = 64u * W * rows_per_block;
-    hipLaunchKernelGGL((scan_backward_kernel<Tr, W, U, ALIGNED>), dim3(blocks), dim3(threads), 0, stream,
+    hipLaunchKernelGGL((scan_backward_kernel<Tr, W, U, ALIGNED, REGULAR>), dim3(blocks), dim3(threads), 0, stream,
                        static_cast<const S*>(gates), static_cast<const S*>(states),
                        static_cast<const S*>(grad_out), static_cast<S*>(d_gates), static_cast<S*>(d_tokens),
                        rows, T);
 }
 
+// Memory-access flavour of a launch.
+//   kRegular    : every row starts on a 16-byte boundary and is a whole number
+//                 of tiles long, so every sub-tile is full: the kernel carries
+//                 no masking code at all (the common case: T a power of two).
+//   kVector     : all tensors share one offset inside a 16-byte block; rows may
+//                 start anywhere and have any length.  Whole dwordx4 accesses
+//                 except where a vector straddles a row end.
+//   kElementwise: tensors at different offsets inside a 16-byte block.
+enum class Access { kRegular, kVector, kElementwise };
+
+bool is_aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
+
+Access choose_access(bool same_phase, const void* first, int64_t T, int64_t tile) {
+    if (!same_phase) return Access::kElementwise;
+    if (is_aligned16(first) && T % tile == 0) return Access::kRegular;
+    return Access::kVector;
+}
+
 template <class Tr>
 int forward_typed(const void* gates, const void* tokens, void* out, int64_t rows, int64_t T, bool reverse,
                   hipStream_t stream) {
-    constexpr int EPV = Tr::EPV;
-    constexpr int64_t SUB = (int64_t)Tuning<Tr>::U * 64 * EPV;
-    const bool aligned = same_phase16(gates, tokens) && same_phase16(gates, out);
-    const Plan plan = choose_plan(T, SUB, (int64_t)sizeof(typename Tr::S));
+    constexpr int64_t kElem = (int64_t)sizeof(typename Tr::S);
+    constexpr int64_t SUB = (int64_t)Tuning<Tr>::U * 64 * Tr::EPV;    // regular kernels
+    constexpr int64_t SUBG = (int64_t)Tuning<Tr>::UG * 64 * Tr::EPV;  // kernels with masking code
+    Plan plan = choose_plan(T, SUB, kElem);
+    const Access access = choose_access(same_phase16(gates, tokens) && same_phase16(gates, out), gates, T,
+                                        SUB * plan.waves_per_row);
+    if (access != Access::kRegular) plan = choose_plan(T, SUBG, kElem);
     const int R = plan.rows_per_block;
-#define ASCAN_FWD(WV, AL, RPB)                                                              \
-    do {                                                                                    \
-        if (reverse)                                                                        \
-            launch_forward<Tr, WV, true, AL>(gates, tokens, out, rows, T, RPB, stream);     \
-        else                                                                                \
-            launch_forward<Tr, WV, false, AL>(gates, tokens, out, rows, T, RPB, stream);    \
+#define ASCAN_FWD(WV, AL, REG)                                                               \
+    do {                                                                                     \
+        if (reverse)                                                                         \
+            launch_forward<Tr, WV, true, AL, REG>(gates, tokens, out, rows, T, R, stream);   \
+        else                                                                                 \
+            launch_forward<Tr, WV, false, AL, REG>(gates, tokens, out, rows, T, R, stream);  \
     } while (0)
-#define ASCAN_FWD_W(AL)                               \
-    switch (plan.waves_per_row) {                     \
-        case 1: ASCAN_FWD(1, AL, R); break;           \
-        case 2: ASCAN_FWD(2, AL, R); break;           \
-        case 4: ASCAN_FWD(4, AL, R); break;           \
-        case 8: ASCAN_FWD(8, AL, R); break;           \
-        default: ASCAN_FWD(16, AL, R); break;         \
+#define ASCAN_FWD_W(AL, REG)                            \
+    switch (plan.waves_per_row) {                       \
+        case 1: ASCAN_FWD(1, AL, REG); break;           \
+        case 2: ASCAN_FWD(2, AL, REG); break;           \
+        case 4: ASCAN_FWD(4, AL, REG); break;           \
+        case 8: ASCAN_FWD(8, AL, REG); break;           \
+        default: ASCAN_FWD(16, AL, REG); break;         \
     }
-    if (aligned) {
-        ASCAN_FWD_W(true);
+    if (access == Access::kRegular) {
+        ASCAN_FWD_W(true, true);
+    } else if (access == Access::kVector) {
+        ASCAN_FWD_W(true, false);
     } else {
-        ASCAN_FWD_W(false);  // same geometry, element-wise memory access
+        ASCAN_FWD_W(false, false);
     }
 #undef ASCAN_FWD_W
 #undef ASCAN_FWD
@@ -898,26 +1023,31 @@ int forward_typed(const void* gates, const void* tokens, void* out, int64_t rows
 template <class Tr>
 int backward_typed(const void* gates, const void* states, const void* grad_out, void* d_gates, void* d_tokens,
                    int64_t rows, int64_t T, hipStream_t stream) {
-    constexpr int EPV = Tr::EPV;
-    constexpr int64_t SUB = (int64_t)Tuning<Tr>::UB * 64 * EPV;
-    const bool aligned = same_phase16(gates, states) && same_phase16(gates, grad_out) &&
-                         same_phase16(gates, d_gates) && same_phase16(gates, d_tokens);
-    const Plan plan = choose_plan(T, SUB, (int64_t)sizeof(typename Tr::S));
+    constexpr int64_t kElem = (int64_t)sizeof(typename Tr::S);
+    constexpr int64_t SUB = (int64_t)Tuning<Tr>::UB * 64 * Tr::EPV;    // regular kernels
+    constexpr int64_t SUBG = (int64_t)Tuning<Tr>::UBG * 64 * Tr::EPV;  // kernels with masking code
+    const bool same_phase = same_phase16(gates, states) && same_phase16(gates, grad_out) &&
+                            same_phase16(gates, d_gates) && same_phase16(gates, d_tokens);
+    Plan plan = choose_plan(T, SUB, kElem);
+    const Access access = choose_access(same_phase, gates, T, SUB * plan.waves_per_row);
+    if (access != Access::kRegular) plan = choose_plan(T, SUBG, kElem);
     const int R = plan.rows_per_block;
-#define ASCAN_BWD(WV, AL, RPB) \
-    launch_backward<Tr, WV, AL>(gates, states, grad_out, d_gates, d_tokens, rows, T, RPB, stream)
-#define ASCAN_BWD_W(AL)                               \
-    switch (plan.waves_per_row) {                     \
-        case 1: ASCAN_BWD(1, AL, R); break;           \
-        case 2: ASCAN_BWD(2, AL, R); break;           \
-        case 4: ASCAN_BWD(4, AL, R); break;           \
-        case 8: ASCAN_BWD(8, AL, R); break;           \
-        default: ASCAN_BWD(16, AL, R); break;         \
+#define ASCAN_BWD(WV, AL, REG) \
+    launch_backward<Tr, WV, AL, REG>(gates, states, grad_out, d_gates, d_tokens, rows, T, R, stream)
+#define ASCAN_BWD_W(AL, REG)                            \
+    switch (plan.waves_per_row) {                       \
+        case 1: ASCAN_BWD(1, AL, REG); break;           \
+        case 2: ASCAN_BWD(2, AL, REG); break;           \
+        case 4: ASCAN_BWD(4, AL, REG); break;           \
+        case 8: ASCAN_BWD(8, AL, REG); break;           \
+        default: ASCAN_BWD(16, AL, REG); break;         \
     }
-    if (aligned) {
-        ASCAN_BWD_W(true);
+    if (access == Access::kRegular) {
+        ASCAN_BWD_W(true, true);
+    } else if (access == Access::kVector) {
+        ASCAN_BWD_W(true, false);
     } else {
-        ASCAN_BWD_W(false);  // same geometry, element-wise memory access
+        ASCAN_BWD_W(false, false);
     }
 #undef ASCAN_BWD_W
 #undef ASCAN_BWD

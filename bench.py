@@ -16,9 +16,9 @@ timings taken inside the timed region; `cpu_baseline` times the torch tree
 scan (oracle/ref_scan.py, the restatement of the reference's ref.scan) on the
 host cores on a bounded sample of the same workload.
 
-Other workloads: --dtype {fp32,bf16,fp16,c64} --shape B D T; --sweep runs the
-(8, 1536, T) sweep, T = 4096..65536, fp32 and bf16, and writes one JSON line
-per point to the file given (the single summary line is still printed).
+Other workloads: --dtype {fp32,bf16,fp16,c64} --shape B D T.  --sweep FILE runs
+the reference's benchmark grid and --precision FILE its max-abs-error table,
+one JSON line per point into FILE (the single summary line is still printed).
 """
 
 import argparse
@@ -55,7 +55,10 @@ def parse_args():
                     help="for rocprofv3 --pmc runs: 3 plain copies of 1 GiB (torch copy_), then 3 steps "
                          "of the workload, no timing; the copy's known traffic scales the counters")
     ap.add_argument("--sweep", type=str, default=None, metavar="FILE",
-                    help="also run the (8,1536,T) fp32/bf16 sweep and write JSON lines to FILE")
+                    help="also run the reference's benchmark grid ((8,1536,T), T=128..65536, forward / "
+                         "reverse / backward / train, fp32 and bf16; complex (1,512,131072)) into FILE")
+    ap.add_argument("--precision", type=str, default=None, metavar="FILE",
+                    help="also write max-abs error vs the fp64 recurrence, T=32..65536, fp32/fp16/bf16")
     return ap.parse_args()
 
 
@@ -126,6 +129,113 @@ def run_workload(shape, dtype_name, steps, warmup):
     }
 
 
+def time_call(fn, steps, warmup):
+    """Mean milliseconds per call of fn() from HIP events on the current stream."""
+    import torch
+
+    for _ in range(warmup):
+        fn()
+    start = torch.cuda.Event(enable_timing=True)
+    stop = torch.cuda.Event(enable_timing=True)
+    torch.cuda.synchronize()
+    start.record()
+    for _ in range(steps):
+        fn()
+    stop.record()
+    torch.cuda.synchronize()
+    return start.elapsed_time(stop) / steps
+
+
+def run_sweep(path, steps, warmup):
+    """The reference's benchmark grid (tests/bench.py:14-31,100-115 of the
+    reference): (8, 1536, T) for T = 128..65536, directions forward, reverse
+    ("backward" in the reference's naming: a reverse forward scan, bench.py:75-77),
+    fused backward, and train (autograd forward + backward including output
+    allocation, bench.py:79-81; T <= 16384 as there); fp32 and bf16.  Then the
+    complex forward + backward point of tests/bench_complex.py:79-90,
+    (1, 512, 131072).  One JSON line per point."""
+    import torch
+
+    from accelerated_scan import _abi
+    from accelerated_scan.complex import scan as complex_scan
+    from accelerated_scan.warp import scan as warp_scan
+
+    device = torch.device("cuda:0")
+    with open(path, "w") as f:
+        def emit(rec):
+            f.write(json.dumps(rec) + "\n")
+            f.flush()
+
+        for dt in ("fp32", "bf16"):
+            for T in [2 ** i for i in range(7, 17)]:
+                shape = (8, 1536, T)
+                gates, tokens, grad_out = make_inputs(shape, dt, device)
+                out, d_gates, d_tokens = (torch.empty_like(tokens) for _ in range(3))
+                nbytes = tokens.numel() * tokens.element_size()
+                rec = {"dtype": dt, "shape": list(shape)}
+                ms = time_call(lambda: _abi.forward(gates, tokens, out, False), steps, warmup)
+                rec["forward_ms"], rec["forward_GBps"] = ms, 3 * nbytes / ms / 1e6
+                ms = time_call(lambda: _abi.forward(gates, tokens, out, True), steps, warmup)
+                rec["reverse_ms"], rec["reverse_GBps"] = ms, 3 * nbytes / ms / 1e6
+                _abi.forward(gates, tokens, out, False)
+                ms = time_call(lambda: _abi.backward(gates, out, grad_out, d_gates, d_tokens), steps, warmup)
+                rec["backward_ms"], rec["backward_GBps"] = ms, 5 * nbytes / ms / 1e6
+                if T <= 16384:
+                    g = gates.clone().requires_grad_(True)
+                    x = tokens.clone().requires_grad_(True)
+                    ms = time_call(lambda: torch.autograd.grad(warp_scan(g, x), (g, x), grad_out), steps, warmup)
+                    rec["train_ms"], rec["train_GBps"] = ms, 8 * nbytes / ms / 1e6
+                emit(rec)
+                del gates, tokens, grad_out, out, d_gates, d_tokens
+
+        shape = (1, 512, 131072)
+        gates, tokens, grad_out = make_inputs(shape, "c64", device)
+        out, d_gates, d_tokens = (torch.empty_like(tokens) for _ in range(3))
+        nbytes = tokens.numel() * tokens.element_size()
+
+        def both():
+            _abi.forward(gates, tokens, out, False)
+            _abi.backward(gates, out, grad_out, d_gates, d_tokens)
+
+        ms = time_call(both, steps, warmup)
+        rec = {"dtype": "c64", "shape": list(shape), "forward_backward_ms": ms,
+               "forward_backward_GBps": 8 * nbytes / ms / 1e6}
+        g = gates.clone().requires_grad_(True)
+        x = tokens.real.contiguous().requires_grad_(True)  # real inputs, as the reference's complex bench
+        ms = time_call(lambda: torch.autograd.grad(complex_scan(g, x), (g, x), grad_out), steps, warmup)
+        rec["train_real_inputs_ms"] = ms
+        emit(rec)
+
+
+def run_precision(path):
+    """Max-abs error against the fp64 recurrence for U(0,1) inputs, T = 32..65536,
+    shape (1, 512, T) -- the quantity the reference plots in max-abs-error.png
+    (README.md:60-64 of the reference).  Also reports the torch tree scan run in
+    the same storage dtype, which is what the reference's kernels are judged by."""
+    import numpy as np
+    import torch
+
+    from accelerated_scan.warp import scan_forward
+    from oracle import ref_scan, seqscan
+
+    with open(path, "w") as f:
+        for T in [2 ** i for i in range(5, 17)]:
+            gen = torch.Generator().manual_seed(3407)
+            gates32 = torch.rand(1, 512, T, generator=gen)
+            tokens32 = torch.rand(1, 512, T, generator=gen)
+            rec = {"T": T}
+            for name, dt in (("fp32", torch.float32), ("fp16", torch.float16), ("bf16", torch.bfloat16)):
+                g = gates32.to(dt)
+                x = tokens32.to(dt)
+                truth = seqscan.forward(g.float().numpy(), x.float().numpy())
+                hip = scan_forward(g.to("cuda:0"), x.to("cuda:0")).float().cpu().numpy()
+                tree = ref_scan.scan(g.to("cuda:0"), x.to("cuda:0")).float().cpu().numpy()
+                rec[f"{name}_hip_max_abs_err"] = float(np.abs(hip - truth).max())
+                rec[f"{name}_tree_scan_same_dtype_max_abs_err"] = float(np.abs(tree - truth).max())
+            f.write(json.dumps(rec) + "\n")
+            f.flush()
+
+
 def cpu_baseline(shape, dtype_name):
     """Tree scan (the reference's CPU path, restated) forward+backward on the
     host cores, on a slice of the workload's rows sized to take ~10-30 s."""
@@ -192,13 +302,9 @@ def main():
     m = run_workload(shape, args.dtype, args.steps, args.warmup)
 
     if args.sweep:
-        with open(args.sweep, "w") as f:
-            for dt in ("fp32", "bf16"):
-                for T in (4096, 8192, 16384, 32768, 65536):
-                    r = run_workload((8, 1536, T), dt, max(5, args.steps), args.warmup)
-                    r.update({"dtype": dt, "shape": [8, 1536, T]})
-                    f.write(json.dumps(r) + "\n")
-                    f.flush()
+        run_sweep(args.sweep, max(5, args.steps), args.warmup)
+    if args.precision:
+        run_precision(args.precision)
 
     dtype_field = {"fp32": "f32", "bf16": "bf16 storage, f32 arithmetic",
                    "fp16": "f16 storage, f32 arithmetic", "c64": "complex64 (f32 pairs)"}[args.dtype]
