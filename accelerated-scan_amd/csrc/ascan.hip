@@ -599,18 +599,18 @@ __global__ void __launch_bounds__(64 * kMaxWavesPerBlock)
 
     V carry = vzero<V>();
 
-    for (int64_t k = 0; k < ntiles; ++k) {
+    // Position of this wave's sub-tile in tile step k.
+    auto sub_tile_base = [&](int64_t k) {
         const int64_t tile = REV ? (ntiles - 1 - k) : k;
-        const int64_t sub_base = tile * TILE + (int64_t)(REV ? (W - 1 - w) : w) * SUB;
+        return tile * TILE + (int64_t)(REV ? (W - 1 - w) : w) * SUB;
+    };
+    // Loads the two input vectors of every block of tile step k.
+    auto load_tile = [&](int64_t k, u32x4_t (&graw)[U], u32x4_t (&traw)[U]) {
+        const int64_t sub_base = sub_tile_base(k);
         const bool full = REGULAR || (sub_base >= lo && sub_base + SUB <= hi);  // wave-uniform
-
         const Window win = make_window(lo, hi, sub_base);
-        const bool touches = win.hi > 0 && win.lo < SUB;  // wave-uniform
         const S* __restrict__ gsub = grow + sub_base;
         const S* __restrict__ tsub = trow + sub_base;
-        S* __restrict__ osub = orow + sub_base;
-
-        u32x4_t graw[U], traw[U];
         if (full) {
 #pragma unroll
             for (int j = 0; j < U; ++j) {
@@ -619,7 +619,7 @@ __global__ void __launch_bounds__(64 * kMaxWavesPerBlock)
                 traw[j] = load_raw<Tr, ALIGNED, true>(tsub, off, win, vzero<V>());
             }
         } else if constexpr (!REGULAR) {
-            if (touches) {
+            if (win.hi > 0 && win.lo < SUB) {
 #pragma unroll
                 for (int j = 0; j < U; ++j) {
                     const int off = vec_offset<U, EPV, REV>(j, lane);
@@ -634,6 +634,20 @@ __global__ void __launch_bounds__(64 * kMaxWavesPerBlock)
                 }
             }
         }
+    };
+
+    // (Issuing the loads of step k+1 before the arithmetic of step k was tried
+    // and measured no faster: the memory system is already saturated by the
+    // other workgroups.)
+    for (int64_t k = 0; k < ntiles; ++k) {
+        const int64_t sub_base = sub_tile_base(k);
+        const bool full = REGULAR || (sub_base >= lo && sub_base + SUB <= hi);  // wave-uniform
+        const Window win = make_window(lo, hi, sub_base);
+        const bool touches = win.hi > 0 && win.lo < SUB;  // wave-uniform
+        S* __restrict__ osub = orow + sub_base;
+
+        u32x4_t graw[U], traw[U];
+        load_tile(k, graw, traw);
 
         // Pass 1: fold each vector into one (A, X) pair and scan the pairs.
         V totA[U], totX[U], exA[U], exX[U];
@@ -725,21 +739,19 @@ __global__ void __launch_bounds__(64 * kMaxWavesPerBlock)
 
     V carry = vzero<V>();
 
-    for (int64_t k = 0; k < ntiles; ++k) {
+    // Position of this wave's sub-tile in tile step k (reverse time).
+    auto sub_tile_base = [&](int64_t k) {
         const int64_t tile = ntiles - 1 - k;
-        const int64_t sub_base = tile * TILE + (int64_t)(W - 1 - w) * SUB;
-        const int64_t sub_end = sub_base + SUB;
-        const bool full = REGULAR || (sub_base >= lo && sub_end <= hi);  // wave-uniform
-
+        return tile * TILE + (int64_t)(W - 1 - w) * SUB;
+    };
+    // Loads the three input vectors of every block of tile step k.
+    auto load_tile = [&](int64_t k, u32x4_t (&araw)[U], u32x4_t (&draw)[U], u32x4_t (&xraw)[U]) {
+        const int64_t sub_base = sub_tile_base(k);
+        const bool full = REGULAR || (sub_base >= lo && sub_base + SUB <= hi);  // wave-uniform
         const Window win = make_window(lo, hi, sub_base);
-        const bool touches = win.hi > 0 && win.lo < SUB;  // wave-uniform
         const S* __restrict__ asub = arow + sub_base;
         const S* __restrict__ dsub = drow + sub_base;
         const S* __restrict__ xsub = xrow + sub_base;
-        S* __restrict__ dgsub = dgrow + sub_base;
-        S* __restrict__ dtsub = dtrow + sub_base;
-
-        u32x4_t araw[U], draw[U], xraw[U];
         if (full) {
 #pragma unroll
             for (int j = 0; j < U; ++j) {
@@ -749,7 +761,7 @@ __global__ void __launch_bounds__(64 * kMaxWavesPerBlock)
                 xraw[j] = load_raw<Tr, ALIGNED, true>(xsub, off, win, vzero<V>());
             }
         } else if constexpr (!REGULAR) {
-            if (touches) {
+            if (win.hi > 0 && win.lo < SUB) {
 #pragma unroll
                 for (int j = 0; j < U; ++j) {
                     const int off = vec_offset<U, EPV, true>(j, lane);
@@ -766,6 +778,19 @@ __global__ void __launch_bounds__(64 * kMaxWavesPerBlock)
                 }
             }
         }
+    };
+
+    for (int64_t k = 0; k < ntiles; ++k) {
+        const int64_t sub_base = sub_tile_base(k);
+        const int64_t sub_end = sub_base + SUB;
+        const bool full = REGULAR || (sub_base >= lo && sub_end <= hi);  // wave-uniform
+        const Window win = make_window(lo, hi, sub_base);
+        const bool touches = win.hi > 0 && win.lo < SUB;  // wave-uniform
+        S* __restrict__ dgsub = dgrow + sub_base;
+        S* __restrict__ dtsub = dtrow + sub_base;
+
+        u32x4_t araw[U], draw[U], xraw[U];
+        load_tile(k, araw, draw, xraw);
 
         // The two elements just outside the sub-tile: gate at sub_end and x at
         // sub_base-1.  Addresses are clamped into the row so the loads are
