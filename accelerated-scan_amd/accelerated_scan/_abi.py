@@ -15,7 +15,7 @@ import torch
 ABI_VERSION = 1
 
 # ascan_dtype codes of include/ascan.h
-F32, BF16, F16, C64 = 0, 1, 2, 3
+F32, BF16, F16, C64, C64_REAL_TOKENS = 0, 1, 2, 3, 4
 
 DTYPE_CODES = {
     torch.float32: F32,
@@ -91,7 +91,15 @@ def check(status: int) -> None:
     raise RuntimeError(f"accelerated_scan: {text}")
 
 
-def dtype_code(dtype: torch.dtype) -> int:
+def dtype_code(dtype: torch.dtype, token_dtype: torch.dtype = None) -> int:
+    """ascan_dtype of a call from the dtype of gates and of tokens / d_tokens."""
+    if dtype == torch.complex64 and token_dtype == torch.float32:
+        return C64_REAL_TOKENS
+    if token_dtype is not None and token_dtype != dtype:
+        raise RuntimeError(
+            f"accelerated_scan: gates are {dtype} but tokens are {token_dtype}: expecting one dtype "
+            "(or complex64 gates with float32 tokens)"
+        )
     try:
         return DTYPE_CODES[dtype]
     except KeyError:
@@ -118,7 +126,7 @@ def forward(gates, tokens, out, reverse: bool) -> None:
     lib = _lib or load()
     seqlen = tokens.shape[-1]
     rows = tokens.numel() // seqlen if seqlen else 0
-    code = dtype_code(tokens.dtype)
+    code = dtype_code(gates.dtype, tokens.dtype)
     _launch(tokens.device, lambda stream: lib.ascan_forward(
         gates.data_ptr(), tokens.data_ptr(), out.data_ptr(), rows, seqlen, code, 1 if reverse else 0, stream))
 
@@ -128,7 +136,7 @@ def backward(gates, states, grad_out, d_gates, d_tokens) -> None:
     lib = _lib or load()
     seqlen = gates.shape[-1]
     rows = gates.numel() // seqlen if seqlen else 0
-    code = dtype_code(gates.dtype)
+    code = dtype_code(gates.dtype, d_tokens.dtype)
     _launch(gates.device, lambda stream: lib.ascan_backward(
         gates.data_ptr(), states.data_ptr(), grad_out.data_ptr(), d_gates.data_ptr(), d_tokens.data_ptr(),
         rows, seqlen, code, stream))

@@ -17,29 +17,36 @@ from . import _abi
 
 @torch.library.custom_op("accelerated_scan::scan_forward", mutates_args=())
 def scan_forward(gates: torch.Tensor, tokens: torch.Tensor, reverse: bool) -> torch.Tensor:
-    out = torch.empty_like(tokens)
+    out = torch.empty_like(gates)  # complex gates with real tokens give complex states
     _abi.forward(gates, tokens, out, reverse)
     return out
 
 
 @scan_forward.register_fake
 def _(gates, tokens, reverse):
-    return torch.empty_like(tokens)
+    return torch.empty_like(gates)
 
 
 @torch.library.custom_op("accelerated_scan::scan_backward", mutates_args=())
 def scan_backward(
-    gates: torch.Tensor, states: torch.Tensor, grad_out: torch.Tensor
+    gates: torch.Tensor, states: torch.Tensor, grad_out: torch.Tensor, real_tokens: bool
 ) -> Tuple[torch.Tensor, torch.Tensor]:
     d_gates = torch.empty_like(gates)
-    d_tokens = torch.empty_like(gates)
+    d_tokens = _empty_token_grad(gates, real_tokens)
     _abi.backward(gates, states, grad_out, d_gates, d_tokens)
     return d_gates, d_tokens
 
 
 @scan_backward.register_fake
-def _(gates, states, grad_out):
-    return torch.empty_like(gates), torch.empty_like(gates)
+def _(gates, states, grad_out, real_tokens):
+    return torch.empty_like(gates), _empty_token_grad(gates, real_tokens)
+
+
+def _empty_token_grad(gates: torch.Tensor, real_tokens: bool) -> torch.Tensor:
+    """Token gradient buffer: real when complex gates were scanned over real tokens."""
+    if real_tokens and gates.is_complex():
+        return torch.empty(gates.shape, dtype=gates.real.dtype, device=gates.device)
+    return torch.empty_like(gates)
 
 
 def capturing() -> bool:

@@ -20,17 +20,19 @@ def _require(cond: bool, what: str) -> None:
 def _launch_forward(forget, inputs, states):
     for t, name in ((forget, "forget"), (inputs, "inputs"), (states, "states")):
         _require(t.is_cuda, f"{name} to be a device tensor")
-        _require(t.dtype == torch.complex64, f"{name} to be complex64")
         _require(t.device == forget.device, f"{name} to be on the device of forget")
+    _require(forget.dtype == torch.complex64 and states.dtype == torch.complex64, "forget and states to be complex64")
+    _require(inputs.dtype in (torch.complex64, torch.float32), "inputs to be complex64 or float32")
     _abi.forward(forget, inputs, states, False)
 
 
 def _launch_backward(forget, states, d_output, d_forget, d_inputs):
-    for t, name in ((forget, "forget"), (states, "states"), (d_output, "d_output")):
+    for t, name in ((forget, "forget"), (states, "states"), (d_output, "d_output"), (d_forget, "d_forget")):
         _require(t.is_cuda, f"{name} to be a device tensor")
         _require(t.dtype == torch.complex64, f"{name} to be complex64")
         _require(t.shape == forget.shape, f"{name} to have the shape of forget")
         _require(t.device == forget.device, f"{name} to be on the device of forget")
+    _require(d_inputs.dtype in (torch.complex64, torch.float32), "d_inputs to be complex64 or float32")
     _abi.backward(forget, states, d_output, d_forget, d_inputs)
 
 
@@ -45,13 +47,12 @@ class Scan(torch.autograd.Function):
         assert forget.is_contiguous()
         assert inputs.is_contiguous()
 
-        if real_inputs:
-            inputs = torch.complex(inputs, torch.zeros_like(inputs))
-
+        # Real inputs are not promoted to a complex copy (the reference does,
+        # complex.py:168-169): the kernel reads them as (input, 0).
         if _ops.capturing():
             states = _ops.scan_forward(forget, inputs, False)
         else:
-            states = torch.empty_like(inputs)
+            states = torch.empty_like(forget)
             _launch_forward(forget, inputs, states)
 
         ctx.save_for_backward(forget, states)
@@ -66,15 +67,17 @@ class Scan(torch.autograd.Function):
         assert forget.is_contiguous()
         assert states.is_contiguous()
 
+        # For real inputs the kernel writes only the real part of the input
+        # gradient (what complex.py:217-218 keeps).
         if _ops.capturing():
-            d_forget, d_inputs = _ops.scan_backward(forget, states, d_output)
+            d_forget, d_inputs = _ops.scan_backward(forget, states, d_output, ctx.real_inputs)
         else:
             d_forget = torch.empty_like(forget)
-            d_inputs = torch.empty_like(states)
+            if ctx.real_inputs:
+                d_inputs = torch.empty(forget.shape, dtype=torch.float32, device=forget.device)
+            else:
+                d_inputs = torch.empty_like(states)
             _launch_backward(forget, states, d_output, d_forget, d_inputs)
-
-        if ctx.real_inputs:
-            d_inputs = d_inputs.real
         return d_forget, d_inputs
 
 

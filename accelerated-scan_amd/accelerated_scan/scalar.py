@@ -37,7 +37,7 @@ class Scan(torch.autograd.Function):
         assert states.is_contiguous()
 
         if _ops.capturing():
-            return _ops.scan_backward(forget, states, d_output)
+            return _ops.scan_backward(forget, states, d_output, False)
         d_forget = torch.empty_like(forget)
         d_inputs = torch.empty_like(states)
         warp.warpscan_backward(forget, states, d_output, d_forget, d_inputs)

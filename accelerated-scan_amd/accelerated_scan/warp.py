@@ -101,7 +101,7 @@ class Scan(torch.autograd.Function):
         assert gates.is_contiguous()
 
         if _ops.capturing():
-            return _ops.scan_backward(gates, states, grad_output)
+            return _ops.scan_backward(gates, states, grad_output, False)
         d_gates = torch.empty_like(gates)
         d_tokens = torch.empty_like(gates)
         warpscan_backward(gates, states, grad_output, d_gates, d_tokens)

@@ -230,14 +230,17 @@ __device__ __forceinline__ cfloat read_lane(cfloat v) {
 // EPV = elements per 16-byte vector.
 // ---------------------------------------------------------------------------
 typedef unsigned int u32x4_t __attribute__((ext_vector_type(4)));  // one 16-byte vector
+typedef unsigned int u32x2_t __attribute__((ext_vector_type(2)));
 typedef float floatx2_t __attribute__((ext_vector_type(2)));
 typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
 typedef _Float16 halfx2_t __attribute__((ext_vector_type(2)));
 
 struct TraitsF32 {
     using S = float;
+    using TokS = S;  // tokens and d_tokens are stored like everything else
     using V = float;
     static constexpr int EPV = 4;
+    static constexpr bool kRealTokens = false;
     static constexpr bool kNarrow = false;  // unpacked form is no larger than the raw vector
     static __device__ __forceinline__ void unpack(const u32x4_t& r, V (&d)[EPV]) {
         d[0] = i2f(r.x);
@@ -259,8 +262,10 @@ struct TraitsF32 {
 
 struct TraitsBF16 {
     using S = uint16_t;
+    using TokS = S;
     using V = float;
     static constexpr int EPV = 8;
+    static constexpr bool kRealTokens = false;
     static constexpr bool kNarrow = true;
     static __device__ __forceinline__ uint32_t pack2(float lo, float hi) {
         floatx2_t f;
@@ -291,8 +296,10 @@ struct TraitsBF16 {
 
 struct TraitsF16 {
     using S = uint16_t;
+    using TokS = S;
     using V = float;
     static constexpr int EPV = 8;
+    static constexpr bool kRealTokens = false;
     static constexpr bool kNarrow = true;
     static __device__ __forceinline__ uint32_t pack2(float lo, float hi) {
         floatx2_t f;
@@ -329,8 +336,10 @@ struct TraitsF16 {
 
 struct TraitsC64 {
     using S = cfloat;  // 8 bytes, interleaved (re, im)
+    using TokS = S;
     using V = cfloat;
     static constexpr int EPV = 2;
+    static constexpr bool kRealTokens = false;
     static constexpr bool kNarrow = false;
     static __device__ __forceinline__ void unpack(const u32x4_t& r, V (&d)[EPV]) {
         d[0].re = i2f(r.x);
@@ -359,6 +368,37 @@ struct TraitsC64 {
         o.y = v.im;
         *reinterpret_cast<float2*>(p) = o;
     }
+};
+
+// complex64 gates / states / gradients with real (fp32) tokens: the tokens are
+// read as (token, 0) and the token gradient keeps its real part, without a
+// complex copy of the tokens ever existing in memory
+// (accelerated_scan/complex.py:162,168-169,217-218 promote and slice instead).
+struct TraitsC64RealTokens : TraitsC64 {
+    using TokS = float;
+    static constexpr bool kRealTokens = true;
+    // two fp32 tokens (8 bytes) <-> the raw form of two complex values
+    static __device__ __forceinline__ u32x4_t tok_widen(u32x2_t r) {
+        u32x4_t o;
+        o.x = r.x;
+        o.y = 0u;
+        o.z = r.y;
+        o.w = 0u;
+        return o;
+    }
+    static __device__ __forceinline__ u32x2_t tok_narrow(const V (&s)[EPV]) {
+        u32x2_t o;
+        o.x = f2i(s[0].re);
+        o.y = f2i(s[1].re);
+        return o;
+    }
+    static __device__ __forceinline__ V tok_load1(const TokS* p) {
+        cfloat r;
+        r.re = *p;
+        r.im = 0.0f;
+        return r;
+    }
+    static __device__ __forceinline__ void tok_store1(TokS* p, V v) { *p = v.re; }
 };
 
 // ---------------------------------------------------------------------------
@@ -476,6 +516,72 @@ __device__ __forceinline__ void store_vec(typename Tr::S* __restrict__ sub, int 
     }
 }
 
+// Token-side access: identical to load_raw / store_vec unless the tokens are
+// real while the scan is complex, in which case a "vector" of EPV tokens is 8
+// bytes of fp32.
+template <class Tr, bool ALIGNED, bool FULL>
+__device__ __forceinline__ u32x4_t load_tok_raw(const typename Tr::TokS* __restrict__ sub, int off, Window win,
+                                                typename Tr::V fill) {
+    if constexpr (!Tr::kRealTokens) {
+        return load_raw<Tr, ALIGNED, FULL>(sub, off, win, fill);
+    } else {
+        constexpr int EPV = Tr::EPV;
+        if constexpr (ALIGNED) {
+            int o = off;
+            if (!FULL) {
+                const int safe = win.lo > 0 ? (win.lo / EPV) * EPV : 0;
+                o = (off + EPV > win.lo && off < win.hi) ? off : safe;
+            }
+#if ASCAN_NT_LOAD
+            u32x4_t raw = Tr::tok_widen(__builtin_nontemporal_load(reinterpret_cast<const u32x2_t*>(sub + o)));
+#else
+            u32x4_t raw = Tr::tok_widen(*reinterpret_cast<const u32x2_t*>(sub + o));
+#endif
+            if (!FULL) {
+                typename Tr::V v[EPV];
+                Tr::unpack(raw, v);
+#pragma unroll
+                for (int e = 0; e < EPV; ++e) v[e] = vselect(in_window(win, off + e), v[e], fill);
+                raw = Tr::pack(v);
+            }
+            return raw;
+        } else {
+            typename Tr::V v[EPV];
+#pragma unroll
+            for (int e = 0; e < EPV; ++e) {
+                if (FULL || in_window(win, off + e)) {
+                    v[e] = Tr::tok_load1(sub + off + e);
+                } else {
+                    v[e] = fill;
+                }
+            }
+            return Tr::pack(v);
+        }
+    }
+}
+
+template <class Tr, bool ALIGNED, bool FULL>
+__device__ __forceinline__ void store_tok_vec(typename Tr::TokS* __restrict__ sub, int off, Window win,
+                                              const typename Tr::V (&src)[Tr::EPV]) {
+    if constexpr (!Tr::kRealTokens) {
+        store_vec<Tr, ALIGNED, FULL>(sub, off, win, src);
+    } else {
+        constexpr int EPV = Tr::EPV;
+        if (ALIGNED && (FULL || (off >= win.lo && off + EPV <= win.hi))) {
+#if ASCAN_NT_STORE
+            __builtin_nontemporal_store(Tr::tok_narrow(src), reinterpret_cast<u32x2_t*>(sub + off));
+#else
+            *reinterpret_cast<u32x2_t*>(sub + off) = Tr::tok_narrow(src);
+#endif
+        } else {
+#pragma unroll
+            for (int e = 0; e < EPV; ++e) {
+                if (FULL || in_window(win, off + e)) Tr::tok_store1(sub + off + e, src[e]);
+            }
+        }
+    }
+}
+
 // Number of tiles every wave of the grid iterates over (the barrier count must
 // be the same for all waves of a workgroup).  `head` is the largest misalignment
 // of a row start, in elements, over all rows.
@@ -573,7 +679,7 @@ __device__ __forceinline__ void exchange_carries(const V (&totA)[U], const V (&t
 // ---------------------------------------------------------------------------
 template <class Tr, int W, int U, bool REV, bool ALIGNED, bool REGULAR>
 __global__ void __launch_bounds__(64 * kMaxWavesPerBlock)
-    scan_forward_kernel(const typename Tr::S* __restrict__ gates, const typename Tr::S* __restrict__ tokens,
+    scan_forward_kernel(const typename Tr::S* __restrict__ gates, const typename Tr::TokS* __restrict__ tokens,
                         typename Tr::S* __restrict__ out, int64_t rows, int64_t T) {
     using S = typename Tr::S;
     using V = typename Tr::V;
@@ -594,7 +700,7 @@ __global__ void __launch_bounds__(64 * kMaxWavesPerBlock)
     const int64_t lo = (ALIGNED && !REGULAR) ? row_lead<Tr>(gates + row * T) : 0;
     const int64_t hi = lo + T;
     const S* __restrict__ grow = gates + row * T - lo;
-    const S* __restrict__ trow = tokens + row * T - lo;
+    const typename Tr::TokS* __restrict__ trow = tokens + row * T - lo;
     S* __restrict__ orow = out + row * T - lo;
 
     V carry = vzero<V>();
@@ -610,13 +716,13 @@ __global__ void __launch_bounds__(64 * kMaxWavesPerBlock)
         const bool full = REGULAR || (sub_base >= lo && sub_base + SUB <= hi);  // wave-uniform
         const Window win = make_window(lo, hi, sub_base);
         const S* __restrict__ gsub = grow + sub_base;
-        const S* __restrict__ tsub = trow + sub_base;
+        const typename Tr::TokS* __restrict__ tsub = trow + sub_base;
         if (full) {
 #pragma unroll
             for (int j = 0; j < U; ++j) {
                 const int off = vec_offset<U, EPV, REV>(j, lane);
                 graw[j] = load_raw<Tr, ALIGNED, true>(gsub, off, win, vone<V>());
-                traw[j] = load_raw<Tr, ALIGNED, true>(tsub, off, win, vzero<V>());
+                traw[j] = load_tok_raw<Tr, ALIGNED, true>(tsub, off, win, vzero<V>());
             }
         } else if constexpr (!REGULAR) {
             if (win.hi > 0 && win.lo < SUB) {
@@ -624,7 +730,7 @@ __global__ void __launch_bounds__(64 * kMaxWavesPerBlock)
                 for (int j = 0; j < U; ++j) {
                     const int off = vec_offset<U, EPV, REV>(j, lane);
                     graw[j] = load_raw<Tr, ALIGNED, false>(gsub, off, win, vone<V>());
-                    traw[j] = load_raw<Tr, ALIGNED, false>(tsub, off, win, vzero<V>());
+                    traw[j] = load_tok_raw<Tr, ALIGNED, false>(tsub, off, win, vzero<V>());
                 }
             } else {
 #pragma unroll
@@ -712,7 +818,7 @@ template <class Tr, int W, int U, bool ALIGNED, bool REGULAR>
 __global__ void __launch_bounds__(64 * kMaxWavesPerBlock)
     scan_backward_kernel(const typename Tr::S* __restrict__ gates, const typename Tr::S* __restrict__ states,
                          const typename Tr::S* __restrict__ grad_out, typename Tr::S* __restrict__ d_gates,
-                         typename Tr::S* __restrict__ d_tokens, int64_t rows, int64_t T) {
+                         typename Tr::TokS* __restrict__ d_tokens, int64_t rows, int64_t T) {
     using S = typename Tr::S;
     using V = typename Tr::V;
     constexpr int EPV = Tr::EPV;
@@ -735,7 +841,7 @@ __global__ void __launch_bounds__(64 * kMaxWavesPerBlock)
     const S* __restrict__ xrow = states + row * T - lo;
     const S* __restrict__ drow = grad_out + row * T - lo;
     S* __restrict__ dgrow = d_gates + row * T - lo;
-    S* __restrict__ dtrow = d_tokens + row * T - lo;
+    typename Tr::TokS* __restrict__ dtrow = d_tokens + row * T - lo;
 
     V carry = vzero<V>();
 
@@ -787,7 +893,7 @@ __global__ void __launch_bounds__(64 * kMaxWavesPerBlock)
         const Window win = make_window(lo, hi, sub_base);
         const bool touches = win.hi > 0 && win.lo < SUB;  // wave-uniform
         S* __restrict__ dgsub = dgrow + sub_base;
-        S* __restrict__ dtsub = dtrow + sub_base;
+        typename Tr::TokS* __restrict__ dtsub = dtrow + sub_base;
 
         u32x4_t araw[U], draw[U], xraw[U];
         load_tile(k, araw, draw, xraw);
@@ -881,11 +987,11 @@ __global__ void __launch_bounds__(64 * kMaxWavesPerBlock)
             }
             const int off = vec_offset<U, EPV, true>(j, lane);
             if (full) {
-                store_vec<Tr, ALIGNED, true>(dtsub, off, win, dt);
+                store_tok_vec<Tr, ALIGNED, true>(dtsub, off, win, dt);
                 store_vec<Tr, ALIGNED, true>(dgsub, off, win, dg);
             } else if constexpr (!REGULAR) {
                 if (touches) {
-                    store_vec<Tr, ALIGNED, false>(dtsub, off, win, dt);
+                    store_tok_vec<Tr, ALIGNED, false>(dtsub, off, win, dt);
                     store_vec<Tr, ALIGNED, false>(dgsub, off, win, dg);
                 }
             }
@@ -908,6 +1014,7 @@ template <> struct Tuning<TraitsF32> { static constexpr int U = ASCAN_U_F32, UG 
 template <> struct Tuning<TraitsBF16> { static constexpr int U = ASCAN_U_16BIT, UG = 2, UB = ASCAN_U_BWD_16BIT, UBG = 2; };
 template <> struct Tuning<TraitsF16> { static constexpr int U = ASCAN_U_16BIT, UG = 2, UB = ASCAN_U_BWD_16BIT, UBG = 2; };
 template <> struct Tuning<TraitsC64> { static constexpr int U = ASCAN_U_C64, UG = ASCAN_U_C64, UB = ASCAN_U_BWD_C64, UBG = 2; };
+template <> struct Tuning<TraitsC64RealTokens> : Tuning<TraitsC64> {};
 
 // Launch geometry: W waves per row, R rows per workgroup (W*R <= 16).
 struct Plan {
@@ -949,10 +1056,11 @@ Plan choose_plan(int64_t T, int64_t sub, int64_t element_bytes) {
     return Plan{w, r};
 }
 
-// True when both addresses have the same offset inside a 16-byte block, i.e.
-// when 16-byte vectors of the two tensors line up row by row.
-bool same_phase16(const void* p, const void* q) {
-    return ((reinterpret_cast<uintptr_t>(p) ^ reinterpret_cast<uintptr_t>(q)) & 15u) == 0;
+// Offset of an address inside its vector, in elements: vectors of a tensor are
+// `epv` elements of `elem_bytes` bytes.  Tensors whose first elements have the
+// same lead line up vector by vector, row by row.
+int lead_of(const void* p, size_t elem_bytes, int epv) {
+    return (int)((reinterpret_cast<uintptr_t>(p) / elem_bytes) % (unsigned)epv);
 }
 
 int finish_launch() {
@@ -972,7 +1080,7 @@ void launch_forward(const void* gates, const void* tokens, void* out, int64_t ro
     const unsigned blocks = (unsigned)((rows + rows_per_block - 1) / rows_per_block);
     const unsigned threads = 64u * W * rows_per_block;
     hipLaunchKernelGGL((scan_forward_kernel<Tr, W, U, REV, ALIGNED, REGULAR>), dim3(blocks), dim3(threads), 0, stream,
-                       static_cast<const S*>(gates), static_cast<const S*>(tokens), static_cast<S*>(out), rows,
+                       static_cast<const S*>(gates), static_cast<const typename Tr::TokS*>(tokens), static_cast<S*>(out), rows,
                        T);
 }
 
@@ -985,7 +1093,8 @@ void launch_backward(const void* gates, const void* states, const void* grad_out
     const unsigned threads = 64u * W * rows_per_block;
     hipLaunchKernelGGL((scan_backward_kernel<Tr, W, U, ALIGNED, REGULAR>), dim3(blocks), dim3(threads), 0, stream,
                        static_cast<const S*>(gates), static_cast<const S*>(states),
-                       static_cast<const S*>(grad_out), static_cast<S*>(d_gates), static_cast<S*>(d_tokens),
+                       static_cast<const S*>(grad_out), static_cast<S*>(d_gates),
+                       static_cast<typename Tr::TokS*>(d_tokens),
                        rows, T);
 }
 
@@ -993,17 +1102,15 @@ void launch_backward(const void* gates, const void* states, const void* grad_out
 //   kRegular    : every row starts on a 16-byte boundary and is a whole number
 //                 of tiles long, so every sub-tile is full: the kernel carries
 //                 no masking code at all (the common case: T a power of two).
-//   kVector     : all tensors share one offset inside a 16-byte block; rows may
-//                 start anywhere and have any length.  Whole dwordx4 accesses
-//                 except where a vector straddles a row end.
-//   kElementwise: tensors at different offsets inside a 16-byte block.
+//   kVector     : all tensors share one offset inside a vector; rows may start
+//                 anywhere and have any length.  Whole-vector accesses except
+//                 where a vector straddles a row end.
+//   kElementwise: tensors at different offsets inside a vector.
 enum class Access { kRegular, kVector, kElementwise };
 
-bool is_aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
-
-Access choose_access(bool same_phase, const void* first, int64_t T, int64_t tile) {
-    if (!same_phase) return Access::kElementwise;
-    if (is_aligned16(first) && T % tile == 0) return Access::kRegular;
+Access choose_access(bool same_lead, int lead, int64_t T, int64_t tile) {
+    if (!same_lead) return Access::kElementwise;
+    if (lead == 0 && T % tile == 0) return Access::kRegular;
     return Access::kVector;
 }
 
@@ -1014,8 +1121,10 @@ int forward_typed(const void* gates, const void* tokens, void* out, int64_t rows
     constexpr int64_t SUB = (int64_t)Tuning<Tr>::U * 64 * Tr::EPV;    // regular kernels
     constexpr int64_t SUBG = (int64_t)Tuning<Tr>::UG * 64 * Tr::EPV;  // kernels with masking code
     Plan plan = choose_plan(T, SUB, kElem);
-    const Access access = choose_access(same_phase16(gates, tokens) && same_phase16(gates, out), gates, T,
-                                        SUB * plan.waves_per_row);
+    const int lead = lead_of(gates, kElem, Tr::EPV);
+    const bool same_lead = lead_of(tokens, sizeof(typename Tr::TokS), Tr::EPV) == lead &&
+                           lead_of(out, kElem, Tr::EPV) == lead;
+    const Access access = choose_access(same_lead, lead, T, SUB * plan.waves_per_row);
     if (access != Access::kRegular) plan = choose_plan(T, SUBG, kElem);
     const int R = plan.rows_per_block;
 #define ASCAN_FWD(WV, AL, REG)                                                               \
@@ -1051,10 +1160,12 @@ int backward_typed(const void* gates, const void* states, const void* grad_out, 
     constexpr int64_t kElem = (int64_t)sizeof(typename Tr::S);
     constexpr int64_t SUB = (int64_t)Tuning<Tr>::UB * 64 * Tr::EPV;    // regular kernels
     constexpr int64_t SUBG = (int64_t)Tuning<Tr>::UBG * 64 * Tr::EPV;  // kernels with masking code
-    const bool same_phase = same_phase16(gates, states) && same_phase16(gates, grad_out) &&
-                            same_phase16(gates, d_gates) && same_phase16(gates, d_tokens);
+    const int lead = lead_of(gates, kElem, Tr::EPV);
+    const bool same_lead = lead_of(states, kElem, Tr::EPV) == lead && lead_of(grad_out, kElem, Tr::EPV) == lead &&
+                           lead_of(d_gates, kElem, Tr::EPV) == lead &&
+                           lead_of(d_tokens, sizeof(typename Tr::TokS), Tr::EPV) == lead;
     Plan plan = choose_plan(T, SUB, kElem);
-    const Access access = choose_access(same_phase, gates, T, SUB * plan.waves_per_row);
+    const Access access = choose_access(same_lead, lead, T, SUB * plan.waves_per_row);
     if (access != Access::kRegular) plan = choose_plan(T, SUBG, kElem);
     const int R = plan.rows_per_block;
 #define ASCAN_BWD(WV, AL, REG) \
@@ -1085,9 +1196,13 @@ size_t element_size(int dtype) {
         case ASCAN_BF16: return 2;
         case ASCAN_F16: return 2;
         case ASCAN_C64: return 8;
+        case ASCAN_C64_REAL_TOKENS: return 8;
         default: return 0;
     }
 }
+
+// Element size of tokens / d_tokens.
+size_t token_size(int dtype) { return dtype == ASCAN_C64_REAL_TOKENS ? 4 : element_size(dtype); }
 
 bool element_aligned(const void* p, size_t es) { return (reinterpret_cast<uintptr_t>(p) % es) == 0; }
 
@@ -1105,7 +1220,7 @@ int ascan_forward(const void* gates, const void* tokens, void* out, int64_t rows
     if (rows < 0 || seqlen < 0 || rows > kMaxBlocks) return ASCAN_ERR_BAD_SHAPE;
     if (rows == 0 || seqlen == 0) return ASCAN_OK;
     if (!gates || !tokens || !out) return ASCAN_ERR_NULL_POINTER;
-    if (!element_aligned(gates, es) || !element_aligned(tokens, es) || !element_aligned(out, es))
+    if (!element_aligned(gates, es) || !element_aligned(tokens, token_size(dtype)) || !element_aligned(out, es))
         return ASCAN_ERR_MISALIGNED;
     hipStream_t s = static_cast<hipStream_t>(stream);
     const bool rev = reverse != 0;
@@ -1113,7 +1228,8 @@ int ascan_forward(const void* gates, const void* tokens, void* out, int64_t rows
         case ASCAN_F32: return forward_typed<TraitsF32>(gates, tokens, out, rows, seqlen, rev, s);
         case ASCAN_BF16: return forward_typed<TraitsBF16>(gates, tokens, out, rows, seqlen, rev, s);
         case ASCAN_F16: return forward_typed<TraitsF16>(gates, tokens, out, rows, seqlen, rev, s);
-        default: return forward_typed<TraitsC64>(gates, tokens, out, rows, seqlen, rev, s);
+        case ASCAN_C64: return forward_typed<TraitsC64>(gates, tokens, out, rows, seqlen, rev, s);
+        default: return forward_typed<TraitsC64RealTokens>(gates, tokens, out, rows, seqlen, rev, s);
     }
 }
 
@@ -1125,7 +1241,7 @@ int ascan_backward(const void* gates, const void* states, const void* grad_out, 
     if (rows == 0 || seqlen == 0) return ASCAN_OK;
     if (!gates || !states || !grad_out || !d_gates || !d_tokens) return ASCAN_ERR_NULL_POINTER;
     if (!element_aligned(gates, es) || !element_aligned(states, es) || !element_aligned(grad_out, es) ||
-        !element_aligned(d_gates, es) || !element_aligned(d_tokens, es))
+        !element_aligned(d_gates, es) || !element_aligned(d_tokens, token_size(dtype)))
         return ASCAN_ERR_MISALIGNED;
     hipStream_t s = static_cast<hipStream_t>(stream);
     switch (dtype) {
@@ -1135,8 +1251,11 @@ int ascan_backward(const void* gates, const void* states, const void* grad_out, 
             return backward_typed<TraitsBF16>(gates, states, grad_out, d_gates, d_tokens, rows, seqlen, s);
         case ASCAN_F16:
             return backward_typed<TraitsF16>(gates, states, grad_out, d_gates, d_tokens, rows, seqlen, s);
-        default:
+        case ASCAN_C64:
             return backward_typed<TraitsC64>(gates, states, grad_out, d_gates, d_tokens, rows, seqlen, s);
+        default:
+            return backward_typed<TraitsC64RealTokens>(gates, states, grad_out, d_gates, d_tokens, rows, seqlen,
+                                                       s);
     }
 }
 
@@ -1145,7 +1264,7 @@ const char* ascan_status_string(int status) {
         case ASCAN_OK: return "ok";
         case ASCAN_ERR_NULL_POINTER: return "a required buffer pointer is NULL";
         case ASCAN_ERR_BAD_SHAPE: return "rows or seqlen is negative, or rows exceeds the grid limit";
-        case ASCAN_ERR_BAD_DTYPE: return "unsupported dtype: expecting float32, bfloat16, float16 or complex64";
+        case ASCAN_ERR_BAD_DTYPE: return "unsupported dtype: expecting float32, bfloat16, float16, complex64 or complex64 with float32 tokens";
         case ASCAN_ERR_MISALIGNED: return "a buffer is not aligned to its element size";
         case ASCAN_ERR_LAUNCH: return "the HIP runtime reported a launch error";
         default: return "unknown status";

@@ -46,12 +46,20 @@ extern "C" {
 
 #define ASCAN_ABI_VERSION 1
 
-/* Element types of gates / tokens / outputs (one code for all tensors of a call). */
+/* Element types of the tensors of a call. */
 enum ascan_dtype {
     ASCAN_F32  = 0, /* float                                   (warp.cuh:388) */
     ASCAN_BF16 = 1, /* bfloat16 storage, fp32 arithmetic       (warp.cuh:384) */
     ASCAN_F16  = 2, /* IEEE half storage, fp32 arithmetic      (warp.cuh:386) */
-    ASCAN_C64  = 3  /* complex64 = interleaved (re, im) floats (complex.py:37-42) */
+    ASCAN_C64  = 3, /* complex64 = interleaved (re, im) floats (complex.py:37-42) */
+    /*
+     * complex64 gates, states, grad_out and d_gates with float tokens and
+     * d_tokens: the case complex.scan accepts by promoting real inputs to a
+     * complex copy and keeping the real part of their gradient
+     * (complex.py:162,168-169,217-218).  Here the tokens are read as
+     * (token, 0) and d_tokens receives Re g[t]; no complex copy is made.
+     */
+    ASCAN_C64_REAL_TOKENS = 4
 };
 
 /* Return codes. */

@@ -27,7 +27,14 @@ def test_opcheck_forward_and_backward_ops():
     torch.library.opcheck(_ops.scan_forward, (g, x, False))
     torch.library.opcheck(_ops.scan_forward, (g, x, True))
     states = _ops.scan_forward(g, x, False)
-    torch.library.opcheck(_ops.scan_backward, (g, states, weight))
+    torch.library.opcheck(_ops.scan_backward, (g, states, weight, False))
+    # complex gates with real tokens: complex states, real token gradient
+    gc = torch.polar(g, x)
+    sc = _ops.scan_forward(gc, x, False)
+    assert sc.dtype == torch.complex64
+    torch.library.opcheck(_ops.scan_forward, (gc, x, False))
+    torch.library.opcheck(_ops.scan_backward, (gc, sc, torch.randn_like(sc), True))
+    assert _ops.scan_backward(gc, sc, torch.randn_like(sc), True)[1].dtype == torch.float32
 
 
 @pytest.mark.parametrize("backend", ["aot_eager", "inductor"])

@@ -127,12 +127,16 @@ def test_eq_backward(seed, seqlen, dtype):
 # Every small T against the fp64 recurrence: tile, wave and vector boundaries,
 # aligned and unaligned rows, all dtypes, forward / reverse / backward.
 # ---------------------------------------------------------------------------
+C64_REAL_TOKENS = "complex64 gates, float32 tokens"  # the mixed case complex.scan accepts
+
+
 def _truth_inputs(rows, T, dtype, seed):
     gen = torch.Generator().manual_seed(seed)
-    if dtype == torch.complex64:
+    if dtype == torch.complex64 or dtype == C64_REAL_TOKENS:
         gates = torch.polar(0.5 + 0.5 * torch.rand(rows, T, generator=gen), 2 * math.pi * torch.rand(rows, T, generator=gen))
         mk = lambda: torch.complex(torch.randn(rows, T, generator=gen), torch.randn(rows, T, generator=gen))
-        return gates, mk(), mk()
+        tokens = mk() if dtype == torch.complex64 else torch.randn(rows, T, generator=gen)
+        return gates, tokens, mk()
     gates = torch.rand(rows, T, generator=gen).to(dtype)
     tokens = torch.randn(rows, T, generator=gen).to(dtype)
     grad_out = torch.randn(rows, T, generator=gen).to(dtype)
@@ -143,30 +147,25 @@ def _np32(t):
     return t.numpy() if t.dtype == torch.complex64 else t.float().numpy()
 
 
-def _check_against_truth(gates, tokens, grad_out, dtype, what=""):
-    """Runs forward, reverse and backward on the GPU for (rows, T) host tensors."""
-    from accelerated_scan import _abi
+def _tolerance(dtype):
+    if dtype in (torch.complex64, torch.float32, C64_REAL_TOKENS):
+        return dict(rtol=2e-5, atol=2e-5)
+    return dict(rtol=2 * storage_ulp[dtype], atol=2 * storage_ulp[dtype])
 
+
+def _compare_with_truth(gates, tokens, grad_out, out, rev, dg, dx, dtype, what=""):
+    """GPU results (any layout with rows*T elements) against the fp64 loops."""
     rows, T = gates.shape
-    g, x, d = (t.to(DEVICE).reshape(1, rows, T) for t in (gates, tokens, grad_out))
-    out = torch.empty_like(x)
-    rev = torch.empty_like(x)
-    _abi.forward(g, x, out, False)
-    _abi.forward(g, x, rev, True)
-    dg = torch.empty_like(x)
-    dx = torch.empty_like(x)
-    _abi.backward(g, out, d, dg, dx)
-    torch.cuda.synchronize()
-
-    if dtype == torch.complex64 or dtype == torch.float32:
-        tol = dict(rtol=2e-5, atol=2e-5)
-    else:
-        tol = dict(rtol=2 * storage_ulp[dtype], atol=2 * storage_ulp[dtype])
-    t_out = seqscan.forward(_np32(gates), _np32(tokens))
-    t_rev = seqscan.forward(_np32(gates), _np32(tokens), reverse=True)
+    tol = _tolerance(dtype)
+    tok = _np32(tokens).astype(np.complex64) if dtype == C64_REAL_TOKENS else _np32(tokens)
+    t_out = seqscan.forward(_np32(gates), tok)
+    t_rev = seqscan.forward(_np32(gates), tok, reverse=True)
     # backward consumes the states the GPU produced (already rounded to storage)
     states = out.reshape(rows, T).cpu()
     t_dg, t_dx = seqscan.backward(_np32(gates), _np32(states), _np32(grad_out))
+    if dtype == C64_REAL_TOKENS:
+        t_dx = t_dx.real  # real tokens keep the real part of their gradient
+        assert dx.dtype == torch.float32
     for name, got, want in (("out", out, t_out), ("rev", rev, t_rev), ("d_tokens", dx, t_dx), ("d_gates", dg, t_dg)):
         got = _np32(got.reshape(rows, T).cpu())
         scale = max(1.0, float(np.abs(want).max()))
@@ -175,8 +174,25 @@ def _check_against_truth(gates, tokens, grad_out, dtype, what=""):
         )
 
 
-ALL_DTYPES = [torch.float32, torch.bfloat16, torch.float16, torch.complex64]
-ALL_IDS = ["fp32", "bf16", "fp16", "c64"]
+def _check_against_truth(gates, tokens, grad_out, dtype, what=""):
+    """Runs forward, reverse and backward on the GPU for (rows, T) host tensors."""
+    from accelerated_scan import _abi
+
+    rows, T = gates.shape
+    g, x, d = (t.to(DEVICE).reshape(1, rows, T) for t in (gates, tokens, grad_out))
+    out = torch.empty_like(g)
+    rev = torch.empty_like(g)
+    _abi.forward(g, x, out, False)
+    _abi.forward(g, x, rev, True)
+    dg = torch.empty_like(g)
+    dx = torch.empty_like(x)
+    _abi.backward(g, out, d, dg, dx)
+    torch.cuda.synchronize()
+    _compare_with_truth(gates, tokens, grad_out, out, rev, dg, dx, dtype, what)
+
+
+ALL_DTYPES = [torch.float32, torch.bfloat16, torch.float16, torch.complex64, C64_REAL_TOKENS]
+ALL_IDS = ["fp32", "bf16", "fp16", "c64", "c64_real_tokens"]
 
 
 @pytest.mark.parametrize("dtype", ALL_DTYPES, ids=ALL_IDS)
@@ -237,28 +253,15 @@ def test_unaligned_base_pointer(dtype, offsets, rows, T):
 
     og, ox, oo = offsets
     g, x, d = offset_copy(gates, og), offset_copy(tokens, ox), offset_copy(grad_out, oo)
-    out, rev = offset_copy(torch.zeros_like(tokens), oo), offset_copy(torch.zeros_like(tokens), og)
-    dg, dx = offset_copy(torch.zeros_like(tokens), ox), offset_copy(torch.zeros_like(tokens), oo)
-    # guard elements just outside the views must stay untouched
-    guards = [t.storage_offset() for t in (out, dg, dx)]
+    out, rev = offset_copy(torch.zeros_like(gates), oo), offset_copy(torch.zeros_like(gates), og)
+    dg, dx = offset_copy(torch.zeros_like(gates), ox), offset_copy(torch.zeros_like(tokens), oo)
     for t in (out, rev, dg, dx):
         t.untyped_storage().fill_(0)
     _abi.forward(g, x, out, False)
     _abi.forward(g, x, rev, True)
     _abi.backward(g, out, d, dg, dx)
     torch.cuda.synchronize()
-
-    if dtype == torch.complex64 or dtype == torch.float32:
-        tol = dict(rtol=2e-5, atol=2e-5)
-    else:
-        tol = dict(rtol=2 * storage_ulp[dtype], atol=2 * storage_ulp[dtype])
-    t_out = seqscan.forward(_np32(gates), _np32(tokens))
-    t_rev = seqscan.forward(_np32(gates), _np32(tokens), reverse=True)
-    t_dg, t_dx = seqscan.backward(_np32(gates), _np32(out.reshape(rows, T).cpu()), _np32(grad_out))
-    for name, got, want in (("out", out, t_out), ("rev", rev, t_rev), ("d_tokens", dx, t_dx), ("d_gates", dg, t_dg)):
-        got = _np32(got.reshape(rows, T).cpu())
-        scale = max(1.0, float(np.abs(want).max()))
-        np.testing.assert_allclose(got, want, rtol=tol["rtol"], atol=tol["atol"] * scale, err_msg=name)
+    _compare_with_truth(gates, tokens, grad_out, out, rev, dg, dx, dtype, what="offset views")
     # nothing was written outside the row range of any output
     for t in (out, rev, dg, dx):
         k = t.storage_offset()
