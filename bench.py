@@ -37,9 +37,10 @@ HBM_PEAK_GBPS = 8000.0  # MI355X HBM3E, published peak
 
 # HBM bytes per launch of the backward kernel, from two rocprofv3 --pmc runs
 # (FETCH_SIZE x 2.000 + WRITE_SIZE x 1.000 KiB, factors from a plain copy of
-# known size; summary in profiles/scan_f32_8x1536x65536_fwd_bwd.md).
+# known size; summaries in profiles/).
 MEASURED_TRAFFIC_BYTES = {
-    ((8, 1536, 65536), "fp32"): (4756376 * 2 + 6315309) * 1024,
+    ((8, 1536, 65536), "fp32"): (4723448 * 2 + 6292029) * 1024,
+    ((8, 1536, 65536), "bf16"): (2367969 * 2 + 3146575) * 1024,
 }
 
 
