@@ -1063,8 +1063,16 @@ int lead_of(const void* p, size_t elem_bytes, int epv) {
     return (int)((reinterpret_cast<uintptr_t>(p) / elem_bytes) % (unsigned)epv);
 }
 
-int finish_launch() {
-    const hipError_t e = hipGetLastError();
+// Launches through hipLaunchKernel so that the launch's own status comes back
+// (the <<<>>> form reports through the thread's sticky last-error slot, which
+// may hold an error of the caller's).
+template <class... Args>
+hipError_t launch(void (*kernel)(Args...), unsigned blocks, unsigned threads, hipStream_t stream, Args... args) {
+    void* argv[] = {static_cast<void*>(&args)...};
+    return hipLaunchKernel(reinterpret_cast<const void*>(kernel), dim3(blocks), dim3(threads), argv, 0, stream);
+}
+
+int launch_status(hipError_t e) {
     if (e != hipSuccess) {
         g_last_hip_error = (int)e;
         return ASCAN_ERR_LAUNCH;
@@ -1073,29 +1081,28 @@ int finish_launch() {
 }
 
 template <class Tr, int W, bool REV, bool ALIGNED, bool REGULAR>
-void launch_forward(const void* gates, const void* tokens, void* out, int64_t rows, int64_t T, int rows_per_block,
-                    hipStream_t stream) {
+hipError_t launch_forward(const void* gates, const void* tokens, void* out, int64_t rows, int64_t T,
+                          int rows_per_block, hipStream_t stream) {
     using S = typename Tr::S;
+    using TokS = typename Tr::TokS;
     constexpr int U = REGULAR ? Tuning<Tr>::U : Tuning<Tr>::UG;
     const unsigned blocks = (unsigned)((rows + rows_per_block - 1) / rows_per_block);
     const unsigned threads = 64u * W * rows_per_block;
-    hipLaunchKernelGGL((scan_forward_kernel<Tr, W, U, REV, ALIGNED, REGULAR>), dim3(blocks), dim3(threads), 0, stream,
-                       static_cast<const S*>(gates), static_cast<const typename Tr::TokS*>(tokens), static_cast<S*>(out), rows,
-                       T);
+    return launch(scan_forward_kernel<Tr, W, U, REV, ALIGNED, REGULAR>, blocks, threads, stream,
+                  static_cast<const S*>(gates), static_cast<const TokS*>(tokens), static_cast<S*>(out), rows, T);
 }
 
 template <class Tr, int W, bool ALIGNED, bool REGULAR>
-void launch_backward(const void* gates, const void* states, const void* grad_out, void* d_gates,
-                     void* d_tokens, int64_t rows, int64_t T, int rows_per_block, hipStream_t stream) {
+hipError_t launch_backward(const void* gates, const void* states, const void* grad_out, void* d_gates,
+                           void* d_tokens, int64_t rows, int64_t T, int rows_per_block, hipStream_t stream) {
     using S = typename Tr::S;
+    using TokS = typename Tr::TokS;
     constexpr int U = REGULAR ? Tuning<Tr>::UB : Tuning<Tr>::UBG;
     const unsigned blocks = (unsigned)((rows + rows_per_block - 1) / rows_per_block);
     const unsigned threads = 64u * W * rows_per_block;
-    hipLaunchKernelGGL((scan_backward_kernel<Tr, W, U, ALIGNED, REGULAR>), dim3(blocks), dim3(threads), 0, stream,
-                       static_cast<const S*>(gates), static_cast<const S*>(states),
-                       static_cast<const S*>(grad_out), static_cast<S*>(d_gates),
-                       static_cast<typename Tr::TokS*>(d_tokens),
-                       rows, T);
+    return launch(scan_backward_kernel<Tr, W, U, ALIGNED, REGULAR>, blocks, threads, stream,
+                  static_cast<const S*>(gates), static_cast<const S*>(states), static_cast<const S*>(grad_out),
+                  static_cast<S*>(d_gates), static_cast<TokS*>(d_tokens), rows, T);
 }
 
 // Memory-access flavour of a launch.
@@ -1127,12 +1134,13 @@ int forward_typed(const void* gates, const void* tokens, void* out, int64_t rows
     const Access access = choose_access(same_lead, lead, T, SUB * plan.waves_per_row);
     if (access != Access::kRegular) plan = choose_plan(T, SUBG, kElem);
     const int R = plan.rows_per_block;
-#define ASCAN_FWD(WV, AL, REG)                                                               \
-    do {                                                                                     \
-        if (reverse)                                                                         \
-            launch_forward<Tr, WV, true, AL, REG>(gates, tokens, out, rows, T, R, stream);   \
-        else                                                                                 \
-            launch_forward<Tr, WV, false, AL, REG>(gates, tokens, out, rows, T, R, stream);  \
+    hipError_t err = hipSuccess;
+#define ASCAN_FWD(WV, AL, REG)                                                                     \
+    do {                                                                                           \
+        if (reverse)                                                                               \
+            err = launch_forward<Tr, WV, true, AL, REG>(gates, tokens, out, rows, T, R, stream);   \
+        else                                                                                       \
+            err = launch_forward<Tr, WV, false, AL, REG>(gates, tokens, out, rows, T, R, stream);  \
     } while (0)
 #define ASCAN_FWD_W(AL, REG)                            \
     switch (plan.waves_per_row) {                       \
@@ -1151,7 +1159,7 @@ int forward_typed(const void* gates, const void* tokens, void* out, int64_t rows
     }
 #undef ASCAN_FWD_W
 #undef ASCAN_FWD
-    return finish_launch();
+    return launch_status(err);
 }
 
 template <class Tr>
@@ -1168,8 +1176,9 @@ int backward_typed(const void* gates, const void* states, const void* grad_out, 
     const Access access = choose_access(same_lead, lead, T, SUB * plan.waves_per_row);
     if (access != Access::kRegular) plan = choose_plan(T, SUBG, kElem);
     const int R = plan.rows_per_block;
+    hipError_t err = hipSuccess;
 #define ASCAN_BWD(WV, AL, REG) \
-    launch_backward<Tr, WV, AL, REG>(gates, states, grad_out, d_gates, d_tokens, rows, T, R, stream)
+    err = launch_backward<Tr, WV, AL, REG>(gates, states, grad_out, d_gates, d_tokens, rows, T, R, stream)
 #define ASCAN_BWD_W(AL, REG)                            \
     switch (plan.waves_per_row) {                       \
         case 1: ASCAN_BWD(1, AL, REG); break;           \
@@ -1187,7 +1196,7 @@ int backward_typed(const void* gates, const void* states, const void* grad_out, 
     }
 #undef ASCAN_BWD_W
 #undef ASCAN_BWD
-    return finish_launch();
+    return launch_status(err);
 }
 
 size_t element_size(int dtype) {
