@@ -12,7 +12,7 @@ from pathlib import Path
 
 import torch
 
-ABI_VERSION = 1
+ABI_VERSION = 2
 
 # ascan_dtype codes of include/ascan.h
 F32, BF16, F16, C64, C64_REAL_TOKENS = 0, 1, 2, 3, 4
@@ -36,6 +36,20 @@ _SIGNATURES = {
         [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p,
          ctypes.c_int64, ctypes.c_int64, ctypes.c_int, ctypes.c_void_p],
     ),
+    "ascan_workspace_bytes": (ctypes.c_size_t, [ctypes.c_int64, ctypes.c_int64, ctypes.c_int]),
+    "ascan_forward_split": (
+        ctypes.c_int,
+        [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p,
+         ctypes.c_int64, ctypes.c_int64, ctypes.c_int, ctypes.c_int,
+         ctypes.c_void_p, ctypes.c_size_t, ctypes.c_void_p],
+    ),
+    "ascan_backward_split": (
+        ctypes.c_int,
+        [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p,
+         ctypes.c_int64, ctypes.c_int64, ctypes.c_int,
+         ctypes.c_void_p, ctypes.c_size_t, ctypes.c_void_p],
+    ),
+    "ascan_workspace_timeouts": (ctypes.c_uint, [ctypes.c_void_p]),
     "ascan_status_string": (ctypes.c_char_p, [ctypes.c_int]),
     "ascan_last_hip_error": (ctypes.c_int, []),
     "ascan_abi_version": (ctypes.c_int, []),
@@ -121,22 +135,52 @@ def _launch(device: torch.device, call) -> None:
         check(status)
 
 
-def forward(gates, tokens, out, reverse: bool) -> None:
-    """Enqueue ascan_forward on the current stream of the tensors' device."""
+def _workspace(lib, rows: int, seqlen: int, code: int, device: torch.device):
+    """Table for split rows (few rows, long sequences), or None.  Freed by the
+    caching allocator in stream order after the kernels that use it."""
+    nbytes = lib.ascan_workspace_bytes(rows, seqlen, code)
+    if nbytes == 0:
+        return None
+    return torch.empty(nbytes, dtype=torch.uint8, device=device)
+
+
+def forward(gates, tokens, out, reverse: bool, workspace=None) -> None:
+    """Enqueue the forward scan on the current stream of the tensors' device."""
     lib = _lib or load()
     seqlen = tokens.shape[-1]
     rows = tokens.numel() // seqlen if seqlen else 0
     code = dtype_code(gates.dtype, tokens.dtype)
-    _launch(tokens.device, lambda stream: lib.ascan_forward(
-        gates.data_ptr(), tokens.data_ptr(), out.data_ptr(), rows, seqlen, code, 1 if reverse else 0, stream))
+    if workspace is None:
+        workspace = _workspace(lib, rows, seqlen, code, tokens.device)
+    if workspace is None:
+        _launch(tokens.device, lambda stream: lib.ascan_forward(
+            gates.data_ptr(), tokens.data_ptr(), out.data_ptr(), rows, seqlen, code, 1 if reverse else 0, stream))
+    else:
+        _launch(tokens.device, lambda stream: lib.ascan_forward_split(
+            gates.data_ptr(), tokens.data_ptr(), out.data_ptr(), rows, seqlen, code, 1 if reverse else 0,
+            workspace.data_ptr(), workspace.numel(), stream))
 
 
-def backward(gates, states, grad_out, d_gates, d_tokens) -> None:
-    """Enqueue ascan_backward on the current stream of the tensors' device."""
+def backward(gates, states, grad_out, d_gates, d_tokens, workspace=None) -> None:
+    """Enqueue the fused backward scan on the current stream of the tensors' device."""
     lib = _lib or load()
     seqlen = gates.shape[-1]
     rows = gates.numel() // seqlen if seqlen else 0
     code = dtype_code(gates.dtype, d_tokens.dtype)
-    _launch(gates.device, lambda stream: lib.ascan_backward(
-        gates.data_ptr(), states.data_ptr(), grad_out.data_ptr(), d_gates.data_ptr(), d_tokens.data_ptr(),
-        rows, seqlen, code, stream))
+    if workspace is None:
+        workspace = _workspace(lib, rows, seqlen, code, gates.device)
+    if workspace is None:
+        _launch(gates.device, lambda stream: lib.ascan_backward(
+            gates.data_ptr(), states.data_ptr(), grad_out.data_ptr(), d_gates.data_ptr(), d_tokens.data_ptr(),
+            rows, seqlen, code, stream))
+    else:
+        _launch(gates.device, lambda stream: lib.ascan_backward_split(
+            gates.data_ptr(), states.data_ptr(), grad_out.data_ptr(), d_gates.data_ptr(), d_tokens.data_ptr(),
+            rows, seqlen, code, workspace.data_ptr(), workspace.numel(), stream))
+
+
+def workspace_timeouts(workspace) -> int:
+    """Waits of a finished split call that ran out (synchronises the device)."""
+    lib = _lib or load()
+    header = workspace[:64].cpu().contiguous()
+    return int(lib.ascan_workspace_timeouts(header.data_ptr()))

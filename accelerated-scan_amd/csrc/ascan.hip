@@ -672,15 +672,235 @@ __device__ __forceinline__ void exchange_carries(const V (&totA)[U], const V (&t
 }
 
 // ---------------------------------------------------------------------------
+// Split rows: several workgroups per row, for calls with too few rows to
+// occupy the machine.  Every workgroup takes ONE tile of one row; the state
+// entering the tile comes from the workgroups of the earlier tiles through a
+// small table in global memory (single pass, "decoupled look-back"):
+//   * a workgroup publishes its tile's aggregate (A, X) as soon as it has it;
+//   * it then walks back over the earlier tiles of its row, folding aggregates
+//     until it meets a tile whose inclusive state P is already published;
+//   * it publishes its own inclusive state and finishes the tile.
+// The launch has no more workgroups than the GPU can hold at once, and
+// workgroup b takes tiles b, b + G, b + 2G, ... of the row-major list of all
+// tiles, so the earliest unfinished tile is always being worked on by a resident
+// workgroup and depends only on finished ones (a ticket counter was tried
+// first: one device-wide atomic per tile costs ~0.1 us and serialises the
+// launch).  Each wait is bounded by a wall-clock limit set by the host; a wait
+// that runs out poisons the result with NaN and is counted in the header.
+// ---------------------------------------------------------------------------
+struct SplitHeader {
+    unsigned long long reserved0;
+    unsigned long long wait_limit;  // longest single wait, in s_memrealtime ticks (100 MHz)
+    unsigned int timeouts;          // waits that ran out
+    unsigned int reserved[11];
+};
+static_assert(sizeof(SplitHeader) == 64, "header is 64 bytes");
+
+// One record per (row, tile).  Every field is a 64-bit word holding an fp32
+// payload in its low half and a tag in its high half (0 = not written yet,
+// 1 = valid), written and read with single relaxed device-scope atomics: the
+// payload arrives together with its tag, so no fence (on this hardware a
+// write-back or invalidate of a whole L2) is needed on either side.
+struct alignas(64) SplitRecord {
+    unsigned long long a[2];  // aggregate gate product of the tile (re, im)
+    unsigned long long x[2];  // aggregate state of the tile from a zero start (re, im)
+    unsigned long long p[2];  // inclusive state at the end of the tile (re, im)
+    unsigned long long pad[2];
+};
+static_assert(sizeof(SplitRecord) == 64, "record is 64 bytes");
+
+constexpr unsigned long long kTagValid = 1ull << 32;
+
+__device__ __forceinline__ void publish_word(unsigned long long* word, float v) {
+    __hip_atomic_store(word, kTagValid | (unsigned long long)(unsigned int)f2i(v), __ATOMIC_RELAXED,
+                       __HIP_MEMORY_SCOPE_AGENT);
+}
+__device__ __forceinline__ unsigned long long peek_word(unsigned long long* word) {
+    return __hip_atomic_load(word, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+__device__ __forceinline__ bool word_valid(unsigned long long w) { return (w >> 32) != 0ull; }
+__device__ __forceinline__ float word_value(unsigned long long w) { return i2f((int)(unsigned int)w); }
+
+__device__ __forceinline__ void publish(unsigned long long (&dst)[2], float v) { publish_word(&dst[0], v); }
+__device__ __forceinline__ void publish(unsigned long long (&dst)[2], cfloat v) {
+    publish_word(&dst[0], v.re);
+    publish_word(&dst[1], v.im);
+}
+// Reads a field; returns false while any of its words is still unwritten.
+__device__ __forceinline__ bool peek(unsigned long long (&src)[2], float& v) {
+    const unsigned long long w = peek_word(&src[0]);
+    v = word_value(w);
+    return word_valid(w);
+}
+__device__ __forceinline__ bool peek(unsigned long long (&src)[2], cfloat& v) {
+    const unsigned long long w0 = peek_word(&src[0]);
+    const unsigned long long w1 = peek_word(&src[1]);
+    v.re = word_value(w0);
+    v.im = word_value(w1);
+    return word_valid(w0) && word_valid(w1);
+}
+__device__ __forceinline__ float poison(float) { return __builtin_nanf(""); }
+__device__ __forceinline__ cfloat poison(cfloat) { return cfloat{__builtin_nanf(""), __builtin_nanf("")}; }
+
+// Clears the table before a split launch (a kernel rather than a memset so that
+// the call can be captured into a graph).
+__global__ void split_reset_kernel(uint32_t* words, size_t nwords, unsigned long long wait_limit) {
+    const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < nwords) words[i] = 0u;
+    if (i == 0) {
+        // the limit occupies words 2 and 3 of the header
+        words[2] = (uint32_t)wait_limit;
+        words[3] = (uint32_t)(wait_limit >> 32);
+    }
+}
+
+// The records follow the header.
+__device__ __forceinline__ SplitRecord* split_records(SplitHeader* header) {
+    return reinterpret_cast<SplitRecord*>(header + 1);
+}
+
+__device__ __forceinline__ float read_lane_at(float v, int lane) {
+    return i2f(__builtin_amdgcn_readlane(f2i(v), lane));
+}
+__device__ __forceinline__ cfloat read_lane_at(cfloat v, int lane) {
+    cfloat r;
+    r.re = read_lane_at(v.re, lane);
+    r.im = read_lane_at(v.im, lane);
+    return r;
+}
+
+// State entering scan-order tile k of a row, for wave 0 of the workgroup that
+// owns the tile.  `mine` is that row's first record; records of successive
+// tiles are `stride` apart.  (tileA, tileX) is this tile's aggregate.
+//
+// The walk back is done 64 tiles at a time: lane i looks at tile k-1-i, all
+// lanes wait for their record in parallel (one memory round trip instead of one
+// per tile), then the records from the nearest inclusive state forward are
+// folded with lane reads.
+template <class V>
+__device__ __forceinline__ V split_look_back(SplitHeader* header, SplitRecord* mine, int64_t stride, int64_t k,
+                                             V tileA, V tileX, int lane) {
+    SplitRecord* rec = mine + k * stride;
+    V carry_in = vzero<V>();
+    if (k > 0) {
+        if (lane == 0) {
+            publish(rec->a, tileA);
+            publish(rec->x, tileX);
+        }
+        const unsigned long long limit = header->wait_limit;
+        V accA = vone<V>(), accX = vzero<V>();  // aggregate of the tiles nearer than the current window
+        bool done = false;
+        for (int64_t base = k - 1; base >= 0 && !done; base -= 64) {
+            const int64_t q = base - lane;
+            const bool active = q >= 0;
+            // 0 nothing seen, 1 aggregate in (A, X), 2 inclusive state in X
+            int seen = 0;
+            V A = vone<V>(), X = vzero<V>();
+            if (active) {
+                SplitRecord* prev = mine + q * stride;
+                const unsigned long long t0 = __builtin_amdgcn_s_memrealtime();
+                for (;;) {
+                    V P, Aq, Xq;
+                    if (peek(prev->p, P)) {
+                        X = P;
+                        seen = 2;
+                        break;
+                    }
+                    const bool has_a = peek(prev->a, Aq);
+                    const bool has_x = peek(prev->x, Xq);
+                    if (has_a && has_x) {
+                        A = Aq;
+                        X = Xq;
+                        seen = 1;
+                        break;
+                    }
+                    if (__builtin_amdgcn_s_memrealtime() - t0 > limit) break;
+                    __builtin_amdgcn_s_sleep(1);
+                }
+            }
+            const int n_active = base + 1 < 64 ? (int)(base + 1) : 64;
+            const unsigned long long inclusive = __ballot(active && seen == 2);
+            const unsigned long long late = __ballot(active && seen == 0);
+            // lanes [0, first) hold aggregates to fold; lane `first`, if active, holds an inclusive state
+            const int first = inclusive ? (int)__builtin_ctzll(inclusive) : n_active;
+            const unsigned long long needed = first >= 63 ? ~0ull : ((2ull << first) - 1ull);
+            if (late & needed) {
+                // a wait ran out: give up on this tile, visibly
+                if (lane == 0) atomicAdd(&header->timeouts, 1u);
+                carry_in = poison(carry_in);
+                done = true;
+            } else {
+                V wA = vone<V>(), wX = vzero<V>();  // aggregate of tiles k-1-(first-1) .. k-1 of this window
+                for (int i = first - 1; i >= 0; --i) {
+                    const V Ai = read_lane_at(A, i);
+                    const V Xi = read_lane_at(X, i);
+                    wX = vfma(wX, Ai, Xi);
+                    wA = vmul(wA, Ai);
+                }
+                // (w) o (acc): the window's tiles come before the nearer ones
+                accX = vfma(wX, accA, accX);
+                accA = vmul(wA, accA);
+                if (first < n_active) {
+                    const V P = read_lane_at(X, first);
+                    carry_in = vfma(accA, P, accX);
+                    done = true;
+                }
+            }
+        }
+        // tile 0 always publishes an inclusive state, so the walk ends there at the latest
+    }
+    if (lane == 0) publish(rec->p, vfma(tileA, carry_in, tileX));
+    return carry_in;
+}
+
+// exchange_carries for a workgroup that owns a single tile of a split row: the
+// tile carry comes from split_look_back instead of the previous loop iteration.
+template <class V, int W, int U>
+__device__ __forceinline__ void exchange_carries_split(const V (&totA)[U], const V (&totX)[U], V& c, V* slots,
+                                                       int w, int lane, SplitHeader* header, SplitRecord* mine,
+                                                       int64_t stride, int64_t k) {
+    V TA = totA[0], TX = totX[0];
+#pragma unroll
+    for (int j = 1; j < U; ++j) {
+        TX = vfma(TX, totA[j], totX[j]);
+        TA = vmul(TA, totA[j]);
+    }
+    if (lane == 0) {
+        slots[2 * w] = TA;
+        slots[2 * w + 1] = TX;
+    }
+    __syncthreads();
+    // aggregate of the waves before this one, and of the whole tile, from the identity
+    V runA = vone<V>(), runX = vzero<V>();
+    V mineA = runA, mineX = runX;
+#pragma unroll
+    for (int i = 0; i < W; ++i) {
+        const V Ai = slots[2 * i];
+        const V Xi = slots[2 * i + 1];
+        mineA = vselect(i == w, runA, mineA);
+        mineX = vselect(i == w, runX, mineX);
+        runX = vfma(runX, Ai, Xi);
+        runA = vmul(runA, Ai);
+    }
+    V* carry_slot = slots + kSlotsPerBuffer;
+    if (w == 0) {  // wave-uniform
+        const V carry_in = split_look_back(header, mine, stride, k, runA, runX, lane);
+        if (lane == 0) *carry_slot = carry_in;
+    }
+    __syncthreads();
+    c = vfma(mineA, *carry_slot, mineX);
+}
+
+// ---------------------------------------------------------------------------
 // Forward kernel (REV = false) and plain reverse scan (REV = true).
 // A workgroup holds R rows x W waves per row (R = blockDim.x / 64 / W); the
 // rows of a workgroup are adjacent in memory, so with W*R = 16 one tile step
 // of the workgroup covers one contiguous span of 16 sub-tiles.
 // ---------------------------------------------------------------------------
-template <class Tr, int W, int U, bool REV, bool ALIGNED, bool REGULAR>
+template <class Tr, int W, int U, bool REV, bool ALIGNED, bool REGULAR, bool SPLIT>
 __global__ void __launch_bounds__(64 * kMaxWavesPerBlock)
     scan_forward_kernel(const typename Tr::S* __restrict__ gates, const typename Tr::TokS* __restrict__ tokens,
-                        typename Tr::S* __restrict__ out, int64_t rows, int64_t T) {
+                        typename Tr::S* __restrict__ out, int64_t rows, int64_t T, SplitHeader* split) {
     using S = typename Tr::S;
     using V = typename Tr::V;
     constexpr int EPV = Tr::EPV;
@@ -692,9 +912,24 @@ __global__ void __launch_bounds__(64 * kMaxWavesPerBlock)
     const int head = REGULAR ? 0 : (ALIGNED ? (T % EPV == 0 ? row_lead<Tr>(gates) : EPV - 1) : 0);
     const int64_t ntiles = tiles_per_row(T, TILE, head);
     __shared__ V slots_all[W == 1 ? 1 : 2 * kSlotsPerBuffer];
+    // Split rows: a fixed set of co-resident workgroups walks over all (row,
+    // tile) pairs in order, all tiles of row 0 first; what is in flight at any
+    // time is one contiguous stretch of memory, and a workgroup only ever waits
+    // for tiles that resident workgroups are already working on.
+    const int64_t visits = SPLIT ? rows * ntiles : 1;
+    for (int64_t visit = SPLIT ? blockIdx.x : 0; visit < visits; visit += SPLIT ? gridDim.x : 1) {
     int64_t row;
     int w, slot_base;
-    if (!locate_wave<W>(rows, ntiles, row, w, slot_base)) return;  // wave-uniform
+    int64_t k_begin = 0, k_end = ntiles;
+    if constexpr (SPLIT) {
+        row = visit / ntiles;
+        k_begin = visit - row * ntiles;
+        k_end = k_begin + 1;
+        w = threadIdx.x >> 6;
+        slot_base = 0;
+    } else {
+        if (!locate_wave<W>(rows, ntiles, row, w, slot_base)) return;  // wave-uniform
+    }
     V* slots = slots_all + (W == 1 ? 0 : slot_base);
 
     const int64_t lo = (ALIGNED && !REGULAR) ? row_lead<Tr>(gates + row * T) : 0;
@@ -745,7 +980,7 @@ __global__ void __launch_bounds__(64 * kMaxWavesPerBlock)
     // (Issuing the loads of step k+1 before the arithmetic of step k was tried
     // and measured no faster: the memory system is already saturated by the
     // other workgroups.)
-    for (int64_t k = 0; k < ntiles; ++k) {
+    for (int64_t k = k_begin; k < k_end; ++k) {
         const int64_t sub_base = sub_tile_base(k);
         const bool full = REGULAR || (sub_base >= lo && sub_base + SUB <= hi);  // wave-uniform
         const Window win = make_window(lo, hi, sub_base);
@@ -779,7 +1014,11 @@ __global__ void __launch_bounds__(64 * kMaxWavesPerBlock)
         }
 
         V c;
-        exchange_carries<V, W, U>(totA, totX, carry, c, slots, (int)(k & 1), w, lane);
+        if constexpr (SPLIT) {
+            exchange_carries_split<V, W, U>(totA, totX, c, slots, w, lane, split, split_records(split) + row * ntiles, 1, k);
+        } else {
+            exchange_carries<V, W, U>(totA, totX, carry, c, slots, (int)(k & 1), w, lane);
+        }
 
         // Pass 2: the plain recurrence from the state entering each lane.
 #pragma unroll
@@ -808,17 +1047,18 @@ __global__ void __launch_bounds__(64 * kMaxWavesPerBlock)
             }
         }
     }
+    }  // visits
 }
 
 // ---------------------------------------------------------------------------
 // Fused backward kernel: reverse-time scan over gate[t+1] producing d_tokens,
 // and d_gates[t] = d_tokens[t] * conj(x[t-1]) in the same pass.
 // ---------------------------------------------------------------------------
-template <class Tr, int W, int U, bool ALIGNED, bool REGULAR>
+template <class Tr, int W, int U, bool ALIGNED, bool REGULAR, bool SPLIT>
 __global__ void __launch_bounds__(64 * kMaxWavesPerBlock)
     scan_backward_kernel(const typename Tr::S* __restrict__ gates, const typename Tr::S* __restrict__ states,
                          const typename Tr::S* __restrict__ grad_out, typename Tr::S* __restrict__ d_gates,
-                         typename Tr::TokS* __restrict__ d_tokens, int64_t rows, int64_t T) {
+                         typename Tr::TokS* __restrict__ d_tokens, int64_t rows, int64_t T, SplitHeader* split) {
     using S = typename Tr::S;
     using V = typename Tr::V;
     constexpr int EPV = Tr::EPV;
@@ -830,9 +1070,24 @@ __global__ void __launch_bounds__(64 * kMaxWavesPerBlock)
     const int head = REGULAR ? 0 : (ALIGNED ? (T % EPV == 0 ? row_lead<Tr>(gates) : EPV - 1) : 0);
     const int64_t ntiles = tiles_per_row(T, TILE, head);
     __shared__ V slots_all[W == 1 ? 1 : 2 * kSlotsPerBuffer];
+    // Split rows: a fixed set of co-resident workgroups walks over all (row,
+    // tile) pairs in order, all tiles of row 0 first; what is in flight at any
+    // time is one contiguous stretch of memory, and a workgroup only ever waits
+    // for tiles that resident workgroups are already working on.
+    const int64_t visits = SPLIT ? rows * ntiles : 1;
+    for (int64_t visit = SPLIT ? blockIdx.x : 0; visit < visits; visit += SPLIT ? gridDim.x : 1) {
     int64_t row;
     int w, slot_base;
-    if (!locate_wave<W>(rows, ntiles, row, w, slot_base)) return;  // wave-uniform
+    int64_t k_begin = 0, k_end = ntiles;
+    if constexpr (SPLIT) {
+        row = visit / ntiles;
+        k_begin = visit - row * ntiles;
+        k_end = k_begin + 1;
+        w = threadIdx.x >> 6;
+        slot_base = 0;
+    } else {
+        if (!locate_wave<W>(rows, ntiles, row, w, slot_base)) return;  // wave-uniform
+    }
     V* slots = slots_all + (W == 1 ? 0 : slot_base);
 
     const int64_t lo = (ALIGNED && !REGULAR) ? row_lead<Tr>(gates + row * T) : 0;
@@ -886,7 +1141,7 @@ __global__ void __launch_bounds__(64 * kMaxWavesPerBlock)
         }
     };
 
-    for (int64_t k = 0; k < ntiles; ++k) {
+    for (int64_t k = k_begin; k < k_end; ++k) {
         const int64_t sub_base = sub_tile_base(k);
         const int64_t sub_end = sub_base + SUB;
         const bool full = REGULAR || (sub_base >= lo && sub_end <= hi);  // wave-uniform
@@ -960,7 +1215,11 @@ __global__ void __launch_bounds__(64 * kMaxWavesPerBlock)
         }
 
         V c;
-        exchange_carries<V, W, U>(totA, totX, carry, c, slots, (int)(k & 1), w, lane);
+        if constexpr (SPLIT) {
+            exchange_carries_split<V, W, U>(totA, totX, c, slots, w, lane, split, split_records(split) + row * ntiles, 1, k);
+        } else {
+            exchange_carries<V, W, U>(totA, totX, carry, c, slots, (int)(k & 1), w, lane);
+        }
 
         // Pass 2: the plain reverse recurrence and the gate gradient.
 #pragma unroll
@@ -997,6 +1256,7 @@ __global__ void __launch_bounds__(64 * kMaxWavesPerBlock)
             }
         }
     }
+    }  // visits
 }
 
 // ---------------------------------------------------------------------------
@@ -1088,8 +1348,9 @@ hipError_t launch_forward(const void* gates, const void* tokens, void* out, int6
     constexpr int U = REGULAR ? Tuning<Tr>::U : Tuning<Tr>::UG;
     const unsigned blocks = (unsigned)((rows + rows_per_block - 1) / rows_per_block);
     const unsigned threads = 64u * W * rows_per_block;
-    return launch(scan_forward_kernel<Tr, W, U, REV, ALIGNED, REGULAR>, blocks, threads, stream,
-                  static_cast<const S*>(gates), static_cast<const TokS*>(tokens), static_cast<S*>(out), rows, T);
+    return launch(scan_forward_kernel<Tr, W, U, REV, ALIGNED, REGULAR, false>, blocks, threads, stream,
+                  static_cast<const S*>(gates), static_cast<const TokS*>(tokens), static_cast<S*>(out), rows, T,
+                  static_cast<SplitHeader*>(nullptr));
 }
 
 template <class Tr, int W, bool ALIGNED, bool REGULAR>
@@ -1100,9 +1361,124 @@ hipError_t launch_backward(const void* gates, const void* states, const void* gr
     constexpr int U = REGULAR ? Tuning<Tr>::UB : Tuning<Tr>::UBG;
     const unsigned blocks = (unsigned)((rows + rows_per_block - 1) / rows_per_block);
     const unsigned threads = 64u * W * rows_per_block;
-    return launch(scan_backward_kernel<Tr, W, U, ALIGNED, REGULAR>, blocks, threads, stream,
+    return launch(scan_backward_kernel<Tr, W, U, ALIGNED, REGULAR, false>, blocks, threads, stream,
                   static_cast<const S*>(gates), static_cast<const S*>(states), static_cast<const S*>(grad_out),
-                  static_cast<S*>(d_gates), static_cast<TokS*>(d_tokens), rows, T);
+                  static_cast<S*>(d_gates), static_cast<TokS*>(d_tokens), rows, T,
+                  static_cast<SplitHeader*>(nullptr));
+}
+
+// Caller-provided table for split rows (may be absent).
+struct Workspace {
+    void* ptr;
+    size_t bytes;
+};
+
+// Split-row policy.  A call is split when its rows alone would leave most
+// compute units without a workgroup and every row has several tiles.  Split
+// tiles are small (4 waves) so that several workgroups share a compute unit
+// and overlap each other's loads, waits and stores.
+constexpr int kSplitWaves = 4;
+constexpr int64_t kSplitMaxRowsDefault = 128;
+
+int64_t split_max_rows() {
+    static const int64_t v = [] {
+        const char* s = getenv("ASCAN_SPLIT_MAX_ROWS");
+        return s ? (int64_t)atoll(s) : kSplitMaxRowsDefault;
+    }();
+    return v;
+}
+
+// Longest single wait of a workgroup for an earlier tile, in 100 MHz ticks
+// (default 2 s; ASCAN_SPLIT_WAIT_US overrides, read once).
+unsigned long long split_wait_limit() {
+    static const unsigned long long v = [] {
+        const char* s = getenv("ASCAN_SPLIT_WAIT_US");
+        const unsigned long long us = s ? strtoull(s, nullptr, 10) : 2000000ull;
+        return us * 100ull;
+    }();
+    return v;
+}
+
+bool want_split(int64_t rows, int64_t ntiles) { return rows <= split_max_rows() && ntiles >= 8; }
+
+size_t split_bytes(int64_t rows, int64_t ntiles) {
+    return sizeof(SplitHeader) + (size_t)rows * (size_t)ntiles * sizeof(SplitRecord);
+}
+
+bool workspace_fits(const Workspace& ws, int64_t rows, int64_t ntiles) {
+    return ws.ptr != nullptr && (reinterpret_cast<uintptr_t>(ws.ptr) % alignof(SplitRecord)) == 0 &&
+           ws.bytes >= split_bytes(rows, ntiles);
+}
+
+hipError_t reset_split_table(const Workspace& ws, int64_t rows, int64_t ntiles, hipStream_t stream) {
+    const size_t nwords = split_bytes(rows, ntiles) / sizeof(uint32_t);
+    const unsigned blocks = (unsigned)((nwords + 255) / 256);
+    return launch(split_reset_kernel, blocks, 256u, stream, static_cast<uint32_t*>(ws.ptr), nwords,
+                  split_wait_limit());
+}
+
+// Number of workgroups of `kernel` (of `threads` threads, no dynamic LDS) the
+// current device holds at one time.  Queried once per kernel and device.
+template <class K>
+unsigned resident_workgroups(K kernel, int threads) {
+    int device = 0;
+    if (hipGetDevice(&device) != hipSuccess) return 0;
+    constexpr int kMaxDevices = 64;
+    static unsigned cache[kMaxDevices] = {};  // 0 = not queried yet; one array per kernel instantiation
+    if (device < 0 || device >= kMaxDevices) return 0;
+    if (cache[device] == 0) {
+        int per_cu = 0, cus = 0;
+        if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, kernel, threads, 0) != hipSuccess ||
+            hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, device) != hipSuccess ||
+            per_cu <= 0 || cus <= 0) {
+            return 0;
+        }
+        cache[device] = (unsigned)per_cu * (unsigned)cus;
+    }
+    return cache[device];
+}
+
+// Tiles per row as the kernels count them (tiles_per_row on the device).
+template <class Tr>
+int64_t host_tiles_per_row(int64_t T, int64_t tile, bool regular, int lead) {
+    const int head = regular ? 0 : (T % Tr::EPV == 0 ? lead : Tr::EPV - 1);
+    return (T + head + tile - 1) / tile;
+}
+
+template <class Tr, bool REV, bool REGULAR>
+hipError_t launch_forward_split(const void* gates, const void* tokens, void* out, int64_t rows, int64_t T,
+                                int64_t ntiles, const Workspace& ws, hipStream_t stream) {
+    using S = typename Tr::S;
+    using TokS = typename Tr::TokS;
+    constexpr int U = REGULAR ? Tuning<Tr>::U : Tuning<Tr>::UG;
+    auto kernel = scan_forward_kernel<Tr, kSplitWaves, U, REV, true, REGULAR, true>;
+    const unsigned resident = resident_workgroups(kernel, 64 * kSplitWaves);
+    if (resident == 0) return hipErrorInvalidConfiguration;
+    const hipError_t e = reset_split_table(ws, rows, ntiles, stream);
+    if (e != hipSuccess) return e;
+    const int64_t tiles = rows * ntiles;
+    return launch(kernel, (unsigned)(tiles < resident ? tiles : resident), 64u * kSplitWaves, stream,
+                  static_cast<const S*>(gates), static_cast<const TokS*>(tokens), static_cast<S*>(out), rows, T,
+                  static_cast<SplitHeader*>(ws.ptr));
+}
+
+template <class Tr, bool REGULAR>
+hipError_t launch_backward_split(const void* gates, const void* states, const void* grad_out, void* d_gates,
+                                 void* d_tokens, int64_t rows, int64_t T, int64_t ntiles, const Workspace& ws,
+                                 hipStream_t stream) {
+    using S = typename Tr::S;
+    using TokS = typename Tr::TokS;
+    constexpr int U = REGULAR ? Tuning<Tr>::UB : Tuning<Tr>::UBG;
+    auto kernel = scan_backward_kernel<Tr, kSplitWaves, U, true, REGULAR, true>;
+    const unsigned resident = resident_workgroups(kernel, 64 * kSplitWaves);
+    if (resident == 0) return hipErrorInvalidConfiguration;
+    const hipError_t e = reset_split_table(ws, rows, ntiles, stream);
+    if (e != hipSuccess) return e;
+    const int64_t tiles = rows * ntiles;
+    return launch(kernel, (unsigned)(tiles < resident ? tiles : resident), 64u * kSplitWaves, stream,
+                  static_cast<const S*>(gates), static_cast<const S*>(states), static_cast<const S*>(grad_out),
+                  static_cast<S*>(d_gates), static_cast<TokS*>(d_tokens), rows, T,
+                  static_cast<SplitHeader*>(ws.ptr));
 }
 
 // Memory-access flavour of a launch.
@@ -1123,7 +1499,7 @@ Access choose_access(bool same_lead, int lead, int64_t T, int64_t tile) {
 
 template <class Tr>
 int forward_typed(const void* gates, const void* tokens, void* out, int64_t rows, int64_t T, bool reverse,
-                  hipStream_t stream) {
+                  const Workspace& ws, hipStream_t stream) {
     constexpr int64_t kElem = (int64_t)sizeof(typename Tr::S);
     constexpr int64_t SUB = (int64_t)Tuning<Tr>::U * 64 * Tr::EPV;    // regular kernels
     constexpr int64_t SUBG = (int64_t)Tuning<Tr>::UG * 64 * Tr::EPV;  // kernels with masking code
@@ -1135,6 +1511,21 @@ int forward_typed(const void* gates, const void* tokens, void* out, int64_t rows
     if (access != Access::kRegular) plan = choose_plan(T, SUBG, kElem);
     const int R = plan.rows_per_block;
     hipError_t err = hipSuccess;
+    if (same_lead && ws.ptr != nullptr) {
+        const bool regular = lead == 0 && T % (SUB * kSplitWaves) == 0;
+        const int64_t ntiles = host_tiles_per_row<Tr>(T, (regular ? SUB : SUBG) * kSplitWaves, regular, lead);
+        if (want_split(rows, ntiles) && workspace_fits(ws, rows, ntiles)) {
+            if (regular) {
+                err = reverse ? launch_forward_split<Tr, true, true>(gates, tokens, out, rows, T, ntiles, ws, stream)
+                              : launch_forward_split<Tr, false, true>(gates, tokens, out, rows, T, ntiles, ws, stream);
+            } else {
+                err = reverse
+                          ? launch_forward_split<Tr, true, false>(gates, tokens, out, rows, T, ntiles, ws, stream)
+                          : launch_forward_split<Tr, false, false>(gates, tokens, out, rows, T, ntiles, ws, stream);
+            }
+            return launch_status(err);
+        }
+    }
 #define ASCAN_FWD(WV, AL, REG)                                                                     \
     do {                                                                                           \
         if (reverse)                                                                               \
@@ -1164,7 +1555,7 @@ int forward_typed(const void* gates, const void* tokens, void* out, int64_t rows
 
 template <class Tr>
 int backward_typed(const void* gates, const void* states, const void* grad_out, void* d_gates, void* d_tokens,
-                   int64_t rows, int64_t T, hipStream_t stream) {
+                   int64_t rows, int64_t T, const Workspace& ws, hipStream_t stream) {
     constexpr int64_t kElem = (int64_t)sizeof(typename Tr::S);
     constexpr int64_t SUB = (int64_t)Tuning<Tr>::UB * 64 * Tr::EPV;    // regular kernels
     constexpr int64_t SUBG = (int64_t)Tuning<Tr>::UBG * 64 * Tr::EPV;  // kernels with masking code
@@ -1177,6 +1568,17 @@ int backward_typed(const void* gates, const void* states, const void* grad_out, 
     if (access != Access::kRegular) plan = choose_plan(T, SUBG, kElem);
     const int R = plan.rows_per_block;
     hipError_t err = hipSuccess;
+    if (same_lead && ws.ptr != nullptr) {
+        const bool regular = lead == 0 && T % (SUB * kSplitWaves) == 0;
+        const int64_t ntiles = host_tiles_per_row<Tr>(T, (regular ? SUB : SUBG) * kSplitWaves, regular, lead);
+        if (want_split(rows, ntiles) && workspace_fits(ws, rows, ntiles)) {
+            err = regular ? launch_backward_split<Tr, true>(gates, states, grad_out, d_gates, d_tokens, rows, T,
+                                                            ntiles, ws, stream)
+                          : launch_backward_split<Tr, false>(gates, states, grad_out, d_gates, d_tokens, rows, T,
+                                                             ntiles, ws, stream);
+            return launch_status(err);
+        }
+    }
 #define ASCAN_BWD(WV, AL, REG) \
     err = launch_backward<Tr, WV, AL, REG>(gates, states, grad_out, d_gates, d_tokens, rows, T, R, stream)
 #define ASCAN_BWD_W(AL, REG)                            \
@@ -1218,12 +1620,8 @@ bool element_aligned(const void* p, size_t es) { return (reinterpret_cast<uintpt
 // Largest row count one launch can address: gridDim.x is limited to 2^31-1.
 constexpr int64_t kMaxBlocks = 2147483647LL;
 
-}  // namespace
-
-extern "C" {
-
-int ascan_forward(const void* gates, const void* tokens, void* out, int64_t rows, int64_t seqlen, int dtype,
-                  int reverse, void* stream) {
+int forward_checked(const void* gates, const void* tokens, void* out, int64_t rows, int64_t seqlen, int dtype,
+                    int reverse, const Workspace& ws, void* stream) {
     const size_t es = element_size(dtype);
     if (es == 0) return ASCAN_ERR_BAD_DTYPE;
     if (rows < 0 || seqlen < 0 || rows > kMaxBlocks) return ASCAN_ERR_BAD_SHAPE;
@@ -1234,16 +1632,16 @@ int ascan_forward(const void* gates, const void* tokens, void* out, int64_t rows
     hipStream_t s = static_cast<hipStream_t>(stream);
     const bool rev = reverse != 0;
     switch (dtype) {
-        case ASCAN_F32: return forward_typed<TraitsF32>(gates, tokens, out, rows, seqlen, rev, s);
-        case ASCAN_BF16: return forward_typed<TraitsBF16>(gates, tokens, out, rows, seqlen, rev, s);
-        case ASCAN_F16: return forward_typed<TraitsF16>(gates, tokens, out, rows, seqlen, rev, s);
-        case ASCAN_C64: return forward_typed<TraitsC64>(gates, tokens, out, rows, seqlen, rev, s);
-        default: return forward_typed<TraitsC64RealTokens>(gates, tokens, out, rows, seqlen, rev, s);
+        case ASCAN_F32: return forward_typed<TraitsF32>(gates, tokens, out, rows, seqlen, rev, ws, s);
+        case ASCAN_BF16: return forward_typed<TraitsBF16>(gates, tokens, out, rows, seqlen, rev, ws, s);
+        case ASCAN_F16: return forward_typed<TraitsF16>(gates, tokens, out, rows, seqlen, rev, ws, s);
+        case ASCAN_C64: return forward_typed<TraitsC64>(gates, tokens, out, rows, seqlen, rev, ws, s);
+        default: return forward_typed<TraitsC64RealTokens>(gates, tokens, out, rows, seqlen, rev, ws, s);
     }
 }
 
-int ascan_backward(const void* gates, const void* states, const void* grad_out, void* d_gates, void* d_tokens,
-                   int64_t rows, int64_t seqlen, int dtype, void* stream) {
+int backward_checked(const void* gates, const void* states, const void* grad_out, void* d_gates, void* d_tokens,
+                     int64_t rows, int64_t seqlen, int dtype, const Workspace& ws, void* stream) {
     const size_t es = element_size(dtype);
     if (es == 0) return ASCAN_ERR_BAD_DTYPE;
     if (rows < 0 || seqlen < 0 || rows > kMaxBlocks) return ASCAN_ERR_BAD_SHAPE;
@@ -1255,17 +1653,60 @@ int ascan_backward(const void* gates, const void* states, const void* grad_out, 
     hipStream_t s = static_cast<hipStream_t>(stream);
     switch (dtype) {
         case ASCAN_F32:
-            return backward_typed<TraitsF32>(gates, states, grad_out, d_gates, d_tokens, rows, seqlen, s);
+            return backward_typed<TraitsF32>(gates, states, grad_out, d_gates, d_tokens, rows, seqlen, ws, s);
         case ASCAN_BF16:
-            return backward_typed<TraitsBF16>(gates, states, grad_out, d_gates, d_tokens, rows, seqlen, s);
+            return backward_typed<TraitsBF16>(gates, states, grad_out, d_gates, d_tokens, rows, seqlen, ws, s);
         case ASCAN_F16:
-            return backward_typed<TraitsF16>(gates, states, grad_out, d_gates, d_tokens, rows, seqlen, s);
+            return backward_typed<TraitsF16>(gates, states, grad_out, d_gates, d_tokens, rows, seqlen, ws, s);
         case ASCAN_C64:
-            return backward_typed<TraitsC64>(gates, states, grad_out, d_gates, d_tokens, rows, seqlen, s);
+            return backward_typed<TraitsC64>(gates, states, grad_out, d_gates, d_tokens, rows, seqlen, ws, s);
         default:
             return backward_typed<TraitsC64RealTokens>(gates, states, grad_out, d_gates, d_tokens, rows, seqlen,
-                                                       s);
+                                                       ws, s);
     }
+}
+
+}  // namespace
+
+extern "C" {
+
+int ascan_forward(const void* gates, const void* tokens, void* out, int64_t rows, int64_t seqlen, int dtype,
+                  int reverse, void* stream) {
+    return forward_checked(gates, tokens, out, rows, seqlen, dtype, reverse, Workspace{nullptr, 0}, stream);
+}
+
+int ascan_backward(const void* gates, const void* states, const void* grad_out, void* d_gates, void* d_tokens,
+                   int64_t rows, int64_t seqlen, int dtype, void* stream) {
+    return backward_checked(gates, states, grad_out, d_gates, d_tokens, rows, seqlen, dtype, Workspace{nullptr, 0},
+                            stream);
+}
+
+size_t ascan_workspace_bytes(int64_t rows, int64_t seqlen, int dtype) {
+    const size_t es = element_size(dtype);
+    if (es == 0 || rows <= 0 || seqlen <= 0) return 0;
+    // the smallest split tile any kernel uses for this dtype: 4 waves x 2 blocks x 64 vectors
+    const int64_t epv = 16 / (int64_t)es;
+    const int64_t tile = (int64_t)kSplitWaves * 2 * 64 * epv;
+    const int64_t ntiles = (seqlen + epv - 1 + tile - 1) / tile;
+    if (!want_split(rows, ntiles) || rows * ntiles > 2147483647LL) return 0;
+    return split_bytes(rows, ntiles);
+}
+
+int ascan_forward_split(const void* gates, const void* tokens, void* out, int64_t rows, int64_t seqlen, int dtype,
+                        int reverse, void* workspace, size_t workspace_bytes, void* stream) {
+    return forward_checked(gates, tokens, out, rows, seqlen, dtype, reverse, Workspace{workspace, workspace_bytes},
+                           stream);
+}
+
+int ascan_backward_split(const void* gates, const void* states, const void* grad_out, void* d_gates,
+                         void* d_tokens, int64_t rows, int64_t seqlen, int dtype, void* workspace,
+                         size_t workspace_bytes, void* stream) {
+    return backward_checked(gates, states, grad_out, d_gates, d_tokens, rows, seqlen, dtype,
+                            Workspace{workspace, workspace_bytes}, stream);
+}
+
+unsigned int ascan_workspace_timeouts(const void* workspace_header_copy) {
+    return static_cast<const SplitHeader*>(workspace_header_copy)->timeouts;
 }
 
 const char* ascan_status_string(int status) {

@@ -21,7 +21,8 @@
  * Conventions
  *   - every buffer is device memory owned by the caller; the library allocates
  *     nothing, keeps no reference after the call returns and holds no mutable
- *     global state, so calls are re-entrant from any host thread;
+ *     global state, so calls are re-entrant from any host thread (the *_split
+ *     calls additionally need a caller-provided workspace per concurrent call);
  *   - work is enqueued on `stream` (a hipStream_t passed as void*, NULL = the
  *     default stream) and the call returns without synchronising;
  *   - rows are dense: row r starts at element r*seqlen; 64-bit element offsets
@@ -38,13 +39,14 @@
 #ifndef ASCAN_H_
 #define ASCAN_H_
 
+#include <stddef.h>
 #include <stdint.h>
 
 #ifdef __cplusplus
 extern "C" {
 #endif
 
-#define ASCAN_ABI_VERSION 1
+#define ASCAN_ABI_VERSION 2
 
 /* Element types of the tensors of a call. */
 enum ascan_dtype {
@@ -94,6 +96,46 @@ int ascan_backward(const void* gates, const void* states, const void* grad_out,
                    void* d_gates, void* d_tokens,
                    int64_t rows, int64_t seqlen, int dtype,
                    void* stream);
+
+/*
+ * Split rows.  With few rows (B*D up to about half the number of compute
+ * units) and long sequences the plain entry points leave most of the GPU idle:
+ * they give each row one workgroup.  The *_split entry points hand the tiles of
+ * every row to separate workgroups that pass the running state through a small
+ * table in caller-provided device memory (one pass over the data, no extra
+ * traffic).  They have no counterpart in the reference, whose kernels give one
+ * thread block to each sequence (warp.cuh:279; scalar.py:98; complex.py:174).
+ *
+ *   ascan_workspace_bytes  size of the table for a problem, or 0 when splitting
+ *                          would not help (then the *_split calls behave exactly
+ *                          like the plain ones and ignore the workspace);
+ *   workspace              device memory, 64-byte aligned, at least that many
+ *                          bytes, not shared with another call that may run at
+ *                          the same time; contents on entry do not matter (it
+ *                          is cleared by a small kernel on `stream` first) and
+ *                          it may be freed or reused once the work on `stream`
+ *                          has completed.  NULL or a too-small buffer selects
+ *                          the plain path.
+ *
+ * A workgroup waits for the workgroups of earlier tiles; tiles are handed out
+ * in order, so those are always running already.  Every wait is bounded
+ * (2 s by default); a wait that runs out writes NaN into the affected tile
+ * and is counted: copy the first 64 bytes of the workspace to the host after
+ * the stream has completed and pass them to ascan_workspace_timeouts (0 = all
+ * waits were served).
+ */
+size_t ascan_workspace_bytes(int64_t rows, int64_t seqlen, int dtype);
+
+int ascan_forward_split(const void* gates, const void* tokens, void* out,
+                        int64_t rows, int64_t seqlen, int dtype, int reverse,
+                        void* workspace, size_t workspace_bytes, void* stream);
+
+int ascan_backward_split(const void* gates, const void* states, const void* grad_out,
+                         void* d_gates, void* d_tokens,
+                         int64_t rows, int64_t seqlen, int dtype,
+                         void* workspace, size_t workspace_bytes, void* stream);
+
+unsigned int ascan_workspace_timeouts(const void* workspace_header_copy);
 
 /* Static, human-readable text for an ascan_status code. */
 const char* ascan_status_string(int status);

@@ -23,6 +23,7 @@ Tolerances
 
 import ctypes
 import math
+from pathlib import Path
 
 import numpy as np
 import pytest
@@ -33,6 +34,7 @@ from oracle import ref_scan, seqscan
 pytestmark = pytest.mark.gpu
 
 DEVICE = "cuda"
+ROOT = Path(__file__).resolve().parent.parent
 
 seeds = [3407, 4, 42, 57]
 seqlens = [2**i for i in range(5, 17)] + [16323, 8000, 33753, 127323]
@@ -570,3 +572,91 @@ def test_linearity_and_concatenation():
     tail_tokens[:, :, 0] += gates[:, :, cut] * a[:, :, cut - 1]
     tail = scan_warp(gates[:, :, cut:].contiguous(), tail_tokens.contiguous())
     torch.testing.assert_close(tail, a[:, :, cut:], atol=1e-6, rtol=1e-6)
+
+
+# ---------------------------------------------------------------------------
+# Split rows: few rows, long sequences, several workgroups per row
+# ---------------------------------------------------------------------------
+@pytest.mark.parametrize("dtype", ALL_DTYPES, ids=ALL_IDS)
+@pytest.mark.parametrize("rows,T", [(1, 1 << 20), (3, 300000), (64, 65536), (128, 32768 + 8), (5, 99999), (2, 16384 * 3)])
+def test_split_rows(dtype, rows, T):
+    """The table-passing kernels (one workgroup per tile) against the fp64 loops,
+    and no wait may have run out."""
+    from accelerated_scan import _abi
+
+    lib = _abi.load()
+    code = _abi.dtype_code(torch.complex64 if dtype == C64_REAL_TOKENS else dtype,
+                           torch.float32 if dtype == C64_REAL_TOKENS else dtype)
+    nbytes = lib.ascan_workspace_bytes(rows, T, code)
+    assert nbytes > 0, "this shape is meant to take the split path"
+    gates, tokens, grad_out = _truth_inputs(rows, T, dtype, seed=rows + T)
+    g, x, d = (t.to(DEVICE).reshape(1, rows, T) for t in (gates, tokens, grad_out))
+    out, rev, dg = (torch.empty_like(g) for _ in range(3))
+    dx = torch.empty_like(x)
+    # zeroed, because a shape the library decides not to split leaves the table untouched
+    spaces = [torch.zeros(nbytes, dtype=torch.uint8, device=DEVICE) for _ in range(3)]
+    _abi.forward(g, x, out, False, workspace=spaces[0])
+    _abi.forward(g, x, rev, True, workspace=spaces[1])
+    _abi.backward(g, out, d, dg, dx, workspace=spaces[2])
+    torch.cuda.synchronize()
+    assert [_abi.workspace_timeouts(w) for w in spaces] == [0, 0, 0]
+    _compare_with_truth(gates, tokens, grad_out, out, rev, dg, dx, dtype, what="split")
+
+
+def test_split_matches_unsplit_and_autograd_path():
+    """With and without the table the tile decomposition is the same; only the
+    association in which tile carries are folded differs (rounding-level
+    differences).  The autograd operator takes the split path on its own."""
+    from accelerated_scan import _abi
+
+    lib = _abi.load()
+    rows, T = 16, 262144
+    assert lib.ascan_workspace_bytes(rows, T, 0) > 0
+    gates, tokens, grad_out = _long_memory((1, rows, T), 11)
+    g, x, d = gates.to(DEVICE), tokens.to(DEVICE), grad_out.to(DEVICE)
+    plain, split = torch.empty_like(x), torch.empty_like(x)
+    assert lib.ascan_forward(g.data_ptr(), x.data_ptr(), plain.data_ptr(), rows, T, 0, 0, None) == 0
+    _abi.forward(g, x, split, False)
+    torch.cuda.synchronize()
+    torch.testing.assert_close(split, plain, rtol=2e-6, atol=0)
+    g.requires_grad_(True)
+    x.requires_grad_(True)
+    out = scan_warp(g, x)
+    dg, dx = torch.autograd.grad(out, (g, x), d)
+    t_out = seqscan.forward(gates.numpy(), tokens.numpy())
+    t_dg, t_dx = seqscan.backward(gates.numpy(), out.detach().cpu().numpy(), grad_out.numpy())
+    assert _rel_err(out.detach(), t_out) <= 1e-5
+    assert _rel_err(dx, t_dx) <= 1e-5
+    assert _rel_err(dg, t_dg) <= 1e-5
+
+
+def test_split_wait_limit_is_an_exit_not_a_hang():
+    """With the wait limit forced to zero from the host every workgroup still
+    finishes; tiles whose predecessor was not ready are poisoned with NaN and
+    counted.  Runs in a child process because the limit is read once per process."""
+    import os
+    import subprocess
+    import sys
+
+    code = r"""
+import sys
+sys.path[:0] = [%r, %r]
+import torch
+from accelerated_scan import _abi
+lib = _abi.load()
+rows, T = 4, 1 << 20
+g = torch.rand(1, rows, T, device="cuda")
+x = torch.rand(1, rows, T, device="cuda")
+out = torch.empty_like(x)
+ws = torch.empty(lib.ascan_workspace_bytes(rows, T, 0), dtype=torch.uint8, device="cuda")
+_abi.forward(g, x, out, False, workspace=ws)
+torch.cuda.synchronize()
+timeouts = _abi.workspace_timeouts(ws)
+nans = int(torch.isnan(out).any(dim=-1).sum())
+print("timeouts", timeouts, "rows_with_nan", nans)
+assert (timeouts == 0) == (nans == 0)
+""" % (str(ROOT), str(ROOT / "accelerated-scan_amd"))
+    env = dict(os.environ, ASCAN_SPLIT_WAIT_US="0")
+    done = subprocess.run([sys.executable, "-c", code], env=env, capture_output=True, text=True, timeout=110)
+    assert done.returncode == 0, done.stdout + done.stderr
+    assert "timeouts" in done.stdout
