@@ -68,6 +68,32 @@ def test_argument_validation_returns_codes():
     assert lib.ascan_backward(p, p, p, p + 2, p, 1, 4, 0, None) == 4
 
 
+def test_workspace_sizing_and_split_entry_validation():
+    lib = _abi.load()
+    buf = ctypes.create_string_buffer(256)
+    p = ctypes.addressof(buf)
+    # many rows, or short rows: the plain kernels are the right choice
+    assert lib.ascan_workspace_bytes(12288, 65536, 0) == 0
+    assert lib.ascan_workspace_bytes(4, 4096, 0) == 0
+    assert lib.ascan_workspace_bytes(4, 1 << 20, 9) == 0  # unknown dtype
+    assert lib.ascan_workspace_bytes(-1, 1 << 20, 0) == 0
+    # few long rows: header (64 bytes) + one 64-byte record per (row, smallest tile)
+    nbytes = lib.ascan_workspace_bytes(4, 1 << 20, 0)
+    assert nbytes == 64 + 4 * ((1 << 20) // 2048 + 1) * 64
+    assert lib.ascan_workspace_bytes(4, 1 << 20, 1) < nbytes  # 16-bit tiles hold more elements
+    # the split entry points validate like the plain ones, before touching the GPU
+    assert lib.ascan_forward_split(p, p, p, 1, 4, 7, 0, None, 0, None) == 3
+    assert lib.ascan_forward_split(None, p, p, 1, 4, 0, 0, None, 0, None) == 1
+    assert lib.ascan_forward_split(p, p, p, -1, 4, 0, 0, None, 0, None) == 2
+    assert lib.ascan_forward_split(None, None, None, 0, 4, 0, 0, None, 0, None) == 0
+    assert lib.ascan_backward_split(p, p, p, p, p + 2, 1, 4, 0, None, 0, None) == 4
+    assert lib.ascan_backward_split(p, p, p, p, None, 1, 4, 0, None, 0, None) == 1
+    # the header accessor reads the count of waits that ran out from a host copy
+    header = (ctypes.c_uint32 * 16)()
+    header[4] = 3
+    assert lib.ascan_workspace_timeouts(ctypes.addressof(header)) == 3
+
+
 def test_status_becomes_runtime_error():
     with pytest.raises(RuntimeError, match="unsupported dtype"):
         _abi.check(3)
