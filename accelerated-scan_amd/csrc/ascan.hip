@@ -12,13 +12,14 @@
 //   * A row is cut into tiles; inside a tile every wave owns a contiguous
 //     sub-tile of U*64 16-byte vectors.  Lane l of the wave loads vector
 //     j*64+l of the sub-tile (j = 0..U-1), so each load instruction of the
-//     wave covers one contiguous KiB.
+//     wave covers one contiguous KiB.  Loads and stores carry the nontemporal
+//     hint: nothing is read twice.
 //   * Each lane folds its vector into one (A, X) pair, A = product of gates,
 //     X = local scan end value.  The 64 pairs are scanned with 6 DPP steps
 //     (row_shr 1,2,4,8, row_bcast 15, row_bcast 31): no LDS, no barrier.
 //   * The carry entering a block is a wave-uniform value; it is chained over
-//     the U blocks and over the tiles of the row in registers.  When several
-//     waves share a row (few rows, long T) their sub-tile totals go through a
+//     the U blocks and over the tiles of the row in registers.  A row gets up
+//     to 16 waves (one per 4 KiB of row); their sub-tile totals go through a
 //     double-buffered LDS slot array, one barrier per tile.
 //   * Every output element is then recomputed by the plain recurrence from the
 //     state entering its lane, so the per-element arithmetic is the sequential
@@ -28,6 +29,9 @@
 //     applies.  The backward pass gets gate[t+1] and x[t-1] from the vectors
 //     it already holds plus one-lane DPP shifts; only the two elements just
 //     outside a wave's sub-tile are loaded separately.
+//   * Calls with few rows and long sequences run the same kernels in a second
+//     mode in which the tiles of a row are spread over many workgroups that
+//     pass the running state through a table in global memory.
 //
 // All arithmetic is fp32 with fused multiply-add.
 
@@ -36,35 +40,6 @@
 #include <stdlib.h>
 
 #include "ascan.h"
-
-#ifndef ASCAN_USE_DPP
-#define ASCAN_USE_DPP 1
-#endif
-// Build-time tuning knobs (defaults are the measured best).
-#ifndef ASCAN_NT_LOAD
-#define ASCAN_NT_LOAD 1
-#endif
-#ifndef ASCAN_NT_STORE
-#define ASCAN_NT_STORE 1
-#endif
-#ifndef ASCAN_U_BWD_F32
-#define ASCAN_U_BWD_F32 ASCAN_U_F32
-#endif
-#ifndef ASCAN_U_F32
-#define ASCAN_U_F32 4
-#endif
-#ifndef ASCAN_U_16BIT
-#define ASCAN_U_16BIT 4
-#endif
-#ifndef ASCAN_U_BWD_16BIT
-#define ASCAN_U_BWD_16BIT 4
-#endif
-#ifndef ASCAN_U_C64
-#define ASCAN_U_C64 4
-#endif
-#ifndef ASCAN_U_BWD_C64
-#define ASCAN_U_BWD_C64 2
-#endif
 
 namespace {
 
@@ -120,7 +95,6 @@ __device__ __forceinline__ cfloat vselect(bool c, cfloat a, cfloat b) {
 __device__ __forceinline__ int f2i(float x) { return __builtin_bit_cast(int, x); }
 __device__ __forceinline__ float i2f(int x) { return __builtin_bit_cast(float, x); }
 
-#if ASCAN_USE_DPP
 // DPP control words (GFX9 encoding).
 constexpr int kRowShr1 = 0x111, kRowShr2 = 0x112, kRowShr4 = 0x114, kRowShr8 = 0x118;
 constexpr int kWaveShl1 = 0x130, kWaveShr1 = 0x138;
@@ -151,9 +125,6 @@ __device__ __forceinline__ void scan_step(V& A, V& X) {
 // Inclusive scan of the 64 (A, X) pairs of a wave, ascending lane order.
 template <class V>
 __device__ __forceinline__ void wave_scan_inclusive(V& A, V& X) {
-#ifdef ASCAN_EXPERIMENT_NOSCAN
-    return;
-#endif
     scan_step<kRowShr1, 0xF>(A, X);
     scan_step<kRowShr2, 0xF>(A, X);
     scan_step<kRowShr4, 0xF>(A, X);
@@ -172,46 +143,6 @@ template <class V>
 __device__ __forceinline__ V shift_down1(V v, V edge) {
     return dpp_move<kWaveShl1, 0xF>(edge, v);
 }
-#else
-// Portable variant of the same primitives through ds_bpermute.
-__device__ __forceinline__ float shfl_up_f(float v, int d) { return __shfl_up(v, d, 64); }
-__device__ __forceinline__ cfloat shfl_up_f(cfloat v, int d) {
-    cfloat r;
-    r.re = __shfl_up(v.re, d, 64);
-    r.im = __shfl_up(v.im, d, 64);
-    return r;
-}
-__device__ __forceinline__ float shfl_down_f(float v, int d) { return __shfl_down(v, d, 64); }
-__device__ __forceinline__ cfloat shfl_down_f(cfloat v, int d) {
-    cfloat r;
-    r.re = __shfl_down(v.re, d, 64);
-    r.im = __shfl_down(v.im, d, 64);
-    return r;
-}
-template <class V>
-__device__ __forceinline__ void wave_scan_inclusive(V& A, V& X) {
-    const int lane = threadIdx.x & 63;
-#pragma unroll
-    for (int d = 1; d < 64; d *= 2) {
-        V Ap = shfl_up_f(A, d);
-        V Xp = shfl_up_f(X, d);
-        Ap = vselect(lane >= d, Ap, vone<V>());
-        Xp = vselect(lane >= d, Xp, vzero<V>());
-        X = vfma(Xp, A, X);
-        A = vmul(Ap, A);
-    }
-}
-template <class V>
-__device__ __forceinline__ V shift_up1(V v, V edge) {
-    const int lane = threadIdx.x & 63;
-    return vselect(lane >= 1, shfl_up_f(v, 1), edge);
-}
-template <class V>
-__device__ __forceinline__ V shift_down1(V v, V edge) {
-    const int lane = threadIdx.x & 63;
-    return vselect(lane < 63, shfl_down_f(v, 1), edge);
-}
-#endif
 
 template <int LANE>
 __device__ __forceinline__ float read_lane(float v) {
@@ -450,11 +381,7 @@ __device__ __forceinline__ u32x4_t load_raw(const typename Tr::S* __restrict__ s
             const int safe = win.lo > 0 ? (win.lo / EPV) * EPV : 0;
             o = (off + EPV > win.lo && off < win.hi) ? off : safe;
         }
-#if ASCAN_NT_LOAD
         u32x4_t raw = __builtin_nontemporal_load(reinterpret_cast<const u32x4_t*>(sub + o));
-#else
-        u32x4_t raw = *reinterpret_cast<const u32x4_t*>(sub + o);
-#endif
         if (!FULL) {
             typename Tr::V v[EPV];
             Tr::unpack(raw, v);
@@ -503,11 +430,7 @@ __device__ __forceinline__ void store_vec(typename Tr::S* __restrict__ sub, int 
                                           const typename Tr::V (&src)[Tr::EPV]) {
     constexpr int EPV = Tr::EPV;
     if (ALIGNED && (FULL || (off >= win.lo && off + EPV <= win.hi))) {
-#if ASCAN_NT_STORE
         __builtin_nontemporal_store(Tr::pack(src), reinterpret_cast<u32x4_t*>(sub + off));
-#else
-        *reinterpret_cast<u32x4_t*>(sub + off) = Tr::pack(src);
-#endif
     } else {
 #pragma unroll
         for (int e = 0; e < EPV; ++e) {
@@ -532,11 +455,7 @@ __device__ __forceinline__ u32x4_t load_tok_raw(const typename Tr::TokS* __restr
                 const int safe = win.lo > 0 ? (win.lo / EPV) * EPV : 0;
                 o = (off + EPV > win.lo && off < win.hi) ? off : safe;
             }
-#if ASCAN_NT_LOAD
             u32x4_t raw = Tr::tok_widen(__builtin_nontemporal_load(reinterpret_cast<const u32x2_t*>(sub + o)));
-#else
-            u32x4_t raw = Tr::tok_widen(*reinterpret_cast<const u32x2_t*>(sub + o));
-#endif
             if (!FULL) {
                 typename Tr::V v[EPV];
                 Tr::unpack(raw, v);
@@ -568,11 +487,7 @@ __device__ __forceinline__ void store_tok_vec(typename Tr::TokS* __restrict__ su
     } else {
         constexpr int EPV = Tr::EPV;
         if (ALIGNED && (FULL || (off >= win.lo && off + EPV <= win.hi))) {
-#if ASCAN_NT_STORE
             __builtin_nontemporal_store(Tr::tok_narrow(src), reinterpret_cast<u32x2_t*>(sub + off));
-#else
-            *reinterpret_cast<u32x2_t*>(sub + off) = Tr::tok_narrow(src);
-#endif
         } else {
 #pragma unroll
             for (int e = 0; e < EPV; ++e) {
@@ -1264,16 +1179,17 @@ __global__ void __launch_bounds__(64 * kMaxWavesPerBlock)
 // ---------------------------------------------------------------------------
 thread_local int g_last_hip_error = 0;
 
-// Blocks per sub-tile by dtype, forward (U) and backward (UB).  Forward
-// sub-tiles are 4 KiB of each tensor; the backward kernel holds three input
-// tensors in registers and takes half of that where 4 KiB would spill.
+// Blocks (64 vectors = 1 KiB of a tensor each) per wave and tile step:
+//   U / UB    forward / backward kernels of regular shapes: 4 KiB of each
+//             tensor per wave, except the complex backward kernel (its three
+//             inputs plus complex temporaries would spill);
+//   UG / UBG  the same for the kernels that carry masking code (rows of
+//             arbitrary start and length), which need registers for the masks.
 template <class Tr> struct Tuning;
-// UG and UBG are the values for the kernels that carry masking code (rows of
-// arbitrary start and length), which need registers for the masks.
-template <> struct Tuning<TraitsF32> { static constexpr int U = ASCAN_U_F32, UG = ASCAN_U_F32, UB = ASCAN_U_BWD_F32, UBG = 2; };
-template <> struct Tuning<TraitsBF16> { static constexpr int U = ASCAN_U_16BIT, UG = 2, UB = ASCAN_U_BWD_16BIT, UBG = 2; };
-template <> struct Tuning<TraitsF16> { static constexpr int U = ASCAN_U_16BIT, UG = 2, UB = ASCAN_U_BWD_16BIT, UBG = 2; };
-template <> struct Tuning<TraitsC64> { static constexpr int U = ASCAN_U_C64, UG = ASCAN_U_C64, UB = ASCAN_U_BWD_C64, UBG = 2; };
+template <> struct Tuning<TraitsF32> { static constexpr int U = 4, UG = 4, UB = 4, UBG = 2; };
+template <> struct Tuning<TraitsBF16> { static constexpr int U = 4, UG = 2, UB = 4, UBG = 2; };
+template <> struct Tuning<TraitsF16> { static constexpr int U = 4, UG = 2, UB = 4, UBG = 2; };
+template <> struct Tuning<TraitsC64> { static constexpr int U = 4, UG = 4, UB = 2, UBG = 2; };
 template <> struct Tuning<TraitsC64RealTokens> : Tuning<TraitsC64> {};
 
 // Launch geometry: W waves per row, R rows per workgroup (W*R <= 16).

@@ -660,3 +660,49 @@ assert (timeouts == 0) == (nans == 0)
     done = subprocess.run([sys.executable, "-c", code], env=env, capture_output=True, text=True, timeout=110)
     assert done.returncode == 0, done.stdout + done.stderr
     assert "timeouts" in done.stdout
+
+
+# ---------------------------------------------------------------------------
+# Seeded random shapes, dtypes and storage offsets against the fp64 loops
+# ---------------------------------------------------------------------------
+def _random_cases(n, seed):
+    rng = np.random.RandomState(seed)
+    cases = []
+    for i in range(n):
+        dtype_index = int(rng.randint(len(ALL_DTYPES)))
+        rows = int(np.exp(rng.uniform(0, np.log(3000)))) if rng.rand() < 0.7 else int(rng.randint(1, 9))
+        max_T = max(2, min(200000, 6_000_000 // rows))
+        T = int(np.exp(rng.uniform(0, np.log(max_T))))
+        same = rng.rand() < 0.7
+        k = int(rng.randint(0, 4))
+        offsets = (k, k, k, k, k, k, k) if same else tuple(int(v) for v in rng.randint(0, 4, size=7))
+        cases.append((i, dtype_index, rows, T, offsets))
+    return cases
+
+
+@pytest.mark.parametrize("case", _random_cases(80, seed=20240607), ids=lambda c: f"{c[0]}-{ALL_IDS[c[1]]}-{c[2]}x{c[3]}")
+def test_random_shapes_and_offsets(case):
+    from accelerated_scan import _abi
+
+    _, dtype_index, rows, T, offsets = case
+    dtype = ALL_DTYPES[dtype_index]
+    gates, tokens, grad_out = _truth_inputs(rows, T, dtype, seed=rows * 7919 + T)
+
+    def offset_copy(t, k):
+        flat = torch.zeros(rows * T + 4, dtype=t.dtype, device=DEVICE)
+        view = flat[k:k + rows * T].view(1, rows, T)
+        view.copy_(t.reshape(1, rows, T))
+        return view
+
+    g, x, d = offset_copy(gates, offsets[0]), offset_copy(tokens, offsets[1]), offset_copy(grad_out, offsets[2])
+    out, rev = offset_copy(torch.zeros_like(gates), offsets[3]), offset_copy(torch.zeros_like(gates), offsets[4])
+    dg, dx = offset_copy(torch.zeros_like(gates), offsets[5]), offset_copy(torch.zeros_like(tokens), offsets[6])
+    _abi.forward(g, x, out, False)
+    _abi.forward(g, x, rev, True)
+    _abi.backward(g, out, d, dg, dx)
+    torch.cuda.synchronize()
+    _compare_with_truth(gates, tokens, grad_out, out, rev, dg, dx, dtype, what=f"random case {case}")
+    for t in (out, rev, dg, dx):
+        k = t.storage_offset()
+        whole = torch.empty(0, dtype=t.dtype, device=DEVICE).set_(t.untyped_storage())
+        assert whole[:k].abs().sum().item() == 0 and whole[k + rows * T:].abs().sum().item() == 0
