@@ -39,6 +39,8 @@
 #include <stdint.h>
 #include <stdlib.h>
 
+#include <type_traits>
+
 #include "ascan.h"
 
 namespace {
@@ -860,50 +862,34 @@ __global__ void __launch_bounds__(64 * kMaxWavesPerBlock)
         const int64_t tile = REV ? (ntiles - 1 - k) : k;
         return tile * TILE + (int64_t)(REV ? (W - 1 - w) : w) * SUB;
     };
-    // Loads the two input vectors of every block of tile step k.
-    auto load_tile = [&](int64_t k, u32x4_t (&graw)[U], u32x4_t (&traw)[U]) {
+    // One tile step of this wave.  FULL (a compile-time flag) says that the
+    // wave's sub-tile lies entirely inside the row: that copy of the body has no
+    // masking code.  The other copy serves the (at most two) ragged tiles of a
+    // row; it exists only in the kernels for arbitrary row starts and lengths.
+    auto tile_step = [&](int64_t k, auto full_tag) {
+        constexpr bool FULL = decltype(full_tag)::value;
         const int64_t sub_base = sub_tile_base(k);
-        const bool full = REGULAR || (sub_base >= lo && sub_base + SUB <= hi);  // wave-uniform
         const Window win = make_window(lo, hi, sub_base);
+        const bool touches = FULL || (win.hi > 0 && win.lo < SUB);  // wave-uniform
         const S* __restrict__ gsub = grow + sub_base;
         const typename Tr::TokS* __restrict__ tsub = trow + sub_base;
-        if (full) {
-#pragma unroll
-            for (int j = 0; j < U; ++j) {
-                const int off = vec_offset<U, EPV, REV>(j, lane);
-                graw[j] = load_raw<Tr, ALIGNED, true>(gsub, off, win, vone<V>());
-                traw[j] = load_tok_raw<Tr, ALIGNED, true>(tsub, off, win, vzero<V>());
-            }
-        } else if constexpr (!REGULAR) {
-            if (win.hi > 0 && win.lo < SUB) {
-#pragma unroll
-                for (int j = 0; j < U; ++j) {
-                    const int off = vec_offset<U, EPV, REV>(j, lane);
-                    graw[j] = load_raw<Tr, ALIGNED, false>(gsub, off, win, vone<V>());
-                    traw[j] = load_tok_raw<Tr, ALIGNED, false>(tsub, off, win, vzero<V>());
-                }
-            } else {
-#pragma unroll
-                for (int j = 0; j < U; ++j) {
-                    graw[j] = fill_raw<Tr>(vone<V>());
-                    traw[j] = fill_raw<Tr>(vzero<V>());
-                }
-            }
-        }
-    };
-
-    // (Issuing the loads of step k+1 before the arithmetic of step k was tried
-    // and measured no faster: the memory system is already saturated by the
-    // other workgroups.)
-    for (int64_t k = k_begin; k < k_end; ++k) {
-        const int64_t sub_base = sub_tile_base(k);
-        const bool full = REGULAR || (sub_base >= lo && sub_base + SUB <= hi);  // wave-uniform
-        const Window win = make_window(lo, hi, sub_base);
-        const bool touches = win.hi > 0 && win.lo < SUB;  // wave-uniform
         S* __restrict__ osub = orow + sub_base;
 
         u32x4_t graw[U], traw[U];
-        load_tile(k, graw, traw);
+        if (touches) {
+#pragma unroll
+            for (int j = 0; j < U; ++j) {
+                const int off = vec_offset<U, EPV, REV>(j, lane);
+                graw[j] = load_raw<Tr, ALIGNED, FULL>(gsub, off, win, vone<V>());
+                traw[j] = load_tok_raw<Tr, ALIGNED, FULL>(tsub, off, win, vzero<V>());
+            }
+        } else {
+#pragma unroll
+            for (int j = 0; j < U; ++j) {
+                graw[j] = fill_raw<Tr>(vone<V>());
+                traw[j] = fill_raw<Tr>(vzero<V>());
+            }
+        }
 
         // Pass 1: fold each vector into one (A, X) pair and scan the pairs.
         V totA[U], totX[U], exA[U], exX[U];
@@ -955,10 +941,22 @@ __global__ void __launch_bounds__(64 * kMaxWavesPerBlock)
                 o[e] = x;
             }
             const int off = vec_offset<U, EPV, REV>(j, lane);
-            if (full) {
-                store_vec<Tr, ALIGNED, true>(osub, off, win, o);
-            } else if constexpr (!REGULAR) {
-                if (touches) store_vec<Tr, ALIGNED, false>(osub, off, win, o);
+            if (touches) store_vec<Tr, ALIGNED, FULL>(osub, off, win, o);
+        }
+    };
+
+    // (Issuing the loads of step k+1 before the arithmetic of step k was tried
+    // and measured no faster: the memory system is already saturated by the
+    // other workgroups.)
+    for (int64_t k = k_begin; k < k_end; ++k) {
+        if constexpr (REGULAR) {
+            tile_step(k, std::true_type{});
+        } else {
+            const int64_t sub_base = sub_tile_base(k);
+            if (sub_base >= lo && sub_base + SUB <= hi) {  // wave-uniform
+                tile_step(k, std::true_type{});
+            } else {
+                tile_step(k, std::false_type{});
             }
         }
     }
@@ -1020,53 +1018,36 @@ __global__ void __launch_bounds__(64 * kMaxWavesPerBlock)
         const int64_t tile = ntiles - 1 - k;
         return tile * TILE + (int64_t)(W - 1 - w) * SUB;
     };
-    // Loads the three input vectors of every block of tile step k.
-    auto load_tile = [&](int64_t k, u32x4_t (&araw)[U], u32x4_t (&draw)[U], u32x4_t (&xraw)[U]) {
+    // One tile step of this wave; FULL as in the forward kernel.
+    auto tile_step = [&](int64_t k, auto full_tag) {
+        constexpr bool FULL = decltype(full_tag)::value;
         const int64_t sub_base = sub_tile_base(k);
-        const bool full = REGULAR || (sub_base >= lo && sub_base + SUB <= hi);  // wave-uniform
+        const int64_t sub_end = sub_base + SUB;
         const Window win = make_window(lo, hi, sub_base);
+        const bool touches = FULL || (win.hi > 0 && win.lo < SUB);  // wave-uniform
         const S* __restrict__ asub = arow + sub_base;
         const S* __restrict__ dsub = drow + sub_base;
         const S* __restrict__ xsub = xrow + sub_base;
-        if (full) {
-#pragma unroll
-            for (int j = 0; j < U; ++j) {
-                const int off = vec_offset<U, EPV, true>(j, lane);
-                araw[j] = load_raw<Tr, ALIGNED, true>(asub, off, win, vone<V>());
-                draw[j] = load_raw<Tr, ALIGNED, true>(dsub, off, win, vzero<V>());
-                xraw[j] = load_raw<Tr, ALIGNED, true>(xsub, off, win, vzero<V>());
-            }
-        } else if constexpr (!REGULAR) {
-            if (win.hi > 0 && win.lo < SUB) {
-#pragma unroll
-                for (int j = 0; j < U; ++j) {
-                    const int off = vec_offset<U, EPV, true>(j, lane);
-                    araw[j] = load_raw<Tr, ALIGNED, false>(asub, off, win, vone<V>());
-                    draw[j] = load_raw<Tr, ALIGNED, false>(dsub, off, win, vzero<V>());
-                    xraw[j] = load_raw<Tr, ALIGNED, false>(xsub, off, win, vzero<V>());
-                }
-            } else {
-#pragma unroll
-                for (int j = 0; j < U; ++j) {
-                    araw[j] = fill_raw<Tr>(vone<V>());
-                    draw[j] = fill_raw<Tr>(vzero<V>());
-                    xraw[j] = fill_raw<Tr>(vzero<V>());
-                }
-            }
-        }
-    };
-
-    for (int64_t k = k_begin; k < k_end; ++k) {
-        const int64_t sub_base = sub_tile_base(k);
-        const int64_t sub_end = sub_base + SUB;
-        const bool full = REGULAR || (sub_base >= lo && sub_end <= hi);  // wave-uniform
-        const Window win = make_window(lo, hi, sub_base);
-        const bool touches = win.hi > 0 && win.lo < SUB;  // wave-uniform
         S* __restrict__ dgsub = dgrow + sub_base;
         typename Tr::TokS* __restrict__ dtsub = dtrow + sub_base;
 
         u32x4_t araw[U], draw[U], xraw[U];
-        load_tile(k, araw, draw, xraw);
+        if (touches) {
+#pragma unroll
+            for (int j = 0; j < U; ++j) {
+                const int off = vec_offset<U, EPV, true>(j, lane);
+                araw[j] = load_raw<Tr, ALIGNED, FULL>(asub, off, win, vone<V>());
+                draw[j] = load_raw<Tr, ALIGNED, FULL>(dsub, off, win, vzero<V>());
+                xraw[j] = load_raw<Tr, ALIGNED, FULL>(xsub, off, win, vzero<V>());
+            }
+        } else {
+#pragma unroll
+            for (int j = 0; j < U; ++j) {
+                araw[j] = fill_raw<Tr>(vone<V>());
+                draw[j] = fill_raw<Tr>(vzero<V>());
+                xraw[j] = fill_raw<Tr>(vzero<V>());
+            }
+        }
 
         // The two elements just outside the sub-tile: gate at sub_end and x at
         // sub_base-1.  Addresses are clamped into the row so the loads are
@@ -1160,14 +1141,22 @@ __global__ void __launch_bounds__(64 * kMaxWavesPerBlock)
                 dg[e] = vmul(gr, xs);
             }
             const int off = vec_offset<U, EPV, true>(j, lane);
-            if (full) {
-                store_tok_vec<Tr, ALIGNED, true>(dtsub, off, win, dt);
-                store_vec<Tr, ALIGNED, true>(dgsub, off, win, dg);
-            } else if constexpr (!REGULAR) {
-                if (touches) {
-                    store_tok_vec<Tr, ALIGNED, false>(dtsub, off, win, dt);
-                    store_vec<Tr, ALIGNED, false>(dgsub, off, win, dg);
-                }
+            if (touches) {
+                store_tok_vec<Tr, ALIGNED, FULL>(dtsub, off, win, dt);
+                store_vec<Tr, ALIGNED, FULL>(dgsub, off, win, dg);
+            }
+        }
+    };
+
+    for (int64_t k = k_begin; k < k_end; ++k) {
+        if constexpr (REGULAR) {
+            tile_step(k, std::true_type{});
+        } else {
+            const int64_t sub_base = sub_tile_base(k);
+            if (sub_base >= lo && sub_base + SUB <= hi) {  // wave-uniform
+                tile_step(k, std::true_type{});
+            } else {
+                tile_step(k, std::false_type{});
             }
         }
     }
