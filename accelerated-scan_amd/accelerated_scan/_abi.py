@@ -12,7 +12,7 @@ from pathlib import Path
 
 import torch
 
-ABI_VERSION = 2
+ABI_VERSION = 3
 
 # ascan_dtype codes of include/ascan.h
 F32, BF16, F16, C64, C64_REAL_TOKENS = 0, 1, 2, 3, 4
@@ -50,6 +50,19 @@ _SIGNATURES = {
          ctypes.c_void_p, ctypes.c_size_t, ctypes.c_void_p],
     ),
     "ascan_workspace_timeouts": (ctypes.c_uint, [ctypes.c_void_p]),
+    "ascan_forward_from": (
+        ctypes.c_int,
+        [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p,
+         ctypes.c_int64, ctypes.c_int64, ctypes.c_int, ctypes.c_int,
+         ctypes.c_void_p, ctypes.c_size_t, ctypes.c_void_p],
+    ),
+    "ascan_backward_from": (
+        ctypes.c_int,
+        [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p,
+         ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p,
+         ctypes.c_int64, ctypes.c_int64, ctypes.c_int,
+         ctypes.c_void_p, ctypes.c_size_t, ctypes.c_void_p],
+    ),
     "ascan_status_string": (ctypes.c_char_p, [ctypes.c_int]),
     "ascan_last_hip_error": (ctypes.c_int, []),
     "ascan_abi_version": (ctypes.c_int, []),
@@ -144,15 +157,34 @@ def _workspace(lib, rows: int, seqlen: int, code: int, device: torch.device):
     return torch.empty(nbytes, dtype=torch.uint8, device=device)
 
 
-def forward(gates, tokens, out, reverse: bool, workspace=None) -> None:
-    """Enqueue the forward scan on the current stream of the tensors' device."""
+def _check_state(state, like, name: str) -> None:
+    """``initial`` / ``d_initial``: one element per row, in the dtype of the states."""
+    if state is None:
+        return
+    if (not state.is_cuda or state.device != like.device or state.dtype != like.dtype
+            or state.shape != like.shape[:-1] or not state.is_contiguous()):
+        raise RuntimeError(
+            f"accelerated_scan: expected {name} to be a contiguous {like.dtype} tensor of shape "
+            f"{tuple(like.shape[:-1])} on {like.device}"
+        )
+
+
+def forward(gates, tokens, out, reverse: bool, workspace=None, initial=None) -> None:
+    """Enqueue the forward scan on the current stream of the tensors' device.
+    ``initial`` (one state per row) starts the scan from that state."""
     lib = _lib or load()
     seqlen = tokens.shape[-1]
     rows = tokens.numel() // seqlen if seqlen else 0
     code = dtype_code(gates.dtype, tokens.dtype)
     if workspace is None:
         workspace = _workspace(lib, rows, seqlen, code, tokens.device)
-    if workspace is None:
+    if initial is not None:
+        _check_state(initial, out, "initial")
+        _launch(tokens.device, lambda stream: lib.ascan_forward_from(
+            gates.data_ptr(), tokens.data_ptr(), initial.data_ptr(), out.data_ptr(), rows, seqlen, code,
+            1 if reverse else 0, workspace.data_ptr() if workspace is not None else None,
+            workspace.numel() if workspace is not None else 0, stream))
+    elif workspace is None:
         _launch(tokens.device, lambda stream: lib.ascan_forward(
             gates.data_ptr(), tokens.data_ptr(), out.data_ptr(), rows, seqlen, code, 1 if reverse else 0, stream))
     else:
@@ -161,15 +193,26 @@ def forward(gates, tokens, out, reverse: bool, workspace=None) -> None:
             workspace.data_ptr(), workspace.numel(), stream))
 
 
-def backward(gates, states, grad_out, d_gates, d_tokens, workspace=None) -> None:
-    """Enqueue the fused backward scan on the current stream of the tensors' device."""
+def backward(gates, states, grad_out, d_gates, d_tokens, workspace=None, initial=None, d_initial=None) -> None:
+    """Enqueue the fused backward scan on the current stream of the tensors' device.
+    ``initial`` is the state the forward scan started from; ``d_initial``
+    receives its gradient (left untouched for an empty sequence)."""
     lib = _lib or load()
     seqlen = gates.shape[-1]
     rows = gates.numel() // seqlen if seqlen else 0
     code = dtype_code(gates.dtype, d_tokens.dtype)
     if workspace is None:
         workspace = _workspace(lib, rows, seqlen, code, gates.device)
-    if workspace is None:
+    if initial is not None or d_initial is not None:
+        _check_state(initial, states, "initial")
+        _check_state(d_initial, states, "d_initial")
+        _launch(gates.device, lambda stream: lib.ascan_backward_from(
+            gates.data_ptr(), states.data_ptr(), initial.data_ptr() if initial is not None else None,
+            grad_out.data_ptr(), d_gates.data_ptr(), d_tokens.data_ptr(),
+            d_initial.data_ptr() if d_initial is not None else None, rows, seqlen, code,
+            workspace.data_ptr() if workspace is not None else None,
+            workspace.numel() if workspace is not None else 0, stream))
+    elif workspace is None:
         _launch(gates.device, lambda stream: lib.ascan_backward(
             gates.data_ptr(), states.data_ptr(), grad_out.data_ptr(), d_gates.data_ptr(), d_tokens.data_ptr(),
             rows, seqlen, code, stream))

@@ -1,4 +1,4 @@
-"""The two HIP entry points as ``torch.library`` custom operators.
+"""The HIP entry points as ``torch.library`` custom operators.
 
 ``torch.compile`` cannot trace a ctypes call; it can trace an opaque custom
 operator that comes with a shape/dtype rule ("fake" implementation).  The
@@ -40,6 +40,34 @@ def scan_backward(
 @scan_backward.register_fake
 def _(gates, states, grad_out, real_tokens):
     return torch.empty_like(gates), _empty_token_grad(gates, real_tokens)
+
+
+@torch.library.custom_op("accelerated_scan::scan_forward_from", mutates_args=())
+def scan_forward_from(gates: torch.Tensor, tokens: torch.Tensor, initial: torch.Tensor, reverse: bool) -> torch.Tensor:
+    out = torch.empty_like(gates)
+    _abi.forward(gates, tokens, out, reverse, initial=initial)
+    return out
+
+
+@scan_forward_from.register_fake
+def _(gates, tokens, initial, reverse):
+    return torch.empty_like(gates)
+
+
+@torch.library.custom_op("accelerated_scan::scan_backward_from", mutates_args=())
+def scan_backward_from(
+    gates: torch.Tensor, states: torch.Tensor, initial: torch.Tensor, grad_out: torch.Tensor, real_tokens: bool
+) -> Tuple[torch.Tensor, torch.Tensor, torch.Tensor]:
+    d_gates = torch.empty_like(gates)
+    d_tokens = _empty_token_grad(gates, real_tokens)
+    d_initial = torch.zeros_like(initial)  # stays zero for an empty sequence
+    _abi.backward(gates, states, grad_out, d_gates, d_tokens, initial=initial, d_initial=d_initial)
+    return d_gates, d_tokens, d_initial
+
+
+@scan_backward_from.register_fake
+def _(gates, states, initial, grad_out, real_tokens):
+    return torch.empty_like(gates), _empty_token_grad(gates, real_tokens), torch.empty_like(initial)
 
 
 def _empty_token_grad(gates: torch.Tensor, real_tokens: bool) -> torch.Tensor:

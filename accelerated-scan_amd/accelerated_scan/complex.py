@@ -9,7 +9,7 @@ backward pass follows complex.py:79-92: with g the adjoint of the states,
 
 import torch
 
-from . import _abi, _ops
+from . import _abi, _ops, stateful
 
 
 def _require(cond: bool, what: str) -> None:
@@ -81,14 +81,20 @@ class Scan(torch.autograd.Function):
         return d_forget, d_inputs
 
 
-def scan(forget, inputs):
+def scan(forget, inputs, initial=None):
     """Solve ``x[t] = forget[t] * x[t-1] + inputs[t]`` over complex numbers.
 
     Arguments:
         forget (torch.Tensor): shape (B, C, T), complex64, contiguous.
         inputs (torch.Tensor): shape (B, C, T), complex64 or float32, contiguous.
+        initial (torch.Tensor, optional): shape (B, C), complex64, the state
+            ``x[-1]`` to start from (not in the reference, which starts from zero).
 
     Returns:
         (torch.Tensor): complex64 states of shape (B, C, T).
     """
+    if initial is not None:
+        if not torch.is_complex(forget):
+            raise TypeError("forget must be a complex tensor")
+        return stateful.scan(forget, inputs, initial)
     return Scan.apply(forget, inputs)

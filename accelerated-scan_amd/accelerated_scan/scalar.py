@@ -44,6 +44,9 @@ class Scan(torch.autograd.Function):
         return d_forget, d_inputs
 
 
-def scan(forget, inputs):
-    """Solve ``x[t] = forget[t] * x[t-1] + inputs[t]`` for (B, C, T) tensors of any T."""
+def scan(forget, inputs, initial=None):
+    """Solve ``x[t] = forget[t] * x[t-1] + inputs[t]`` for (B, C, T) tensors of any T.
+    ``initial`` (shape (B, C), optional, not in the reference) is the state ``x[-1]``."""
+    if initial is not None:
+        return warp.scan(forget, inputs, initial)
     return Scan.apply(forget, inputs)

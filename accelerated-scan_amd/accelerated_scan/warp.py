@@ -10,7 +10,7 @@ output before the kernel runs.
 
 import torch
 
-from . import _abi, _ops
+from . import _abi, _ops, stateful
 
 _REAL_DTYPES = (torch.float32, torch.bfloat16, torch.float16)
 
@@ -108,15 +108,20 @@ class Scan(torch.autograd.Function):
         return d_gates, d_tokens
 
 
-def scan(gates, tokens):
+def scan(gates, tokens, initial=None):
     """Solve the first-order recurrence ``x[t] = gates[t] * x[t-1] + tokens[t]``.
 
     Arguments:
         gates (torch.Tensor): shape (B, C, T), contiguous, on the GPU.
         tokens (torch.Tensor): shape (B, C, T), contiguous, same dtype.
+        initial (torch.Tensor, optional): shape (B, C), the state ``x[-1]`` to
+            start from (not in the reference, which starts from zero).
 
     Returns:
         (torch.Tensor): shape (B, C, T), the states ``x``; differentiable in
-        both arguments.
+        all arguments.
     """
+    if initial is not None:
+        _check_dtype(gates)
+        return stateful.scan(gates, tokens, initial)
     return Scan.apply(gates, tokens)

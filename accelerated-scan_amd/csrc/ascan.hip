@@ -688,7 +688,8 @@ __device__ __forceinline__ cfloat read_lane_at(cfloat v, int lane) {
 
 // State entering scan-order tile k of a row, for wave 0 of the workgroup that
 // owns the tile.  `mine` is that row's first record; records of successive
-// tiles are `stride` apart.  (tileA, tileX) is this tile's aggregate.
+// tiles are `stride` apart.  (tileA, tileX) is this tile's aggregate and
+// `row_start` the state entering tile 0.
 //
 // The walk back is done 64 tiles at a time: lane i looks at tile k-1-i, all
 // lanes wait for their record in parallel (one memory round trip instead of one
@@ -696,9 +697,9 @@ __device__ __forceinline__ cfloat read_lane_at(cfloat v, int lane) {
 // folded with lane reads.
 template <class V>
 __device__ __forceinline__ V split_look_back(SplitHeader* header, SplitRecord* mine, int64_t stride, int64_t k,
-                                             V tileA, V tileX, int lane) {
+                                             V tileA, V tileX, V row_start, int lane) {
     SplitRecord* rec = mine + k * stride;
-    V carry_in = vzero<V>();
+    V carry_in = row_start;  // the state entering tile 0
     if (k > 0) {
         if (lane == 0) {
             publish(rec->a, tileA);
@@ -775,7 +776,7 @@ __device__ __forceinline__ V split_look_back(SplitHeader* header, SplitRecord* m
 template <class V, int W, int U>
 __device__ __forceinline__ void exchange_carries_split(const V (&totA)[U], const V (&totX)[U], V& c, V* slots,
                                                        int w, int lane, SplitHeader* header, SplitRecord* mine,
-                                                       int64_t stride, int64_t k) {
+                                                       int64_t stride, int64_t k, V row_start) {
     V TA = totA[0], TX = totX[0];
 #pragma unroll
     for (int j = 1; j < U; ++j) {
@@ -801,7 +802,7 @@ __device__ __forceinline__ void exchange_carries_split(const V (&totA)[U], const
     }
     V* carry_slot = slots + kSlotsPerBuffer;
     if (w == 0) {  // wave-uniform
-        const V carry_in = split_look_back(header, mine, stride, k, runA, runX, lane);
+        const V carry_in = split_look_back(header, mine, stride, k, runA, runX, row_start, lane);
         if (lane == 0) *carry_slot = carry_in;
     }
     __syncthreads();
@@ -817,7 +818,8 @@ __device__ __forceinline__ void exchange_carries_split(const V (&totA)[U], const
 template <class Tr, int W, int U, bool REV, bool ALIGNED, bool REGULAR, bool SPLIT>
 __global__ void __launch_bounds__(64 * kMaxWavesPerBlock)
     scan_forward_kernel(const typename Tr::S* __restrict__ gates, const typename Tr::TokS* __restrict__ tokens,
-                        typename Tr::S* __restrict__ out, int64_t rows, int64_t T, SplitHeader* split) {
+                        typename Tr::S* __restrict__ out, int64_t rows, int64_t T, SplitHeader* split,
+                        const typename Tr::S* __restrict__ initial) {
     using S = typename Tr::S;
     using V = typename Tr::V;
     constexpr int EPV = Tr::EPV;
@@ -855,7 +857,10 @@ __global__ void __launch_bounds__(64 * kMaxWavesPerBlock)
     const typename Tr::TokS* __restrict__ trow = tokens + row * T - lo;
     S* __restrict__ orow = out + row * T - lo;
 
-    V carry = vzero<V>();
+    // state the row starts from (one element per row; absent = zero); a split
+    // row needs it in its first tile only
+    const V row_start = (initial != nullptr && (!SPLIT || k_begin == 0)) ? Tr::load1(initial + row) : vzero<V>();
+    V carry = row_start;
 
     // Position of this wave's sub-tile in tile step k.
     auto sub_tile_base = [&](int64_t k) {
@@ -916,7 +921,8 @@ __global__ void __launch_bounds__(64 * kMaxWavesPerBlock)
 
         V c;
         if constexpr (SPLIT) {
-            exchange_carries_split<V, W, U>(totA, totX, c, slots, w, lane, split, split_records(split) + row * ntiles, 1, k);
+            exchange_carries_split<V, W, U>(totA, totX, c, slots, w, lane, split, split_records(split) + row * ntiles, 1, k,
+                                            row_start);
         } else {
             exchange_carries<V, W, U>(totA, totX, carry, c, slots, (int)(k & 1), w, lane);
         }
@@ -971,7 +977,8 @@ template <class Tr, int W, int U, bool ALIGNED, bool REGULAR, bool SPLIT>
 __global__ void __launch_bounds__(64 * kMaxWavesPerBlock)
     scan_backward_kernel(const typename Tr::S* __restrict__ gates, const typename Tr::S* __restrict__ states,
                          const typename Tr::S* __restrict__ grad_out, typename Tr::S* __restrict__ d_gates,
-                         typename Tr::TokS* __restrict__ d_tokens, int64_t rows, int64_t T, SplitHeader* split) {
+                         typename Tr::TokS* __restrict__ d_tokens, int64_t rows, int64_t T, SplitHeader* split,
+                         const typename Tr::S* __restrict__ initial, typename Tr::S* __restrict__ d_initial) {
     using S = typename Tr::S;
     using V = typename Tr::V;
     constexpr int EPV = Tr::EPV;
@@ -1013,6 +1020,15 @@ __global__ void __launch_bounds__(64 * kMaxWavesPerBlock)
 
     V carry = vzero<V>();
 
+    // Gradient of x[-1], conj(gate[0]) * g[0], from g at position 0 of the row's
+    // first tile.  Positions below the row's first element (position lo) carry
+    // gate 1 and grad_out 0, so with lo > 0 that g already is the gradient;
+    // with lo == 0 the last factor is still missing.
+    auto store_start_gradient = [&](V g_low) {
+        if (lo == 0) g_low = vmul(vconj(Tr::load1(arow)), g_low);
+        if (lane == 0) Tr::store1(d_initial + row, g_low);
+    };
+
     // Position of this wave's sub-tile in tile step k (reverse time).
     auto sub_tile_base = [&](int64_t k) {
         const int64_t tile = ntiles - 1 - k;
@@ -1031,6 +1047,11 @@ __global__ void __launch_bounds__(64 * kMaxWavesPerBlock)
         S* __restrict__ dgsub = dgrow + sub_base;
         typename Tr::TokS* __restrict__ dtsub = dtrow + sub_base;
 
+        // x[-1], the state the forward scan started from (absent = zero), is
+        // needed by the sub-tile that holds the row's first element
+        V x_start = vzero<V>();
+        if (initial != nullptr && sub_base <= lo && lo < sub_end) x_start = Tr::load1(initial + row);  // wave-uniform
+
         u32x4_t araw[U], draw[U], xraw[U];
         if (touches) {
 #pragma unroll
@@ -1038,20 +1059,20 @@ __global__ void __launch_bounds__(64 * kMaxWavesPerBlock)
                 const int off = vec_offset<U, EPV, true>(j, lane);
                 araw[j] = load_raw<Tr, ALIGNED, FULL>(asub, off, win, vone<V>());
                 draw[j] = load_raw<Tr, ALIGNED, FULL>(dsub, off, win, vzero<V>());
-                xraw[j] = load_raw<Tr, ALIGNED, FULL>(xsub, off, win, vzero<V>());
+                xraw[j] = load_raw<Tr, ALIGNED, FULL>(xsub, off, win, x_start);
             }
         } else {
 #pragma unroll
             for (int j = 0; j < U; ++j) {
                 araw[j] = fill_raw<Tr>(vone<V>());
                 draw[j] = fill_raw<Tr>(vzero<V>());
-                xraw[j] = fill_raw<Tr>(vzero<V>());
+                xraw[j] = fill_raw<Tr>(x_start);
             }
         }
 
         // The two elements just outside the sub-tile: gate at sub_end and x at
         // sub_base-1.  Addresses are clamped into the row so the loads are
-        // unconditional; out-of-row positions take the identity values.
+        // unconditional; out-of-row positions take the identity gate and x[-1].
         V a_edge, x_edge;
         {
             const int64_t ia = sub_end < hi ? (sub_end > lo ? sub_end : lo) : hi - 1;
@@ -1060,7 +1081,7 @@ __global__ void __launch_bounds__(64 * kMaxWavesPerBlock)
             const V av = Tr::load1(arow + ia);
             const V xv = Tr::load1(xrow + ix);
             a_edge = vselect(sub_end >= lo && sub_end < hi, av, vone<V>());
-            x_edge = vselect(sub_base - 1 >= lo && sub_base - 1 < hi, xv, vzero<V>());
+            x_edge = vselect(sub_base - 1 >= lo && sub_base - 1 < hi, xv, x_start);
         }
 
         // Pass 1.  Gates are needed one element later (gate[t+1]) and states one
@@ -1112,11 +1133,11 @@ __global__ void __launch_bounds__(64 * kMaxWavesPerBlock)
 
         V c;
         if constexpr (SPLIT) {
-            exchange_carries_split<V, W, U>(totA, totX, c, slots, w, lane, split, split_records(split) + row * ntiles, 1, k);
+            exchange_carries_split<V, W, U>(totA, totX, c, slots, w, lane, split, split_records(split) + row * ntiles, 1, k,
+                                            vzero<V>());
         } else {
             exchange_carries<V, W, U>(totA, totX, carry, c, slots, (int)(k & 1), w, lane);
         }
-
         // Pass 2: the plain reverse recurrence and the gate gradient.
 #pragma unroll
         for (int j = 0; j < U; ++j) {
@@ -1146,6 +1167,12 @@ __global__ void __launch_bounds__(64 * kMaxWavesPerBlock)
                 store_vec<Tr, ALIGNED, FULL>(dgsub, off, win, dg);
             }
         }
+
+        // A split row's last tile step ends at the row's first element: after
+        // pass 2, c is g at the lowest position of this wave's sub-tile.
+        if constexpr (SPLIT) {
+            if (d_initial != nullptr && k == ntiles - 1 && w == W - 1) store_start_gradient(c);  // wave-uniform
+        }
     };
 
     for (int64_t k = k_begin; k < k_end; ++k) {
@@ -1159,6 +1186,10 @@ __global__ void __launch_bounds__(64 * kMaxWavesPerBlock)
                 tile_step(k, std::false_type{});
             }
         }
+    }
+    // after the last tile step the carry is g at position 0 of the first tile
+    if constexpr (!SPLIT) {
+        if (d_initial != nullptr && w == 0) store_start_gradient(carry);  // wave-uniform
     }
     }  // visits
 }
@@ -1246,8 +1277,8 @@ int launch_status(hipError_t e) {
 }
 
 template <class Tr, int W, bool REV, bool ALIGNED, bool REGULAR>
-hipError_t launch_forward(const void* gates, const void* tokens, void* out, int64_t rows, int64_t T,
-                          int rows_per_block, hipStream_t stream) {
+hipError_t launch_forward(const void* gates, const void* tokens, void* out, const void* initial, int64_t rows,
+                          int64_t T, int rows_per_block, hipStream_t stream) {
     using S = typename Tr::S;
     using TokS = typename Tr::TokS;
     constexpr int U = REGULAR ? Tuning<Tr>::U : Tuning<Tr>::UG;
@@ -1255,12 +1286,13 @@ hipError_t launch_forward(const void* gates, const void* tokens, void* out, int6
     const unsigned threads = 64u * W * rows_per_block;
     return launch(scan_forward_kernel<Tr, W, U, REV, ALIGNED, REGULAR, false>, blocks, threads, stream,
                   static_cast<const S*>(gates), static_cast<const TokS*>(tokens), static_cast<S*>(out), rows, T,
-                  static_cast<SplitHeader*>(nullptr));
+                  static_cast<SplitHeader*>(nullptr), static_cast<const S*>(initial));
 }
 
 template <class Tr, int W, bool ALIGNED, bool REGULAR>
 hipError_t launch_backward(const void* gates, const void* states, const void* grad_out, void* d_gates,
-                           void* d_tokens, int64_t rows, int64_t T, int rows_per_block, hipStream_t stream) {
+                           void* d_tokens, const void* initial, void* d_initial, int64_t rows, int64_t T,
+                           int rows_per_block, hipStream_t stream) {
     using S = typename Tr::S;
     using TokS = typename Tr::TokS;
     constexpr int U = REGULAR ? Tuning<Tr>::UB : Tuning<Tr>::UBG;
@@ -1269,7 +1301,7 @@ hipError_t launch_backward(const void* gates, const void* states, const void* gr
     return launch(scan_backward_kernel<Tr, W, U, ALIGNED, REGULAR, false>, blocks, threads, stream,
                   static_cast<const S*>(gates), static_cast<const S*>(states), static_cast<const S*>(grad_out),
                   static_cast<S*>(d_gates), static_cast<TokS*>(d_tokens), rows, T,
-                  static_cast<SplitHeader*>(nullptr));
+                  static_cast<SplitHeader*>(nullptr), static_cast<const S*>(initial), static_cast<S*>(d_initial));
 }
 
 // Caller-provided table for split rows (may be absent).
@@ -1351,8 +1383,8 @@ int64_t host_tiles_per_row(int64_t T, int64_t tile, bool regular, int lead) {
 }
 
 template <class Tr, bool REV, bool REGULAR>
-hipError_t launch_forward_split(const void* gates, const void* tokens, void* out, int64_t rows, int64_t T,
-                                int64_t ntiles, const Workspace& ws, hipStream_t stream) {
+hipError_t launch_forward_split(const void* gates, const void* tokens, void* out, const void* initial, int64_t rows,
+                                int64_t T, int64_t ntiles, const Workspace& ws, hipStream_t stream) {
     using S = typename Tr::S;
     using TokS = typename Tr::TokS;
     constexpr int U = REGULAR ? Tuning<Tr>::U : Tuning<Tr>::UG;
@@ -1364,13 +1396,13 @@ hipError_t launch_forward_split(const void* gates, const void* tokens, void* out
     const int64_t tiles = rows * ntiles;
     return launch(kernel, (unsigned)(tiles < resident ? tiles : resident), 64u * kSplitWaves, stream,
                   static_cast<const S*>(gates), static_cast<const TokS*>(tokens), static_cast<S*>(out), rows, T,
-                  static_cast<SplitHeader*>(ws.ptr));
+                  static_cast<SplitHeader*>(ws.ptr), static_cast<const S*>(initial));
 }
 
 template <class Tr, bool REGULAR>
 hipError_t launch_backward_split(const void* gates, const void* states, const void* grad_out, void* d_gates,
-                                 void* d_tokens, int64_t rows, int64_t T, int64_t ntiles, const Workspace& ws,
-                                 hipStream_t stream) {
+                                 void* d_tokens, const void* initial, void* d_initial, int64_t rows, int64_t T,
+                                 int64_t ntiles, const Workspace& ws, hipStream_t stream) {
     using S = typename Tr::S;
     using TokS = typename Tr::TokS;
     constexpr int U = REGULAR ? Tuning<Tr>::UB : Tuning<Tr>::UBG;
@@ -1383,7 +1415,7 @@ hipError_t launch_backward_split(const void* gates, const void* states, const vo
     return launch(kernel, (unsigned)(tiles < resident ? tiles : resident), 64u * kSplitWaves, stream,
                   static_cast<const S*>(gates), static_cast<const S*>(states), static_cast<const S*>(grad_out),
                   static_cast<S*>(d_gates), static_cast<TokS*>(d_tokens), rows, T,
-                  static_cast<SplitHeader*>(ws.ptr));
+                  static_cast<SplitHeader*>(ws.ptr), static_cast<const S*>(initial), static_cast<S*>(d_initial));
 }
 
 // Memory-access flavour of a launch.
@@ -1403,8 +1435,8 @@ Access choose_access(bool same_lead, int lead, int64_t T, int64_t tile) {
 }
 
 template <class Tr>
-int forward_typed(const void* gates, const void* tokens, void* out, int64_t rows, int64_t T, bool reverse,
-                  const Workspace& ws, hipStream_t stream) {
+int forward_typed(const void* gates, const void* tokens, void* out, const void* initial, int64_t rows, int64_t T,
+                  bool reverse, const Workspace& ws, hipStream_t stream) {
     constexpr int64_t kElem = (int64_t)sizeof(typename Tr::S);
     constexpr int64_t SUB = (int64_t)Tuning<Tr>::U * 64 * Tr::EPV;    // regular kernels
     constexpr int64_t SUBG = (int64_t)Tuning<Tr>::UG * 64 * Tr::EPV;  // kernels with masking code
@@ -1421,12 +1453,15 @@ int forward_typed(const void* gates, const void* tokens, void* out, int64_t rows
         const int64_t ntiles = host_tiles_per_row<Tr>(T, (regular ? SUB : SUBG) * kSplitWaves, regular, lead);
         if (want_split(rows, ntiles) && workspace_fits(ws, rows, ntiles)) {
             if (regular) {
-                err = reverse ? launch_forward_split<Tr, true, true>(gates, tokens, out, rows, T, ntiles, ws, stream)
-                              : launch_forward_split<Tr, false, true>(gates, tokens, out, rows, T, ntiles, ws, stream);
+                err = reverse ? launch_forward_split<Tr, true, true>(gates, tokens, out, initial, rows, T, ntiles, ws,
+                                                                     stream)
+                              : launch_forward_split<Tr, false, true>(gates, tokens, out, initial, rows, T, ntiles, ws,
+                                                                      stream);
             } else {
-                err = reverse
-                          ? launch_forward_split<Tr, true, false>(gates, tokens, out, rows, T, ntiles, ws, stream)
-                          : launch_forward_split<Tr, false, false>(gates, tokens, out, rows, T, ntiles, ws, stream);
+                err = reverse ? launch_forward_split<Tr, true, false>(gates, tokens, out, initial, rows, T, ntiles, ws,
+                                                                      stream)
+                              : launch_forward_split<Tr, false, false>(gates, tokens, out, initial, rows, T, ntiles,
+                                                                       ws, stream);
             }
             return launch_status(err);
         }
@@ -1434,9 +1469,9 @@ int forward_typed(const void* gates, const void* tokens, void* out, int64_t rows
 #define ASCAN_FWD(WV, AL, REG)                                                                     \
     do {                                                                                           \
         if (reverse)                                                                               \
-            err = launch_forward<Tr, WV, true, AL, REG>(gates, tokens, out, rows, T, R, stream);   \
+            err = launch_forward<Tr, WV, true, AL, REG>(gates, tokens, out, initial, rows, T, R, stream);   \
         else                                                                                       \
-            err = launch_forward<Tr, WV, false, AL, REG>(gates, tokens, out, rows, T, R, stream);  \
+            err = launch_forward<Tr, WV, false, AL, REG>(gates, tokens, out, initial, rows, T, R, stream);  \
     } while (0)
 #define ASCAN_FWD_W(AL, REG)                            \
     switch (plan.waves_per_row) {                       \
@@ -1460,7 +1495,8 @@ int forward_typed(const void* gates, const void* tokens, void* out, int64_t rows
 
 template <class Tr>
 int backward_typed(const void* gates, const void* states, const void* grad_out, void* d_gates, void* d_tokens,
-                   int64_t rows, int64_t T, const Workspace& ws, hipStream_t stream) {
+                   const void* initial, void* d_initial, int64_t rows, int64_t T, const Workspace& ws,
+                   hipStream_t stream) {
     constexpr int64_t kElem = (int64_t)sizeof(typename Tr::S);
     constexpr int64_t SUB = (int64_t)Tuning<Tr>::UB * 64 * Tr::EPV;    // regular kernels
     constexpr int64_t SUBG = (int64_t)Tuning<Tr>::UBG * 64 * Tr::EPV;  // kernels with masking code
@@ -1477,15 +1513,16 @@ int backward_typed(const void* gates, const void* states, const void* grad_out, 
         const bool regular = lead == 0 && T % (SUB * kSplitWaves) == 0;
         const int64_t ntiles = host_tiles_per_row<Tr>(T, (regular ? SUB : SUBG) * kSplitWaves, regular, lead);
         if (want_split(rows, ntiles) && workspace_fits(ws, rows, ntiles)) {
-            err = regular ? launch_backward_split<Tr, true>(gates, states, grad_out, d_gates, d_tokens, rows, T,
-                                                            ntiles, ws, stream)
-                          : launch_backward_split<Tr, false>(gates, states, grad_out, d_gates, d_tokens, rows, T,
-                                                             ntiles, ws, stream);
+            err = regular ? launch_backward_split<Tr, true>(gates, states, grad_out, d_gates, d_tokens, initial,
+                                                            d_initial, rows, T, ntiles, ws, stream)
+                          : launch_backward_split<Tr, false>(gates, states, grad_out, d_gates, d_tokens, initial,
+                                                             d_initial, rows, T, ntiles, ws, stream);
             return launch_status(err);
         }
     }
 #define ASCAN_BWD(WV, AL, REG) \
-    err = launch_backward<Tr, WV, AL, REG>(gates, states, grad_out, d_gates, d_tokens, rows, T, R, stream)
+    err = launch_backward<Tr, WV, AL, REG>(gates, states, grad_out, d_gates, d_tokens, initial, d_initial, rows, T, \
+                                           R, stream)
 #define ASCAN_BWD_W(AL, REG)                            \
     switch (plan.waves_per_row) {                       \
         case 1: ASCAN_BWD(1, AL, REG); break;           \
@@ -1525,49 +1562,56 @@ bool element_aligned(const void* p, size_t es) { return (reinterpret_cast<uintpt
 // Largest row count one launch can address: gridDim.x is limited to 2^31-1.
 constexpr int64_t kMaxBlocks = 2147483647LL;
 
-int forward_checked(const void* gates, const void* tokens, void* out, int64_t rows, int64_t seqlen, int dtype,
-                    int reverse, const Workspace& ws, void* stream) {
+int forward_checked(const void* gates, const void* tokens, void* out, const void* initial, int64_t rows,
+                    int64_t seqlen, int dtype, int reverse, const Workspace& ws, void* stream) {
     const size_t es = element_size(dtype);
     if (es == 0) return ASCAN_ERR_BAD_DTYPE;
     if (rows < 0 || seqlen < 0 || rows > kMaxBlocks) return ASCAN_ERR_BAD_SHAPE;
     if (rows == 0 || seqlen == 0) return ASCAN_OK;
     if (!gates || !tokens || !out) return ASCAN_ERR_NULL_POINTER;
-    if (!element_aligned(gates, es) || !element_aligned(tokens, token_size(dtype)) || !element_aligned(out, es))
+    if (!element_aligned(gates, es) || !element_aligned(tokens, token_size(dtype)) || !element_aligned(out, es) ||
+        !element_aligned(initial, es))
         return ASCAN_ERR_MISALIGNED;
     hipStream_t s = static_cast<hipStream_t>(stream);
     const bool rev = reverse != 0;
     switch (dtype) {
-        case ASCAN_F32: return forward_typed<TraitsF32>(gates, tokens, out, rows, seqlen, rev, ws, s);
-        case ASCAN_BF16: return forward_typed<TraitsBF16>(gates, tokens, out, rows, seqlen, rev, ws, s);
-        case ASCAN_F16: return forward_typed<TraitsF16>(gates, tokens, out, rows, seqlen, rev, ws, s);
-        case ASCAN_C64: return forward_typed<TraitsC64>(gates, tokens, out, rows, seqlen, rev, ws, s);
-        default: return forward_typed<TraitsC64RealTokens>(gates, tokens, out, rows, seqlen, rev, ws, s);
+        case ASCAN_F32: return forward_typed<TraitsF32>(gates, tokens, out, initial, rows, seqlen, rev, ws, s);
+        case ASCAN_BF16: return forward_typed<TraitsBF16>(gates, tokens, out, initial, rows, seqlen, rev, ws, s);
+        case ASCAN_F16: return forward_typed<TraitsF16>(gates, tokens, out, initial, rows, seqlen, rev, ws, s);
+        case ASCAN_C64: return forward_typed<TraitsC64>(gates, tokens, out, initial, rows, seqlen, rev, ws, s);
+        default: return forward_typed<TraitsC64RealTokens>(gates, tokens, out, initial, rows, seqlen, rev, ws, s);
     }
 }
 
 int backward_checked(const void* gates, const void* states, const void* grad_out, void* d_gates, void* d_tokens,
-                     int64_t rows, int64_t seqlen, int dtype, const Workspace& ws, void* stream) {
+                     const void* initial, void* d_initial, int64_t rows, int64_t seqlen, int dtype,
+                     const Workspace& ws, void* stream) {
     const size_t es = element_size(dtype);
     if (es == 0) return ASCAN_ERR_BAD_DTYPE;
     if (rows < 0 || seqlen < 0 || rows > kMaxBlocks) return ASCAN_ERR_BAD_SHAPE;
     if (rows == 0 || seqlen == 0) return ASCAN_OK;
     if (!gates || !states || !grad_out || !d_gates || !d_tokens) return ASCAN_ERR_NULL_POINTER;
     if (!element_aligned(gates, es) || !element_aligned(states, es) || !element_aligned(grad_out, es) ||
-        !element_aligned(d_gates, es) || !element_aligned(d_tokens, token_size(dtype)))
+        !element_aligned(d_gates, es) || !element_aligned(d_tokens, token_size(dtype)) ||
+        !element_aligned(initial, es) || !element_aligned(d_initial, es))
         return ASCAN_ERR_MISALIGNED;
     hipStream_t s = static_cast<hipStream_t>(stream);
     switch (dtype) {
         case ASCAN_F32:
-            return backward_typed<TraitsF32>(gates, states, grad_out, d_gates, d_tokens, rows, seqlen, ws, s);
+            return backward_typed<TraitsF32>(gates, states, grad_out, d_gates, d_tokens, initial, d_initial, rows,
+                                             seqlen, ws, s);
         case ASCAN_BF16:
-            return backward_typed<TraitsBF16>(gates, states, grad_out, d_gates, d_tokens, rows, seqlen, ws, s);
+            return backward_typed<TraitsBF16>(gates, states, grad_out, d_gates, d_tokens, initial, d_initial, rows,
+                                             seqlen, ws, s);
         case ASCAN_F16:
-            return backward_typed<TraitsF16>(gates, states, grad_out, d_gates, d_tokens, rows, seqlen, ws, s);
+            return backward_typed<TraitsF16>(gates, states, grad_out, d_gates, d_tokens, initial, d_initial, rows,
+                                             seqlen, ws, s);
         case ASCAN_C64:
-            return backward_typed<TraitsC64>(gates, states, grad_out, d_gates, d_tokens, rows, seqlen, ws, s);
+            return backward_typed<TraitsC64>(gates, states, grad_out, d_gates, d_tokens, initial, d_initial, rows,
+                                             seqlen, ws, s);
         default:
-            return backward_typed<TraitsC64RealTokens>(gates, states, grad_out, d_gates, d_tokens, rows, seqlen,
-                                                       ws, s);
+            return backward_typed<TraitsC64RealTokens>(gates, states, grad_out, d_gates, d_tokens, initial,
+                                                       d_initial, rows, seqlen, ws, s);
     }
 }
 
@@ -1577,13 +1621,13 @@ extern "C" {
 
 int ascan_forward(const void* gates, const void* tokens, void* out, int64_t rows, int64_t seqlen, int dtype,
                   int reverse, void* stream) {
-    return forward_checked(gates, tokens, out, rows, seqlen, dtype, reverse, Workspace{nullptr, 0}, stream);
+    return forward_checked(gates, tokens, out, nullptr, rows, seqlen, dtype, reverse, Workspace{nullptr, 0}, stream);
 }
 
 int ascan_backward(const void* gates, const void* states, const void* grad_out, void* d_gates, void* d_tokens,
                    int64_t rows, int64_t seqlen, int dtype, void* stream) {
-    return backward_checked(gates, states, grad_out, d_gates, d_tokens, rows, seqlen, dtype, Workspace{nullptr, 0},
-                            stream);
+    return backward_checked(gates, states, grad_out, d_gates, d_tokens, nullptr, nullptr, rows, seqlen, dtype,
+                            Workspace{nullptr, 0}, stream);
 }
 
 size_t ascan_workspace_bytes(int64_t rows, int64_t seqlen, int dtype) {
@@ -1599,14 +1643,28 @@ size_t ascan_workspace_bytes(int64_t rows, int64_t seqlen, int dtype) {
 
 int ascan_forward_split(const void* gates, const void* tokens, void* out, int64_t rows, int64_t seqlen, int dtype,
                         int reverse, void* workspace, size_t workspace_bytes, void* stream) {
-    return forward_checked(gates, tokens, out, rows, seqlen, dtype, reverse, Workspace{workspace, workspace_bytes},
-                           stream);
+    return forward_checked(gates, tokens, out, nullptr, rows, seqlen, dtype, reverse,
+                           Workspace{workspace, workspace_bytes}, stream);
 }
 
 int ascan_backward_split(const void* gates, const void* states, const void* grad_out, void* d_gates,
                          void* d_tokens, int64_t rows, int64_t seqlen, int dtype, void* workspace,
                          size_t workspace_bytes, void* stream) {
-    return backward_checked(gates, states, grad_out, d_gates, d_tokens, rows, seqlen, dtype,
+    return backward_checked(gates, states, grad_out, d_gates, d_tokens, nullptr, nullptr, rows, seqlen, dtype,
+                            Workspace{workspace, workspace_bytes}, stream);
+}
+
+int ascan_forward_from(const void* gates, const void* tokens, const void* initial, void* out, int64_t rows,
+                       int64_t seqlen, int dtype, int reverse, void* workspace, size_t workspace_bytes,
+                       void* stream) {
+    return forward_checked(gates, tokens, out, initial, rows, seqlen, dtype, reverse,
+                           Workspace{workspace, workspace_bytes}, stream);
+}
+
+int ascan_backward_from(const void* gates, const void* states, const void* initial, const void* grad_out,
+                        void* d_gates, void* d_tokens, void* d_initial, int64_t rows, int64_t seqlen, int dtype,
+                        void* workspace, size_t workspace_bytes, void* stream) {
+    return backward_checked(gates, states, grad_out, d_gates, d_tokens, initial, d_initial, rows, seqlen, dtype,
                             Workspace{workspace, workspace_bytes}, stream);
 }
 

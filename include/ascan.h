@@ -46,7 +46,7 @@
 extern "C" {
 #endif
 
-#define ASCAN_ABI_VERSION 2
+#define ASCAN_ABI_VERSION 3
 
 /* Element types of the tensors of a call. */
 enum ascan_dtype {
@@ -136,6 +136,35 @@ int ascan_backward_split(const void* gates, const void* states, const void* grad
                          void* workspace, size_t workspace_bytes, void* stream);
 
 unsigned int ascan_workspace_timeouts(const void* workspace_header_copy);
+
+/*
+ * Scans that start from a given state, for callers that process a long
+ * sequence in chunks (streaming inference, truncated back-propagation): the
+ * final state of one chunk, out[:, seqlen-1], is the `initial` of the next.
+ *
+ *     forward :  x[-1] = initial[row]       (reverse: y[seqlen] = initial[row])
+ *     backward:  d_gates[0]     = g[0] * conj(initial[row])
+ *                d_initial[row] = conj(gate[0]) * g[0]
+ *
+ * No counterpart in the reference, whose scans always start from zero
+ * (warp.cuh:76 kEmptyToken, scalar.py:28 h0 and complex.py:32-33 state_x = zeros).
+ *
+ *   initial    `rows` elements of the dtype of `out` (complex64 for both complex
+ *              dtypes), or NULL for zeros;
+ *   d_initial  `rows` elements of that dtype, or NULL when the gradient is not
+ *              wanted; not written when seqlen == 0;
+ *   workspace  as for the *_split calls; NULL selects the plain path.
+ *
+ * With initial == NULL and d_initial == NULL these calls are the *_split ones.
+ */
+int ascan_forward_from(const void* gates, const void* tokens, const void* initial, void* out,
+                       int64_t rows, int64_t seqlen, int dtype, int reverse,
+                       void* workspace, size_t workspace_bytes, void* stream);
+
+int ascan_backward_from(const void* gates, const void* states, const void* initial,
+                        const void* grad_out, void* d_gates, void* d_tokens, void* d_initial,
+                        int64_t rows, int64_t seqlen, int dtype,
+                        void* workspace, size_t workspace_bytes, void* stream);
 
 /* Static, human-readable text for an ascan_status code. */
 const char* ascan_status_string(int status);

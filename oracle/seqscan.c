@@ -119,3 +119,112 @@ void seq_backward_c64(const float* g, const float* state, const float* dout, dou
         }
     }
 }
+
+/*
+ * Scans that start from a given state (one per row), for sequences processed in
+ * chunks.  The reference always starts from zero (warp.cuh:76, scalar.py:28,
+ * complex.py:32-33); these restate the same recurrences with x[-1] = init[r]:
+ *   forward :  out[r,-1] = init[r]   (reverse: out[r,T] = init[r])
+ *   backward:  dg[r,0]  = a[0] * conj(init[r]),   dinit[r] = conj(g[r,0]) * a[0]
+ * Pinned by tests/test_oracle.py: equality with the zero-start functions above
+ * for init = 0, the chunking identity (a scan cut in two, the second half
+ * started from the first half's last state, equals the uncut scan, values and
+ * gradients), and torch autograd through the plain loop in float64.
+ */
+void seq_forward_from_f32(const float* g, const float* x, const float* init, double* out, int64_t rows, int64_t T,
+                          int reverse) {
+#pragma omp parallel for schedule(static)
+    for (int64_t r = 0; r < rows; ++r) {
+        const float* gr = g + r * T;
+        const float* xr = x + r * T;
+        double* o = out + r * T;
+        double s = init ? (double)init[r] : 0.0;
+        for (int64_t k = 0; k < T; ++k) {
+            const int64_t t = reverse ? T - 1 - k : k;
+            s = (double)gr[t] * s + (double)xr[t];
+            o[t] = s;
+        }
+    }
+}
+
+void seq_backward_from_f32(const float* g, const float* state, const float* init, const float* dout, double* dg,
+                           double* dx, double* dinit, int64_t rows, int64_t T) {
+#pragma omp parallel for schedule(static)
+    for (int64_t r = 0; r < rows; ++r) {
+        const float* gr = g + r * T;
+        const float* sr = state + r * T;
+        const float* dr = dout + r * T;
+        double* dgr = dg + r * T;
+        double* dxr = dx + r * T;
+        const double x0 = init ? (double)init[r] : 0.0;
+        double a = 0.0;
+        for (int64_t t = T - 1; t >= 0; --t) {
+            const double gnext = (t + 1 < T) ? (double)gr[t + 1] : 1.0;
+            a = (double)dr[t] + gnext * a;
+            dxr[t] = a;
+            dgr[t] = a * ((t > 0) ? (double)sr[t - 1] : x0);
+        }
+        if (dinit) dinit[r] = (T > 0) ? (double)gr[0] * a : 0.0;
+    }
+}
+
+void seq_forward_from_c64(const float* g, const float* x, const float* init, double* out, int64_t rows, int64_t T,
+                          int reverse) {
+#pragma omp parallel for schedule(static)
+    for (int64_t r = 0; r < rows; ++r) {
+        const float* gr = g + 2 * r * T;
+        const float* xr = x + 2 * r * T;
+        double* o = out + 2 * r * T;
+        double sr = init ? (double)init[2 * r] : 0.0, si = init ? (double)init[2 * r + 1] : 0.0;
+        for (int64_t k = 0; k < T; ++k) {
+            const int64_t t = reverse ? T - 1 - k : k;
+            const double a = gr[2 * t], b = gr[2 * t + 1];
+            const double nr = a * sr - b * si + (double)xr[2 * t];
+            const double ni = a * si + b * sr + (double)xr[2 * t + 1];
+            sr = nr;
+            si = ni;
+            o[2 * t] = sr;
+            o[2 * t + 1] = si;
+        }
+    }
+}
+
+void seq_backward_from_c64(const float* g, const float* state, const float* init, const float* dout, double* dg,
+                           double* dx, double* dinit, int64_t rows, int64_t T) {
+#pragma omp parallel for schedule(static)
+    for (int64_t r = 0; r < rows; ++r) {
+        const float* gr = g + 2 * r * T;
+        const float* sr = state + 2 * r * T;
+        const float* dr = dout + 2 * r * T;
+        double* dgr = dg + 2 * r * T;
+        double* dxr = dx + 2 * r * T;
+        const double x0r = init ? (double)init[2 * r] : 0.0, x0i = init ? (double)init[2 * r + 1] : 0.0;
+        double ar = 0.0, ai = 0.0;
+        for (int64_t t = T - 1; t >= 0; --t) {
+            double cr = 1.0, ci = 0.0; /* conj(g[t+1]) */
+            if (t + 1 < T) {
+                cr = gr[2 * (t + 1)];
+                ci = -(double)gr[2 * (t + 1) + 1];
+            }
+            const double nr = (double)dr[2 * t] + cr * ar - ci * ai;
+            const double ni = (double)dr[2 * t + 1] + cr * ai + ci * ar;
+            ar = nr;
+            ai = ni;
+            dxr[2 * t] = ar;
+            dxr[2 * t + 1] = ai;
+            double pr = x0r, pi = -x0i; /* conj(state[t-1]) */
+            if (t > 0) {
+                pr = sr[2 * (t - 1)];
+                pi = -(double)sr[2 * (t - 1) + 1];
+            }
+            dgr[2 * t] = ar * pr - ai * pi;
+            dgr[2 * t + 1] = ar * pi + ai * pr;
+        }
+        if (dinit) {
+            /* conj(g[0]) * a[0] */
+            const double cr = (T > 0) ? (double)gr[0] : 0.0, ci = (T > 0) ? -(double)gr[1] : 0.0;
+            dinit[2 * r] = cr * ar - ci * ai;
+            dinit[2 * r + 1] = cr * ai + ci * ar;
+        }
+    }
+}

@@ -33,7 +33,13 @@ def _load():
         lib.seq_forward_c64.argtypes = [p, p, p, i64, i64, ctypes.c_int]
         lib.seq_backward_f32.argtypes = [p, p, p, p, p, i64, i64]
         lib.seq_backward_c64.argtypes = [p, p, p, p, p, i64, i64]
-        for f in (lib.seq_forward_f32, lib.seq_forward_c64, lib.seq_backward_f32, lib.seq_backward_c64):
+        lib.seq_forward_from_f32.argtypes = [p, p, p, p, i64, i64, ctypes.c_int]
+        lib.seq_forward_from_c64.argtypes = [p, p, p, p, i64, i64, ctypes.c_int]
+        lib.seq_backward_from_f32.argtypes = [p, p, p, p, p, p, p, i64, i64]
+        lib.seq_backward_from_c64.argtypes = [p, p, p, p, p, p, p, i64, i64]
+        for f in (lib.seq_forward_f32, lib.seq_forward_c64, lib.seq_backward_f32, lib.seq_backward_c64,
+                  lib.seq_forward_from_f32, lib.seq_forward_from_c64, lib.seq_backward_from_f32,
+                  lib.seq_backward_from_c64):
             f.restype = None
         _lib = lib
     return _lib
@@ -77,3 +83,43 @@ def backward(gates, states, grad_out):
     fn = lib.seq_backward_c64 if cplx else lib.seq_backward_f32
     fn(gp, sp, dp, dg.ctypes.data_as(ctypes.c_void_p), dx.ctypes.data_as(ctypes.c_void_p), rows, T)
     return dg, dx
+
+
+def forward_from(gates, tokens, initial, reverse=False):
+    """Sequential scan in fp64 started from ``initial`` (shape = gates.shape[:-1])."""
+    lib = _load()
+    cplx = np.iscomplexobj(gates) or np.iscomplexobj(tokens) or np.iscomplexobj(initial)
+    dt = np.complex64 if cplx else np.float32
+    g, gp = _prep(gates, dt)
+    x, xp = _prep(tokens, dt)
+    i, ip = _prep(initial, dt)
+    assert g.shape == x.shape and i.shape == g.shape[:-1]
+    T = g.shape[-1]
+    rows = g.size // T if T else 0
+    out = np.empty(g.shape, dtype=np.complex128 if cplx else np.float64)
+    fn = lib.seq_forward_from_c64 if cplx else lib.seq_forward_from_f32
+    fn(gp, xp, ip, out.ctypes.data_as(ctypes.c_void_p), rows, T, int(bool(reverse)))
+    return out
+
+
+def backward_from(gates, states, initial, grad_out):
+    """(d_gates, d_tokens, d_initial) of the scan started from ``initial``, in fp64."""
+    lib = _load()
+    cplx = any(np.iscomplexobj(a) for a in (gates, states, initial, grad_out))
+    dt = np.complex64 if cplx else np.float32
+    g, gp = _prep(gates, dt)
+    s, sp = _prep(states, dt)
+    i, ip = _prep(initial, dt)
+    d, dp = _prep(grad_out, dt)
+    assert g.shape == s.shape == d.shape and i.shape == g.shape[:-1]
+    T = g.shape[-1]
+    rows = g.size // T if T else 0
+    odt = np.complex128 if cplx else np.float64
+    dg = np.empty(g.shape, dtype=odt)
+    dx = np.empty(g.shape, dtype=odt)
+    di = np.zeros(i.shape, dtype=odt)
+    if rows:
+        fn = lib.seq_backward_from_c64 if cplx else lib.seq_backward_from_f32
+        fn(gp, sp, ip, dp, dg.ctypes.data_as(ctypes.c_void_p), dx.ctypes.data_as(ctypes.c_void_p),
+           di.ctypes.data_as(ctypes.c_void_p), rows, T)
+    return dg, dx, di

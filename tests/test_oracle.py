@@ -216,3 +216,97 @@ def test_tree_scan_complex_vs_sequential():
     out = ref_scan.scan(gates, tokens).numpy()
     truth = seqscan.forward(gates.numpy(), tokens.numpy().astype(np.complex64))
     np.testing.assert_allclose(out, truth, rtol=1e-4, atol=1e-5)
+
+
+# ---------------------------------------------------------------------------
+# Scans started from a given state (oracle functions *_from)
+# ---------------------------------------------------------------------------
+def _loop_scan_from(gates, tokens, initial, reverse=False):
+    state = initial
+    outs = [None] * gates.shape[-1]
+    order = range(gates.shape[-1] - 1, -1, -1) if reverse else range(gates.shape[-1])
+    for t in order:
+        state = gates[..., t] * state + tokens[..., t]
+        outs[t] = state
+    return torch.stack(outs, dim=-1)
+
+
+def _complex_inputs(gen, shape):
+    gates = torch.polar(0.9 + 0.1 * torch.rand(*shape, generator=gen), 2 * math.pi * torch.rand(*shape, generator=gen))
+    tokens = torch.complex(torch.randn(*shape, generator=gen), torch.randn(*shape, generator=gen))
+    grad_out = torch.complex(torch.randn(*shape, generator=gen), torch.randn(*shape, generator=gen))
+    initial = torch.complex(torch.randn(*shape[:-1], generator=gen), torch.randn(*shape[:-1], generator=gen))
+    return gates, tokens, grad_out, initial
+
+
+@pytest.mark.parametrize("cplx", [False, True])
+def test_from_zero_equals_zero_start(cplx):
+    gen = torch.Generator().manual_seed(7)
+    if cplx:
+        gates, tokens, grad_out, initial = (t.numpy() for t in _complex_inputs(gen, (2, 3, 77)))
+    else:
+        gates, tokens, grad_out = (torch.randn(2, 3, 77, generator=gen).numpy() for _ in range(3))
+        initial = np.zeros((2, 3), dtype=np.float32)
+    zero = np.zeros_like(initial)
+    for reverse in (False, True):
+        np.testing.assert_array_equal(seqscan.forward_from(gates, tokens, zero, reverse),
+                                      seqscan.forward(gates, tokens, reverse))
+    states = seqscan.forward(gates, tokens).astype(gates.dtype)
+    dg, dx, di = seqscan.backward_from(gates, states, zero, grad_out)
+    dg0, dx0 = seqscan.backward(gates, states, grad_out)
+    np.testing.assert_array_equal(dg, dg0)
+    np.testing.assert_array_equal(dx, dx0)
+    np.testing.assert_allclose(di, np.conj(gates[..., 0].astype(di.dtype)) * dx0[..., 0], rtol=1e-14)
+
+
+@pytest.mark.parametrize("cplx", [False, True])
+@pytest.mark.parametrize("cut", [1, 50, 129])
+def test_from_chunking_identity(cplx, cut):
+    """A scan cut in two, the second part started from the last state of the
+    first, is the uncut scan; gradients chain through d_initial."""
+    gen = torch.Generator().manual_seed(11 + cut)
+    T = 130
+    if cplx:
+        gates, tokens, grad_out, _ = (t.numpy() for t in _complex_inputs(gen, (2, 2, T)))
+    else:
+        gates = torch.rand(2, 2, T, generator=gen).numpy()
+        tokens, grad_out = (torch.randn(2, 2, T, generator=gen).numpy() for _ in range(2))
+    whole = seqscan.forward(gates, tokens)
+    first = seqscan.forward(gates[..., :cut], tokens[..., :cut])
+    carry = first[..., -1].astype(gates.dtype)  # handed over in storage precision
+    second = seqscan.forward_from(gates[..., cut:], tokens[..., cut:], carry)
+    np.testing.assert_allclose(second, whole[..., cut:], rtol=2e-6, atol=2e-6)
+
+    # gradients, with exact (fp32-representable) states so the identity is tight
+    states = whole.astype(gates.dtype)
+    dg, dx = seqscan.backward(gates, states, grad_out)
+    dg2, dx2, di2 = seqscan.backward_from(gates[..., cut:], states[..., cut:], states[..., cut - 1], grad_out[..., cut:])
+    np.testing.assert_allclose(dg2, dg[..., cut:], rtol=1e-13, atol=1e-13)
+    np.testing.assert_allclose(dx2, dx[..., cut:], rtol=1e-13, atol=1e-13)
+    # the adjoint entering the first part at its last step is grad_out there plus d_initial of the second part
+    np.testing.assert_allclose(grad_out[..., cut - 1] + di2, dx[..., cut - 1], rtol=1e-12, atol=1e-12)
+
+
+@pytest.mark.parametrize("T", [1, 2, 9, 64])
+@pytest.mark.parametrize("cplx", [False, True])
+def test_from_vs_autograd_of_loop(T, cplx):
+    gen = torch.Generator().manual_seed(300 + T)
+    if cplx:
+        gates, tokens, grad_out, initial = _complex_inputs(gen, (2, 2, T))
+        wide = torch.complex128
+    else:
+        gates = torch.rand(2, 2, T, generator=gen)
+        tokens, grad_out = (torch.randn(2, 2, T, generator=gen) for _ in range(2))
+        initial = torch.randn(2, 2, generator=gen)
+        wide = torch.float64
+    gw, tw, iw = (t.to(wide).requires_grad_(True) for t in (gates, tokens, initial))
+    out = _loop_scan_from(gw, tw, iw)
+    dg_ref, dt_ref, di_ref = torch.autograd.grad(out, (gw, tw, iw), grad_out.to(wide))
+    fwd = seqscan.forward_from(gates.numpy(), tokens.numpy(), initial.numpy())
+    np.testing.assert_allclose(fwd, out.detach().numpy(), rtol=1e-12, atol=1e-12)
+    rev = seqscan.forward_from(gates.numpy(), tokens.numpy(), initial.numpy(), reverse=True)
+    np.testing.assert_allclose(rev, _loop_scan_from(gw, tw, iw, reverse=True).detach().numpy(), rtol=1e-12, atol=1e-12)
+    dg, dt, di = seqscan.backward_from(gates.numpy(), fwd.astype(gates.numpy().dtype), initial.numpy(), grad_out.numpy())
+    np.testing.assert_allclose(dt, dt_ref.numpy(), rtol=1e-12, atol=1e-12)
+    np.testing.assert_allclose(di, di_ref.numpy(), rtol=1e-12, atol=1e-12)
+    np.testing.assert_allclose(dg, dg_ref.numpy(), rtol=1e-5, atol=1e-5)  # states rounded to fp32 before the multiply
