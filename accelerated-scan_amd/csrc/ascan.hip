@@ -335,9 +335,13 @@ struct TraitsC64RealTokens : TraitsC64 {
 };
 
 // ---------------------------------------------------------------------------
-// Vector access.  A row is addressed in "virtual" positions: position 0 is the
-// 16-byte boundary at or just below the row's first element and the row's
-// elements occupy [lo, hi) with 0 <= lo < EPV.  Inside the tile loop everything
+// Vector access.  A row is addressed in "virtual" positions: position 0 is an
+// aligned boundary at or just below the row's first element -- a 128-byte one
+// when all tensors of the call sit alike on that grid, so that the 1 KiB a wave
+// moves per instruction is eight whole cache lines wherever the row starts
+// (rows on the 16-byte grid only measured 10 % slower), else a 16-byte one --
+// and the row's elements occupy [lo, hi) with 0 <= lo < G, G being the number
+// of elements between two such boundaries.  Inside the tile loop everything
 // is expressed relative to the wave's sub-tile: `sub` points at the first
 // element of the sub-tile (wave-uniform, 64-bit), `off` is the lane's 32-bit
 // element offset inside it, and a Window holds the row's valid range relative
@@ -506,12 +510,12 @@ __device__ __forceinline__ int64_t tiles_per_row(int64_t T, int64_t tile, int he
     return (T + head + tile - 1) / tile;
 }
 
-// Misalignment of the row start in elements (0 <= result < EPV).  All tensors
-// of a call share it: the host checks that their base addresses are congruent
-// modulo 16.
+// Misalignment of the row start in elements (0 <= result < G, G a power of
+// two).  All tensors of a call share it: the host checks that their base
+// addresses are congruent on that grid.
 template <class Tr>
-__device__ __forceinline__ int row_lead(const typename Tr::S* row_start) {
-    return (int)((reinterpret_cast<uintptr_t>(row_start) / sizeof(typename Tr::S)) % Tr::EPV);
+__device__ __forceinline__ int row_lead(const typename Tr::S* row_start, int G) {
+    return (int)((reinterpret_cast<uintptr_t>(row_start) / sizeof(typename Tr::S)) & (uintptr_t)(G - 1));
 }
 
 // Element index (inside the sub-tile) of the vector that lane `lane` owns in
@@ -819,7 +823,7 @@ template <class Tr, int W, int U, bool REV, bool ALIGNED, bool REGULAR, bool SPL
 __global__ void __launch_bounds__(64 * kMaxWavesPerBlock)
     scan_forward_kernel(const typename Tr::S* __restrict__ gates, const typename Tr::TokS* __restrict__ tokens,
                         typename Tr::S* __restrict__ out, int64_t rows, int64_t T, SplitHeader* split,
-                        const typename Tr::S* __restrict__ initial) {
+                        const typename Tr::S* __restrict__ initial, int G) {
     using S = typename Tr::S;
     using V = typename Tr::V;
     constexpr int EPV = Tr::EPV;
@@ -827,8 +831,8 @@ __global__ void __launch_bounds__(64 * kMaxWavesPerBlock)
     constexpr int64_t TILE = SUB * W;
 
     const int lane = threadIdx.x & 63;
-    // rows start at the same misalignment when T is a multiple of the vector width
-    const int head = REGULAR ? 0 : (ALIGNED ? (T % EPV == 0 ? row_lead<Tr>(gates) : EPV - 1) : 0);
+    // rows start at the same misalignment when T is a multiple of the grid spacing
+    const int head = REGULAR ? 0 : (ALIGNED ? (T % G == 0 ? row_lead<Tr>(gates, G) : G - 1) : 0);
     const int64_t ntiles = tiles_per_row(T, TILE, head);
     __shared__ V slots_all[W == 1 ? 1 : 2 * kSlotsPerBuffer];
     // Split rows: a fixed set of co-resident workgroups walks over all (row,
@@ -851,7 +855,7 @@ __global__ void __launch_bounds__(64 * kMaxWavesPerBlock)
     }
     V* slots = slots_all + (W == 1 ? 0 : slot_base);
 
-    const int64_t lo = (ALIGNED && !REGULAR) ? row_lead<Tr>(gates + row * T) : 0;
+    const int64_t lo = (ALIGNED && !REGULAR) ? row_lead<Tr>(gates + row * T, G) : 0;
     const int64_t hi = lo + T;
     const S* __restrict__ grow = gates + row * T - lo;
     const typename Tr::TokS* __restrict__ trow = tokens + row * T - lo;
@@ -978,7 +982,7 @@ __global__ void __launch_bounds__(64 * kMaxWavesPerBlock)
     scan_backward_kernel(const typename Tr::S* __restrict__ gates, const typename Tr::S* __restrict__ states,
                          const typename Tr::S* __restrict__ grad_out, typename Tr::S* __restrict__ d_gates,
                          typename Tr::TokS* __restrict__ d_tokens, int64_t rows, int64_t T, SplitHeader* split,
-                         const typename Tr::S* __restrict__ initial, typename Tr::S* __restrict__ d_initial) {
+                         const typename Tr::S* __restrict__ initial, typename Tr::S* __restrict__ d_initial, int G) {
     using S = typename Tr::S;
     using V = typename Tr::V;
     constexpr int EPV = Tr::EPV;
@@ -986,8 +990,8 @@ __global__ void __launch_bounds__(64 * kMaxWavesPerBlock)
     constexpr int64_t TILE = SUB * W;
 
     const int lane = threadIdx.x & 63;
-    // rows start at the same misalignment when T is a multiple of the vector width
-    const int head = REGULAR ? 0 : (ALIGNED ? (T % EPV == 0 ? row_lead<Tr>(gates) : EPV - 1) : 0);
+    // rows start at the same misalignment when T is a multiple of the grid spacing
+    const int head = REGULAR ? 0 : (ALIGNED ? (T % G == 0 ? row_lead<Tr>(gates, G) : G - 1) : 0);
     const int64_t ntiles = tiles_per_row(T, TILE, head);
     __shared__ V slots_all[W == 1 ? 1 : 2 * kSlotsPerBuffer];
     // Split rows: a fixed set of co-resident workgroups walks over all (row,
@@ -1010,7 +1014,7 @@ __global__ void __launch_bounds__(64 * kMaxWavesPerBlock)
     }
     V* slots = slots_all + (W == 1 ? 0 : slot_base);
 
-    const int64_t lo = (ALIGNED && !REGULAR) ? row_lead<Tr>(gates + row * T) : 0;
+    const int64_t lo = (ALIGNED && !REGULAR) ? row_lead<Tr>(gates + row * T, G) : 0;
     const int64_t hi = lo + T;
     const S* __restrict__ arow = gates + row * T - lo;
     const S* __restrict__ xrow = states + row * T - lo;
@@ -1252,11 +1256,31 @@ Plan choose_plan(int64_t T, int64_t sub, int64_t element_bytes) {
     return Plan{w, r};
 }
 
-// Offset of an address inside its vector, in elements: vectors of a tensor are
-// `epv` elements of `elem_bytes` bytes.  Tensors whose first elements have the
-// same lead line up vector by vector, row by row.
-int lead_of(const void* p, size_t elem_bytes, int epv) {
-    return (int)((reinterpret_cast<uintptr_t>(p) / elem_bytes) % (unsigned)epv);
+// Offset of an address from the grid boundary below it, in elements of
+// `elem_bytes` bytes; boundaries are `grid` elements apart.  Tensors whose first
+// elements have the same lead line up vector by vector, row by row.
+int lead_of(const void* p, size_t elem_bytes, int grid) {
+    return (int)((reinterpret_cast<uintptr_t>(p) / elem_bytes) % (unsigned)grid);
+}
+
+// The grid rows are addressed from (elements between boundaries) and where the
+// call's tensors sit on it.
+struct Lead {
+    int grid;   // 128 bytes of states when all tensors agree there, else one 16-byte vector
+    int lead;   // of the first tensor
+    bool same;  // all tensors share `lead` on `grid`
+};
+
+template <class Tr, size_t N>
+Lead find_lead(const void* const (&state_like)[N], const void* token_like) {
+    constexpr size_t kElem = sizeof(typename Tr::S);
+    for (int grid : {(int)(128 / kElem), Tr::EPV}) {
+        const int lead = lead_of(state_like[0], kElem, grid);
+        bool same = lead_of(token_like, sizeof(typename Tr::TokS), grid) == lead;
+        for (size_t i = 1; i < N; ++i) same = same && lead_of(state_like[i], kElem, grid) == lead;
+        if (same || grid == Tr::EPV) return Lead{grid, lead, same};
+    }
+    return Lead{Tr::EPV, 0, false};  // not reached
 }
 
 // Launches through hipLaunchKernel so that the launch's own status comes back
@@ -1278,7 +1302,7 @@ int launch_status(hipError_t e) {
 
 template <class Tr, int W, bool REV, bool ALIGNED, bool REGULAR>
 hipError_t launch_forward(const void* gates, const void* tokens, void* out, const void* initial, int64_t rows,
-                          int64_t T, int rows_per_block, hipStream_t stream) {
+                          int64_t T, int grid, int rows_per_block, hipStream_t stream) {
     using S = typename Tr::S;
     using TokS = typename Tr::TokS;
     constexpr int U = REGULAR ? Tuning<Tr>::U : Tuning<Tr>::UG;
@@ -1286,12 +1310,12 @@ hipError_t launch_forward(const void* gates, const void* tokens, void* out, cons
     const unsigned threads = 64u * W * rows_per_block;
     return launch(scan_forward_kernel<Tr, W, U, REV, ALIGNED, REGULAR, false>, blocks, threads, stream,
                   static_cast<const S*>(gates), static_cast<const TokS*>(tokens), static_cast<S*>(out), rows, T,
-                  static_cast<SplitHeader*>(nullptr), static_cast<const S*>(initial));
+                  static_cast<SplitHeader*>(nullptr), static_cast<const S*>(initial), grid);
 }
 
 template <class Tr, int W, bool ALIGNED, bool REGULAR>
 hipError_t launch_backward(const void* gates, const void* states, const void* grad_out, void* d_gates,
-                           void* d_tokens, const void* initial, void* d_initial, int64_t rows, int64_t T,
+                           void* d_tokens, const void* initial, void* d_initial, int64_t rows, int64_t T, int grid,
                            int rows_per_block, hipStream_t stream) {
     using S = typename Tr::S;
     using TokS = typename Tr::TokS;
@@ -1301,7 +1325,7 @@ hipError_t launch_backward(const void* gates, const void* states, const void* gr
     return launch(scan_backward_kernel<Tr, W, U, ALIGNED, REGULAR, false>, blocks, threads, stream,
                   static_cast<const S*>(gates), static_cast<const S*>(states), static_cast<const S*>(grad_out),
                   static_cast<S*>(d_gates), static_cast<TokS*>(d_tokens), rows, T,
-                  static_cast<SplitHeader*>(nullptr), static_cast<const S*>(initial), static_cast<S*>(d_initial));
+                  static_cast<SplitHeader*>(nullptr), static_cast<const S*>(initial), static_cast<S*>(d_initial), grid);
 }
 
 // Caller-provided table for split rows (may be absent).
@@ -1377,14 +1401,14 @@ unsigned resident_workgroups(K kernel, int threads) {
 
 // Tiles per row as the kernels count them (tiles_per_row on the device).
 template <class Tr>
-int64_t host_tiles_per_row(int64_t T, int64_t tile, bool regular, int lead) {
-    const int head = regular ? 0 : (T % Tr::EPV == 0 ? lead : Tr::EPV - 1);
+int64_t host_tiles_per_row(int64_t T, int64_t tile, bool regular, const Lead& at) {
+    const int head = regular ? 0 : (T % at.grid == 0 ? at.lead : at.grid - 1);
     return (T + head + tile - 1) / tile;
 }
 
 template <class Tr, bool REV, bool REGULAR>
 hipError_t launch_forward_split(const void* gates, const void* tokens, void* out, const void* initial, int64_t rows,
-                                int64_t T, int64_t ntiles, const Workspace& ws, hipStream_t stream) {
+                                int64_t T, int grid, int64_t ntiles, const Workspace& ws, hipStream_t stream) {
     using S = typename Tr::S;
     using TokS = typename Tr::TokS;
     constexpr int U = REGULAR ? Tuning<Tr>::U : Tuning<Tr>::UG;
@@ -1396,13 +1420,13 @@ hipError_t launch_forward_split(const void* gates, const void* tokens, void* out
     const int64_t tiles = rows * ntiles;
     return launch(kernel, (unsigned)(tiles < resident ? tiles : resident), 64u * kSplitWaves, stream,
                   static_cast<const S*>(gates), static_cast<const TokS*>(tokens), static_cast<S*>(out), rows, T,
-                  static_cast<SplitHeader*>(ws.ptr), static_cast<const S*>(initial));
+                  static_cast<SplitHeader*>(ws.ptr), static_cast<const S*>(initial), grid);
 }
 
 template <class Tr, bool REGULAR>
 hipError_t launch_backward_split(const void* gates, const void* states, const void* grad_out, void* d_gates,
                                  void* d_tokens, const void* initial, void* d_initial, int64_t rows, int64_t T,
-                                 int64_t ntiles, const Workspace& ws, hipStream_t stream) {
+                                 int grid, int64_t ntiles, const Workspace& ws, hipStream_t stream) {
     using S = typename Tr::S;
     using TokS = typename Tr::TokS;
     constexpr int U = REGULAR ? Tuning<Tr>::UB : Tuning<Tr>::UBG;
@@ -1415,17 +1439,17 @@ hipError_t launch_backward_split(const void* gates, const void* states, const vo
     return launch(kernel, (unsigned)(tiles < resident ? tiles : resident), 64u * kSplitWaves, stream,
                   static_cast<const S*>(gates), static_cast<const S*>(states), static_cast<const S*>(grad_out),
                   static_cast<S*>(d_gates), static_cast<TokS*>(d_tokens), rows, T,
-                  static_cast<SplitHeader*>(ws.ptr), static_cast<const S*>(initial), static_cast<S*>(d_initial));
+                  static_cast<SplitHeader*>(ws.ptr), static_cast<const S*>(initial), static_cast<S*>(d_initial), grid);
 }
 
 // Memory-access flavour of a launch.
-//   kRegular    : every row starts on a 16-byte boundary and is a whole number
+//   kRegular    : every row starts on a grid boundary and is a whole number
 //                 of tiles long, so every sub-tile is full: the kernel carries
 //                 no masking code at all (the common case: T a power of two).
-//   kVector     : all tensors share one offset inside a vector; rows may start
+//   kVector     : all tensors share one offset from the grid; rows may start
 //                 anywhere and have any length.  Whole-vector accesses except
 //                 where a vector straddles a row end.
-//   kElementwise: tensors at different offsets inside a vector.
+//   kElementwise: tensors at different offsets inside a 16-byte vector.
 enum class Access { kRegular, kVector, kElementwise };
 
 Access choose_access(bool same_lead, int lead, int64_t T, int64_t tile) {
@@ -1441,37 +1465,35 @@ int forward_typed(const void* gates, const void* tokens, void* out, const void* 
     constexpr int64_t SUB = (int64_t)Tuning<Tr>::U * 64 * Tr::EPV;    // regular kernels
     constexpr int64_t SUBG = (int64_t)Tuning<Tr>::UG * 64 * Tr::EPV;  // kernels with masking code
     Plan plan = choose_plan(T, SUB, kElem);
-    const int lead = lead_of(gates, kElem, Tr::EPV);
-    const bool same_lead = lead_of(tokens, sizeof(typename Tr::TokS), Tr::EPV) == lead &&
-                           lead_of(out, kElem, Tr::EPV) == lead;
+    const void* const state_like[] = {gates, out};
+    const Lead at = find_lead<Tr>(state_like, tokens);
+    const bool same_lead = at.same;
+    const int lead = at.lead;
     const Access access = choose_access(same_lead, lead, T, SUB * plan.waves_per_row);
     if (access != Access::kRegular) plan = choose_plan(T, SUBG, kElem);
     const int R = plan.rows_per_block;
     hipError_t err = hipSuccess;
     if (same_lead && ws.ptr != nullptr) {
         const bool regular = lead == 0 && T % (SUB * kSplitWaves) == 0;
-        const int64_t ntiles = host_tiles_per_row<Tr>(T, (regular ? SUB : SUBG) * kSplitWaves, regular, lead);
+        const int64_t ntiles = host_tiles_per_row<Tr>(T, (regular ? SUB : SUBG) * kSplitWaves, regular, at);
         if (want_split(rows, ntiles) && workspace_fits(ws, rows, ntiles)) {
+#define ASCAN_FWD_SPLIT(REV, REG) \
+    launch_forward_split<Tr, REV, REG>(gates, tokens, out, initial, rows, T, at.grid, ntiles, ws, stream)
             if (regular) {
-                err = reverse ? launch_forward_split<Tr, true, true>(gates, tokens, out, initial, rows, T, ntiles, ws,
-                                                                     stream)
-                              : launch_forward_split<Tr, false, true>(gates, tokens, out, initial, rows, T, ntiles, ws,
-                                                                      stream);
+                err = reverse ? ASCAN_FWD_SPLIT(true, true) : ASCAN_FWD_SPLIT(false, true);
             } else {
-                err = reverse ? launch_forward_split<Tr, true, false>(gates, tokens, out, initial, rows, T, ntiles, ws,
-                                                                      stream)
-                              : launch_forward_split<Tr, false, false>(gates, tokens, out, initial, rows, T, ntiles,
-                                                                       ws, stream);
+                err = reverse ? ASCAN_FWD_SPLIT(true, false) : ASCAN_FWD_SPLIT(false, false);
             }
+#undef ASCAN_FWD_SPLIT
             return launch_status(err);
         }
     }
 #define ASCAN_FWD(WV, AL, REG)                                                                     \
     do {                                                                                           \
         if (reverse)                                                                               \
-            err = launch_forward<Tr, WV, true, AL, REG>(gates, tokens, out, initial, rows, T, R, stream);   \
-        else                                                                                       \
-            err = launch_forward<Tr, WV, false, AL, REG>(gates, tokens, out, initial, rows, T, R, stream);  \
+            err = launch_forward<Tr, WV, true, AL, REG>(gates, tokens, out, initial, rows, T, at.grid, R, stream);  \
+        else                                                                                                       \
+            err = launch_forward<Tr, WV, false, AL, REG>(gates, tokens, out, initial, rows, T, at.grid, R, stream); \
     } while (0)
 #define ASCAN_FWD_W(AL, REG)                            \
     switch (plan.waves_per_row) {                       \
@@ -1500,10 +1522,10 @@ int backward_typed(const void* gates, const void* states, const void* grad_out, 
     constexpr int64_t kElem = (int64_t)sizeof(typename Tr::S);
     constexpr int64_t SUB = (int64_t)Tuning<Tr>::UB * 64 * Tr::EPV;    // regular kernels
     constexpr int64_t SUBG = (int64_t)Tuning<Tr>::UBG * 64 * Tr::EPV;  // kernels with masking code
-    const int lead = lead_of(gates, kElem, Tr::EPV);
-    const bool same_lead = lead_of(states, kElem, Tr::EPV) == lead && lead_of(grad_out, kElem, Tr::EPV) == lead &&
-                           lead_of(d_gates, kElem, Tr::EPV) == lead &&
-                           lead_of(d_tokens, sizeof(typename Tr::TokS), Tr::EPV) == lead;
+    const void* const state_like[] = {gates, states, grad_out, d_gates};
+    const Lead at = find_lead<Tr>(state_like, d_tokens);
+    const bool same_lead = at.same;
+    const int lead = at.lead;
     Plan plan = choose_plan(T, SUB, kElem);
     const Access access = choose_access(same_lead, lead, T, SUB * plan.waves_per_row);
     if (access != Access::kRegular) plan = choose_plan(T, SUBG, kElem);
@@ -1511,18 +1533,18 @@ int backward_typed(const void* gates, const void* states, const void* grad_out, 
     hipError_t err = hipSuccess;
     if (same_lead && ws.ptr != nullptr) {
         const bool regular = lead == 0 && T % (SUB * kSplitWaves) == 0;
-        const int64_t ntiles = host_tiles_per_row<Tr>(T, (regular ? SUB : SUBG) * kSplitWaves, regular, lead);
+        const int64_t ntiles = host_tiles_per_row<Tr>(T, (regular ? SUB : SUBG) * kSplitWaves, regular, at);
         if (want_split(rows, ntiles) && workspace_fits(ws, rows, ntiles)) {
             err = regular ? launch_backward_split<Tr, true>(gates, states, grad_out, d_gates, d_tokens, initial,
-                                                            d_initial, rows, T, ntiles, ws, stream)
+                                                            d_initial, rows, T, at.grid, ntiles, ws, stream)
                           : launch_backward_split<Tr, false>(gates, states, grad_out, d_gates, d_tokens, initial,
-                                                             d_initial, rows, T, ntiles, ws, stream);
+                                                             d_initial, rows, T, at.grid, ntiles, ws, stream);
             return launch_status(err);
         }
     }
 #define ASCAN_BWD(WV, AL, REG) \
     err = launch_backward<Tr, WV, AL, REG>(gates, states, grad_out, d_gates, d_tokens, initial, d_initial, rows, T, \
-                                           R, stream)
+                                           at.grid, R, stream)
 #define ASCAN_BWD_W(AL, REG)                            \
     switch (plan.waves_per_row) {                       \
         case 1: ASCAN_BWD(1, AL, REG); break;           \
@@ -1636,7 +1658,9 @@ size_t ascan_workspace_bytes(int64_t rows, int64_t seqlen, int dtype) {
     // the smallest split tile any kernel uses for this dtype: 4 waves x 2 blocks x 64 vectors
     const int64_t epv = 16 / (int64_t)es;
     const int64_t tile = (int64_t)kSplitWaves * 2 * 64 * epv;
-    const int64_t ntiles = (seqlen + epv - 1 + tile - 1) / tile;
+    // rows are addressed from the 128-byte boundary below their first element at most
+    const int64_t head = 128 / (int64_t)es - 1;
+    const int64_t ntiles = (seqlen + head + tile - 1) / tile;
     if (!want_split(rows, ntiles) || rows * ntiles > 2147483647LL) return 0;
     return split_bytes(rows, ntiles);
 }

@@ -32,8 +32,9 @@
  *     formats, rounded to nearest-even on store);
  *   - buffers whose addresses agree modulo 16 (the usual case: allocator
  *     blocks, or equal storage offsets) take the vectorised kernels for any
- *     seqlen; buffers at different offsets inside a 16-byte block take
- *     element-wise kernels with the same arithmetic;
+ *     seqlen, at full speed when they also agree modulo 128; buffers at
+ *     different offsets inside a 16-byte block take element-wise kernels with
+ *     the same arithmetic;
  *   - errors are reported by return code, never by abort or exception.
  */
 #ifndef ASCAN_H_

@@ -235,19 +235,22 @@ def test_unaligned_rows(dtype, rows, T):
 
 
 @pytest.mark.parametrize("dtype", ALL_DTYPES, ids=ALL_IDS)
-@pytest.mark.parametrize("offsets", [(1, 1, 1), (3, 3, 3), (1, 0, 2)], ids=["same1", "same3", "mixed"])
+@pytest.mark.parametrize("offsets", [(1, 1, 1), (3, 3, 3), (1, 0, 2), (1, 9, 17), (4, 12, 8)],
+                         ids=["same1", "same3", "mixed", "same-mod-8", "multiples-of-4"])
 @pytest.mark.parametrize("rows,T", [(6, 2048), (3, 40000), (2050, 1031)])
 def test_unaligned_base_pointer(dtype, offsets, rows, T):
     """Views with a storage offset: base pointers off the 16-byte grid.  Equal
-    offsets keep the vectorised kernels (rows are addressed from the 16-byte
-    boundary below their start); different offsets per tensor take the
+    offsets keep the vectorised kernels (rows are addressed from the 128-byte
+    boundary below their start, or from the 16-byte one when the tensors agree
+    only on that grid: the last two offset sets, depending on the element
+    size); tensors at different offsets inside a 16-byte vector take the
     element-wise kernels."""
     from accelerated_scan import _abi
 
     gates, tokens, grad_out = _truth_inputs(rows, T, dtype, seed=9)
 
     def offset_copy(t, k):
-        flat = torch.empty(rows * T + 4, dtype=t.dtype, device=DEVICE)
+        flat = torch.empty(rows * T + 32, dtype=t.dtype, device=DEVICE)
         view = flat[k:k + rows * T].view(1, rows, T)
         view.copy_(t.reshape(1, rows, T))
         assert view.is_contiguous()

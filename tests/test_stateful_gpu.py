@@ -84,7 +84,7 @@ def _compare(gates, tokens, grad_out, initial, out, rev, dg, dx, di, dtype, what
 
 def _offset_copy(t, shape, k):
     """Device copy of host tensor t whose storage starts k elements off the allocation."""
-    flat = torch.empty(t.numel() + 4, dtype=t.dtype, device=DEVICE)
+    flat = torch.empty(t.numel() + 32, dtype=t.dtype, device=DEVICE)
     view = flat[k:k + t.numel()].view(shape)
     view.copy_(t.reshape(shape))
     return view
@@ -122,7 +122,8 @@ def test_tile_and_wave_boundaries(dtype, rows, T):
 
 
 @pytest.mark.parametrize("dtype", ALL_DTYPES, ids=ALL_IDS)
-@pytest.mark.parametrize("offsets", [(1, 1, 1), (3, 3, 3), (1, 0, 2)], ids=["same1", "same3", "mixed"])
+@pytest.mark.parametrize("offsets", [(1, 1, 1), (3, 3, 3), (1, 0, 2), (1, 9, 17), (4, 12, 8)],
+                         ids=["same1", "same3", "mixed", "same-mod-8", "multiples-of-4"])
 @pytest.mark.parametrize("rows,T", [(6, 2048), (3, 40000), (2050, 1031), (4, 7)])
 def test_unaligned_base_pointer(dtype, offsets, rows, T):
     _run_and_compare(rows, T, dtype, seed=9, what="offset views", offsets=offsets)
