@@ -153,3 +153,25 @@ def test_module_surface_matches_reference():
     for mod in (scalar, cscan):
         assert hasattr(mod, "scan") and hasattr(mod, "Scan")
         assert issubclass(mod.Scan, torch.autograd.Function)
+
+
+def test_wheel_carries_library_and_header(tmp_path):
+    """The wheel is a platform wheel with the prebuilt library and the C header
+    inside the package, under the reference's distribution name
+    (pyproject.toml:6 of the reference)."""
+    import subprocess
+    import sys
+    import zipfile
+
+    src = ROOT / "accelerated-scan_amd"
+    subprocess.run(
+        [sys.executable, "setup.py", "-q", "egg_info", "--egg-base", str(tmp_path),
+         "bdist_wheel", "-d", str(tmp_path / "dist"), "-b", str(tmp_path / "build")],
+        cwd=src, check=True, capture_output=True,
+    )
+    (wheel,) = (tmp_path / "dist").glob("*.whl")
+    assert wheel.name.startswith("accelerated_scan-") and wheel.name.endswith("-py3-none-linux_x86_64.whl")
+    names = {n.split("accelerated_scan/", 1)[1] for n in zipfile.ZipFile(wheel).namelist() if "accelerated_scan/" in n}
+    assert {"libascan.so", "include/ascan.h", "__init__.py", "_abi.py", "_ops.py", "warp.py", "scalar.py",
+            "complex.py", "stateful.py"} <= names
+    assert not (src / "accelerated_scan" / "include").exists()  # the header copy is temporary
