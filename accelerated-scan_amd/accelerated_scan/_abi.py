@@ -7,6 +7,7 @@ the ``ASCAN_LIBRARY`` environment variable.
 """
 
 import ctypes
+import functools
 import os
 from pathlib import Path
 
@@ -136,22 +137,40 @@ def dtype_code(dtype: torch.dtype, token_dtype: torch.dtype = None) -> int:
         ) from None
 
 
+def _stream_handle(index: int) -> int:
+    """hipStream_t of torch's current stream on device ``index`` as an integer."""
+    return torch.cuda.current_stream(index).cuda_stream
+
+
+# torch keeps a direct accessor for the same handle (what its own compiled
+# kernels launch on); it skips building a Stream object, several microseconds
+# per call that matter for short sequences.
+_stream_handle = getattr(torch._C, "_cuda_getCurrentRawStream", _stream_handle)
+
+
 def _launch(device: torch.device, call) -> None:
     """Run ``call(stream_handle)`` with ``device`` current (kernels launch on the
     current device) and map the status."""
-    if device.index is None or device.index == torch.cuda.current_device():
-        status = call(torch.cuda.current_stream(device).cuda_stream)
+    current = torch.cuda.current_device()
+    index = current if device.index is None else device.index
+    if index == current:
+        status = call(_stream_handle(index))
     else:
-        with torch.cuda.device(device):
-            status = call(torch.cuda.current_stream(device).cuda_stream)
+        with torch.cuda.device(index):
+            status = call(_stream_handle(index))
     if status:
         check(status)
+
+
+@functools.lru_cache(maxsize=1024)
+def _workspace_bytes(rows: int, seqlen: int, code: int) -> int:
+    return (_lib or load()).ascan_workspace_bytes(rows, seqlen, code)
 
 
 def _workspace(lib, rows: int, seqlen: int, code: int, device: torch.device):
     """Table for split rows (few rows, long sequences), or None.  Freed by the
     caching allocator in stream order after the kernels that use it."""
-    nbytes = lib.ascan_workspace_bytes(rows, seqlen, code)
+    nbytes = _workspace_bytes(rows, seqlen, code)
     if nbytes == 0:
         return None
     return torch.empty(nbytes, dtype=torch.uint8, device=device)

@@ -28,6 +28,26 @@ def _check_dtype(t: torch.Tensor) -> None:
         )
 
 
+def _check_launch(tensors, names) -> None:
+    """Device, layout, dtype and shape checks shared by the two launchers; the
+    first tensor is the yardstick.  The passing case builds no message."""
+    first = tensors[0]
+    dtype, shape, device = first.dtype, first.shape, first.device
+    for t in tensors:
+        if not (t.is_cuda and t.dtype == dtype and t.shape == shape and t.device == device and t.is_contiguous()):
+            break
+    else:
+        if dtype in _REAL_DTYPES:
+            return
+    for t, name in zip(tensors, names):
+        _require(t.is_cuda, f"{name} to be a device tensor")
+        _require(t.is_contiguous(), f"{name} to be contiguous")
+        _require(t.dtype == dtype, f"{name} to have the dtype of {names[0]}")
+        _require(t.shape == shape, f"{name} to have the shape of {names[0]}")
+        _require(t.device == device, f"{name} to be on the device of {names[0]}")
+    _check_dtype(first)
+
+
 def warpscan_forward(gates, tokens, out, reverse=False):
     """Write the scan of (gates, tokens) into ``out`` and return ``out``.
 
@@ -35,17 +55,7 @@ def warpscan_forward(gates, tokens, out, reverse=False):
     contiguous inputs, one dtype for all three.  ``reverse=True`` solves
     ``y[t] = gates[t] * y[t+1] + tokens[t]``.
     """
-    _require(tokens.is_cuda, "tokens to be a device tensor")
-    _require(gates.is_cuda, "gates to be a device tensor")
-    _require(out.is_cuda, "out to be a device tensor")
-    _require(tokens.is_contiguous(), "tokens to be contiguous")
-    _require(gates.is_contiguous(), "gates to be contiguous")
-    _require(out.is_contiguous(), "out to be contiguous")
-    _require(tokens.dtype == gates.dtype, "tokens and gates of one dtype")
-    _require(tokens.dtype == out.dtype, "tokens and out of one dtype")
-    _require(gates.shape == tokens.shape and out.shape == tokens.shape, "gates, tokens and out of one shape")
-    _require(gates.device == tokens.device and out.device == tokens.device, "all tensors on one device")
-    _check_dtype(gates)
+    _check_launch((tokens, gates, out), ("tokens", "gates", "out"))
     _abi.forward(gates, tokens, out, reverse)
     return out
 
@@ -56,15 +66,8 @@ def warpscan_backward(gates, output, outGrad, gateGradOut, tokenGradOut):
     ``output`` is the forward result, ``outGrad`` the incoming gradient.
     Checks mirror accelerated_scan/warp.cuh:407-421.
     """
-    tensors = (gates, output, outGrad, gateGradOut, tokenGradOut)
-    names = ("gates", "output", "outGrad", "gateGradOut", "tokenGradOut")
-    for t, name in zip(tensors, names):
-        _require(t.is_cuda, f"{name} to be a device tensor")
-        _require(t.is_contiguous(), f"{name} to be contiguous")
-        _require(t.dtype == gates.dtype, f"{name} to have the dtype of gates")
-        _require(t.shape == gates.shape, f"{name} to have the shape of gates")
-        _require(t.device == gates.device, f"{name} to be on the device of gates")
-    _check_dtype(gates)
+    _check_launch((gates, output, outGrad, gateGradOut, tokenGradOut),
+                  ("gates", "output", "outGrad", "gateGradOut", "tokenGradOut"))
     _abi.backward(gates, output, outGrad, gateGradOut, tokenGradOut)
 
 

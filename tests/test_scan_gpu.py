@@ -527,7 +527,7 @@ def test_device_side_validation():
     from accelerated_scan import warp
 
     g = torch.rand(1, 4, 64, device=DEVICE)
-    with pytest.raises(RuntimeError, match="one dtype"):
+    with pytest.raises(RuntimeError, match="dtype of tokens"):
         warp.warpscan_forward(g, g.half(), torch.empty_like(g), False)
     with pytest.raises(RuntimeError, match="unsupported tensor dtype"):
         warp.scan(g.double(), g.double())
