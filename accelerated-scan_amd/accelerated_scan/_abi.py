@@ -13,7 +13,10 @@ from pathlib import Path
 
 import torch
 
-ABI_VERSION = 3
+ABI_VERSION = 4
+
+# ascan_gate codes of include/ascan.h
+GATE_IDENTITY, GATE_SIGMOID = 0, 1
 
 # ascan_dtype codes of include/ascan.h
 F32, BF16, F16, C64, C64_REAL_TOKENS = 0, 1, 2, 3, 4
@@ -62,6 +65,19 @@ _SIGNATURES = {
         [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p,
          ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p,
          ctypes.c_int64, ctypes.c_int64, ctypes.c_int,
+         ctypes.c_void_p, ctypes.c_size_t, ctypes.c_void_p],
+    ),
+    "ascan_forward_gated": (
+        ctypes.c_int,
+        [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p,
+         ctypes.c_int64, ctypes.c_int64, ctypes.c_int, ctypes.c_int,
+         ctypes.c_void_p, ctypes.c_size_t, ctypes.c_void_p],
+    ),
+    "ascan_backward_gated": (
+        ctypes.c_int,
+        [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p,
+         ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p,
+         ctypes.c_int64, ctypes.c_int64, ctypes.c_int, ctypes.c_int,
          ctypes.c_void_p, ctypes.c_size_t, ctypes.c_void_p],
     ),
     "ascan_status_string": (ctypes.c_char_p, [ctypes.c_int]),
@@ -239,6 +255,41 @@ def backward(gates, states, grad_out, d_gates, d_tokens, workspace=None, initial
         _launch(gates.device, lambda stream: lib.ascan_backward_split(
             gates.data_ptr(), states.data_ptr(), grad_out.data_ptr(), d_gates.data_ptr(), d_tokens.data_ptr(),
             rows, seqlen, code, workspace.data_ptr(), workspace.numel(), stream))
+
+
+def _ptr(t):
+    return t.data_ptr() if t is not None else None
+
+
+def forward_gated(gate_inputs, tokens, out, gate: int, workspace=None, initial=None) -> None:
+    """Forward scan whose gates are ``gate`` (an ascan_gate code) of ``gate_inputs``."""
+    lib = _lib or load()
+    seqlen = tokens.shape[-1]
+    rows = tokens.numel() // seqlen if seqlen else 0
+    code = dtype_code(gate_inputs.dtype, tokens.dtype)
+    if workspace is None:
+        workspace = _workspace(lib, rows, seqlen, code, tokens.device)
+    _check_state(initial, out, "initial")
+    _launch(tokens.device, lambda stream: lib.ascan_forward_gated(
+        gate_inputs.data_ptr(), tokens.data_ptr(), _ptr(initial), out.data_ptr(), rows, seqlen, code, gate,
+        _ptr(workspace), workspace.numel() if workspace is not None else 0, stream))
+
+
+def backward_gated(gate_inputs, states, grad_out, d_gate_inputs, d_tokens, gate: int, workspace=None,
+                   initial=None, d_initial=None) -> None:
+    """Backward of ``forward_gated``: gradients of the gate inputs, the tokens and the initial state."""
+    lib = _lib or load()
+    seqlen = gate_inputs.shape[-1]
+    rows = gate_inputs.numel() // seqlen if seqlen else 0
+    code = dtype_code(gate_inputs.dtype, d_tokens.dtype)
+    if workspace is None:
+        workspace = _workspace(lib, rows, seqlen, code, gate_inputs.device)
+    _check_state(initial, states, "initial")
+    _check_state(d_initial, states, "d_initial")
+    _launch(gate_inputs.device, lambda stream: lib.ascan_backward_gated(
+        gate_inputs.data_ptr(), states.data_ptr(), _ptr(initial), grad_out.data_ptr(), d_gate_inputs.data_ptr(),
+        d_tokens.data_ptr(), _ptr(d_initial), rows, seqlen, code, gate,
+        _ptr(workspace), workspace.numel() if workspace is not None else 0, stream))
 
 
 def workspace_timeouts(workspace) -> int:

@@ -70,6 +70,35 @@ def _(gates, states, initial, grad_out, real_tokens):
     return torch.empty_like(gates), _empty_token_grad(gates, real_tokens), torch.empty_like(initial)
 
 
+@torch.library.custom_op("accelerated_scan::scan_forward_gated", mutates_args=())
+def scan_forward_gated(gate_inputs: torch.Tensor, tokens: torch.Tensor, initial: torch.Tensor, gate: int) -> torch.Tensor:
+    out = torch.empty_like(gate_inputs)
+    _abi.forward_gated(gate_inputs, tokens, out, gate, initial=initial)
+    return out
+
+
+@scan_forward_gated.register_fake
+def _(gate_inputs, tokens, initial, gate):
+    return torch.empty_like(gate_inputs)
+
+
+@torch.library.custom_op("accelerated_scan::scan_backward_gated", mutates_args=())
+def scan_backward_gated(
+    gate_inputs: torch.Tensor, states: torch.Tensor, initial: torch.Tensor, grad_out: torch.Tensor, gate: int
+) -> Tuple[torch.Tensor, torch.Tensor, torch.Tensor]:
+    d_gate_inputs = torch.empty_like(gate_inputs)
+    d_tokens = torch.empty_like(gate_inputs)
+    d_initial = torch.zeros_like(initial)  # stays zero for an empty sequence
+    _abi.backward_gated(gate_inputs, states, grad_out, d_gate_inputs, d_tokens, gate, initial=initial,
+                        d_initial=d_initial)
+    return d_gate_inputs, d_tokens, d_initial
+
+
+@scan_backward_gated.register_fake
+def _(gate_inputs, states, initial, grad_out, gate):
+    return torch.empty_like(gate_inputs), torch.empty_like(gate_inputs), torch.empty_like(initial)
+
+
 def _empty_token_grad(gates: torch.Tensor, real_tokens: bool) -> torch.Tensor:
     """Token gradient buffer: real when complex gates were scanned over real tokens."""
     if real_tokens and gates.is_complex():

@@ -1,0 +1,85 @@
+"""Scans whose gates come out of a sigmoid, with the sigmoid done inside the kernels.
+
+``sigmoid_scan(gate_logits, tokens)`` equals
+``warp.scan(torch.sigmoid(gate_logits), tokens)`` and is differentiable in the
+logits, the tokens and the optional initial state, but never materialises the
+gates: the forward kernel reads the logits and applies the sigmoid in
+registers, the backward kernel writes the gradient of the logits directly.
+Against the unfused pair of calls that saves the sigmoid's forward pass (one
+read, one write), its backward pass (two reads, one write) and the saved gates
+tensor.
+
+The reference's ``scan`` takes finished gates (accelerated_scan/warp.py:68-83);
+the linear-RNN layers that call it (README.md:8,42 of the reference) typically
+compute them with a sigmoid just before the scan.
+"""
+
+import torch
+
+from . import _abi, _ops
+
+_REAL_DTYPES = (torch.float32, torch.bfloat16, torch.float16)
+
+
+def _check(gate_logits, tokens, initial):
+    if gate_logits.dim() != 3 or tokens.shape != gate_logits.shape:
+        raise RuntimeError("accelerated_scan: expected gate_logits and tokens of one shape (B, C, T)")
+    if gate_logits.dtype not in _REAL_DTYPES or tokens.dtype != gate_logits.dtype:
+        raise RuntimeError(
+            f"accelerated_scan: unsupported tensor dtypes {gate_logits.dtype}, {tokens.dtype}: "
+            "expecting gate_logits and tokens both bfloat16, float16 or float32"
+        )
+    if not (gate_logits.is_cuda and tokens.is_cuda and initial.is_cuda):
+        raise RuntimeError("accelerated_scan: expected gate_logits, tokens and initial to be device tensors")
+    if not (gate_logits.is_contiguous() and tokens.is_contiguous()):
+        raise RuntimeError("accelerated_scan: expected gate_logits and tokens to be contiguous")
+    if initial.shape != gate_logits.shape[:-1] or initial.dtype != gate_logits.dtype:
+        raise RuntimeError(
+            f"accelerated_scan: expected initial of shape {tuple(gate_logits.shape[:-1])} and dtype "
+            f"{gate_logits.dtype}, got {tuple(initial.shape)} and {initial.dtype}"
+        )
+
+
+class SigmoidScan(torch.autograd.Function):
+    """Autograd node: saves (gate_logits, states, initial); no gates tensor exists."""
+
+    @staticmethod
+    def forward(ctx, gate_logits, tokens, initial):
+        _check(gate_logits, tokens, initial)
+        initial = initial.contiguous()
+        if _ops.capturing():
+            states = _ops.scan_forward_gated(gate_logits, tokens, initial, _abi.GATE_SIGMOID)
+        else:
+            states = torch.empty_like(gate_logits)
+            _abi.forward_gated(gate_logits, tokens, states, _abi.GATE_SIGMOID, initial=initial)
+        ctx.save_for_backward(gate_logits, states, initial)
+        return states
+
+    @staticmethod
+    def backward(ctx, grad_output):
+        gate_logits, states, initial = ctx.saved_tensors
+        grad_output = grad_output.contiguous()
+        if _ops.capturing():
+            return _ops.scan_backward_gated(gate_logits, states, initial, grad_output, _abi.GATE_SIGMOID)
+        d_logits = torch.empty_like(gate_logits)
+        d_tokens = torch.empty_like(gate_logits)
+        d_initial = torch.zeros_like(initial)  # stays zero for an empty sequence
+        _abi.backward_gated(gate_logits, states, grad_output, d_logits, d_tokens, _abi.GATE_SIGMOID,
+                            initial=initial, d_initial=d_initial)
+        return d_logits, d_tokens, d_initial
+
+
+def sigmoid_scan(gate_logits, tokens, initial=None):
+    """Solve ``x[t] = sigmoid(gate_logits[t]) * x[t-1] + tokens[t]``.
+
+    Arguments:
+        gate_logits (torch.Tensor): shape (B, C, T), contiguous; fp32, bf16 or fp16.
+        tokens (torch.Tensor): shape (B, C, T), contiguous, same dtype.
+        initial (torch.Tensor, optional): shape (B, C), the state ``x[-1]`` (zero if absent).
+
+    Returns:
+        (torch.Tensor): the states, shape (B, C, T).
+    """
+    if initial is None:
+        initial = torch.zeros(gate_logits.shape[:-1], dtype=gate_logits.dtype, device=gate_logits.device)
+    return SigmoidScan.apply(gate_logits, tokens, initial)

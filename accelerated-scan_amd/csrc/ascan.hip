@@ -335,6 +335,55 @@ struct TraitsC64RealTokens : TraitsC64 {
 };
 
 // ---------------------------------------------------------------------------
+// Gate activation.  The kernels can read gate pre-activations ("logits") and
+// apply the non-linearity in registers as the values are unpacked, which spares
+// the caller a pass that materialises the gates and, in the backward pass, one
+// that turns d_gates into the gradient of the logits.
+//   kGateIdentity: the stored values are the gates (the reference's operator);
+//   kGateSigmoid : gate = 1 / (1 + exp(-stored)), real dtypes only.
+// ---------------------------------------------------------------------------
+constexpr int kGateIdentity = 0, kGateSigmoid = 1;
+
+__device__ __forceinline__ float sigmoid(float v) {
+    // v_exp_f32 computes 2^x; v_rcp_f32 is accurate to 1 ulp
+    return __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(v * -1.4426950408889634f));
+}
+
+template <int ACT, class V, int N>
+__device__ __forceinline__ void activate(V (&g)[N]) {
+    if constexpr (ACT == kGateSigmoid) {
+#pragma unroll
+        for (int e = 0; e < N; ++e) g[e] = sigmoid(g[e]);
+    }
+}
+template <int ACT, class V>
+__device__ __forceinline__ V activate1(V g) {
+    if constexpr (ACT == kGateSigmoid) {
+        return sigmoid(g);
+    } else {
+        return g;
+    }
+}
+// Stored value whose activation is the identity gate 1 (for out-of-row positions).
+template <int ACT, class V>
+__device__ __forceinline__ V identity_gate() {
+    if constexpr (ACT == kGateSigmoid) {
+        return __builtin_inff();
+    } else {
+        return vone<V>();
+    }
+}
+// d gate / d stored, from the gate's value.
+template <int ACT, class V>
+__device__ __forceinline__ V gate_slope(V gate) {
+    if constexpr (ACT == kGateSigmoid) {
+        return gate * (1.0f - gate);
+    } else {
+        return vone<V>();
+    }
+}
+
+// ---------------------------------------------------------------------------
 // Vector access.  A row is addressed in "virtual" positions: position 0 is an
 // aligned boundary at or just below the row's first element -- a 128-byte one
 // when all tensors of the call sit alike on that grid, so that the 1 KiB a wave
@@ -819,7 +868,7 @@ __device__ __forceinline__ void exchange_carries_split(const V (&totA)[U], const
 // rows of a workgroup are adjacent in memory, so with W*R = 16 one tile step
 // of the workgroup covers one contiguous span of 16 sub-tiles.
 // ---------------------------------------------------------------------------
-template <class Tr, int W, int U, bool REV, bool ALIGNED, bool REGULAR, bool SPLIT>
+template <class Tr, int W, int U, bool REV, bool ALIGNED, bool REGULAR, bool SPLIT, int ACT>
 __global__ void __launch_bounds__(64 * kMaxWavesPerBlock)
     scan_forward_kernel(const typename Tr::S* __restrict__ gates, const typename Tr::TokS* __restrict__ tokens,
                         typename Tr::S* __restrict__ out, int64_t rows, int64_t T, SplitHeader* split,
@@ -889,13 +938,13 @@ __global__ void __launch_bounds__(64 * kMaxWavesPerBlock)
 #pragma unroll
             for (int j = 0; j < U; ++j) {
                 const int off = vec_offset<U, EPV, REV>(j, lane);
-                graw[j] = load_raw<Tr, ALIGNED, FULL>(gsub, off, win, vone<V>());
+                graw[j] = load_raw<Tr, ALIGNED, FULL>(gsub, off, win, identity_gate<ACT, V>());
                 traw[j] = load_tok_raw<Tr, ALIGNED, FULL>(tsub, off, win, vzero<V>());
             }
         } else {
 #pragma unroll
             for (int j = 0; j < U; ++j) {
-                graw[j] = fill_raw<Tr>(vone<V>());
+                graw[j] = fill_raw<Tr>(identity_gate<ACT, V>());
                 traw[j] = fill_raw<Tr>(vzero<V>());
             }
         }
@@ -906,6 +955,7 @@ __global__ void __launch_bounds__(64 * kMaxWavesPerBlock)
         for (int j = 0; j < U; ++j) {
             V g[EPV], t[EPV];
             Tr::unpack(graw[j], g);
+            activate<ACT>(g);
             Tr::unpack(traw[j], t);
             constexpr int e0 = REV ? EPV - 1 : 0;
             V A = g[e0];
@@ -940,6 +990,7 @@ __global__ void __launch_bounds__(64 * kMaxWavesPerBlock)
             }
             V g[EPV], t[EPV];
             Tr::unpack(graw[j], g);
+            activate<ACT>(g);
             Tr::unpack(traw[j], t);
             V x = vfma(exA[j], c, exX[j]);  // state entering this lane's vector
             c = vfma(totA[j], c, totX[j]);  // state entering the next block
@@ -977,7 +1028,7 @@ __global__ void __launch_bounds__(64 * kMaxWavesPerBlock)
 // Fused backward kernel: reverse-time scan over gate[t+1] producing d_tokens,
 // and d_gates[t] = d_tokens[t] * conj(x[t-1]) in the same pass.
 // ---------------------------------------------------------------------------
-template <class Tr, int W, int U, bool ALIGNED, bool REGULAR, bool SPLIT>
+template <class Tr, int W, int U, bool ALIGNED, bool REGULAR, bool SPLIT, int ACT>
 __global__ void __launch_bounds__(64 * kMaxWavesPerBlock)
     scan_backward_kernel(const typename Tr::S* __restrict__ gates, const typename Tr::S* __restrict__ states,
                          const typename Tr::S* __restrict__ grad_out, typename Tr::S* __restrict__ d_gates,
@@ -1029,7 +1080,7 @@ __global__ void __launch_bounds__(64 * kMaxWavesPerBlock)
     // gate 1 and grad_out 0, so with lo > 0 that g already is the gradient;
     // with lo == 0 the last factor is still missing.
     auto store_start_gradient = [&](V g_low) {
-        if (lo == 0) g_low = vmul(vconj(Tr::load1(arow)), g_low);
+        if (lo == 0) g_low = vmul(vconj(activate1<ACT>(Tr::load1(arow))), g_low);
         if (lane == 0) Tr::store1(d_initial + row, g_low);
     };
 
@@ -1061,14 +1112,14 @@ __global__ void __launch_bounds__(64 * kMaxWavesPerBlock)
 #pragma unroll
             for (int j = 0; j < U; ++j) {
                 const int off = vec_offset<U, EPV, true>(j, lane);
-                araw[j] = load_raw<Tr, ALIGNED, FULL>(asub, off, win, vone<V>());
+                araw[j] = load_raw<Tr, ALIGNED, FULL>(asub, off, win, identity_gate<ACT, V>());
                 draw[j] = load_raw<Tr, ALIGNED, FULL>(dsub, off, win, vzero<V>());
                 xraw[j] = load_raw<Tr, ALIGNED, FULL>(xsub, off, win, x_start);
             }
         } else {
 #pragma unroll
             for (int j = 0; j < U; ++j) {
-                araw[j] = fill_raw<Tr>(vone<V>());
+                araw[j] = fill_raw<Tr>(identity_gate<ACT, V>());
                 draw[j] = fill_raw<Tr>(vzero<V>());
                 xraw[j] = fill_raw<Tr>(x_start);
             }
@@ -1082,7 +1133,7 @@ __global__ void __launch_bounds__(64 * kMaxWavesPerBlock)
             const int64_t ia = sub_end < hi ? (sub_end > lo ? sub_end : lo) : hi - 1;
             int64_t ix = sub_base - 1;
             ix = ix < lo ? lo : (ix < hi ? ix : hi - 1);
-            const V av = Tr::load1(arow + ia);
+            const V av = activate1<ACT>(Tr::load1(arow + ia));
             const V xv = Tr::load1(xrow + ix);
             a_edge = vselect(sub_end >= lo && sub_end < hi, av, vone<V>());
             x_edge = vselect(sub_base - 1 >= lo && sub_base - 1 < hi, xv, x_start);
@@ -1100,6 +1151,7 @@ __global__ void __launch_bounds__(64 * kMaxWavesPerBlock)
         for (int j = 0; j < U; ++j) {
             V a[EPV], d[EPV], x[EPV];
             Tr::unpack(araw[j], a);
+            activate<ACT>(a);
             Tr::unpack(draw[j], d);
             Tr::unpack(xraw[j], x);
             V hi_edge, lo_edge;
@@ -1108,7 +1160,7 @@ __global__ void __launch_bounds__(64 * kMaxWavesPerBlock)
             } else {
                 V above[EPV];
                 Tr::unpack(araw[j > 0 ? j - 1 : 0], above);
-                hi_edge = read_lane<63>(above[0]);
+                hi_edge = read_lane<63>(activate1<ACT>(above[0]));
             }
             if (j == U - 1) {
                 lo_edge = x_edge;
@@ -1152,6 +1204,7 @@ __global__ void __launch_bounds__(64 * kMaxWavesPerBlock)
             }
             V a[EPV], d[EPV], x[EPV];
             Tr::unpack(araw[j], a);
+            activate<ACT>(a);
             Tr::unpack(draw[j], d);
             Tr::unpack(xraw[j], x);
             V gr = vfma(exA[j], c, exX[j]);  // g entering this lane's vector from above
@@ -1164,6 +1217,7 @@ __global__ void __launch_bounds__(64 * kMaxWavesPerBlock)
                 gr = vfma(ga, gr, d[e]);
                 dt[e] = gr;
                 dg[e] = vmul(gr, xs);
+                if constexpr (ACT != kGateIdentity) dg[e] = vmul(dg[e], gate_slope<ACT>(a[e]));
             }
             const int off = vec_offset<U, EPV, true>(j, lane);
             if (touches) {
@@ -1300,7 +1354,7 @@ int launch_status(hipError_t e) {
     return ASCAN_OK;
 }
 
-template <class Tr, int W, bool REV, bool ALIGNED, bool REGULAR>
+template <class Tr, int W, bool REV, bool ALIGNED, bool REGULAR, int ACT>
 hipError_t launch_forward(const void* gates, const void* tokens, void* out, const void* initial, int64_t rows,
                           int64_t T, int grid, int rows_per_block, hipStream_t stream) {
     using S = typename Tr::S;
@@ -1308,12 +1362,12 @@ hipError_t launch_forward(const void* gates, const void* tokens, void* out, cons
     constexpr int U = REGULAR ? Tuning<Tr>::U : Tuning<Tr>::UG;
     const unsigned blocks = (unsigned)((rows + rows_per_block - 1) / rows_per_block);
     const unsigned threads = 64u * W * rows_per_block;
-    return launch(scan_forward_kernel<Tr, W, U, REV, ALIGNED, REGULAR, false>, blocks, threads, stream,
+    return launch(scan_forward_kernel<Tr, W, U, REV, ALIGNED, REGULAR, false, ACT>, blocks, threads, stream,
                   static_cast<const S*>(gates), static_cast<const TokS*>(tokens), static_cast<S*>(out), rows, T,
                   static_cast<SplitHeader*>(nullptr), static_cast<const S*>(initial), grid);
 }
 
-template <class Tr, int W, bool ALIGNED, bool REGULAR>
+template <class Tr, int W, bool ALIGNED, bool REGULAR, int ACT>
 hipError_t launch_backward(const void* gates, const void* states, const void* grad_out, void* d_gates,
                            void* d_tokens, const void* initial, void* d_initial, int64_t rows, int64_t T, int grid,
                            int rows_per_block, hipStream_t stream) {
@@ -1322,7 +1376,7 @@ hipError_t launch_backward(const void* gates, const void* states, const void* gr
     constexpr int U = REGULAR ? Tuning<Tr>::UB : Tuning<Tr>::UBG;
     const unsigned blocks = (unsigned)((rows + rows_per_block - 1) / rows_per_block);
     const unsigned threads = 64u * W * rows_per_block;
-    return launch(scan_backward_kernel<Tr, W, U, ALIGNED, REGULAR, false>, blocks, threads, stream,
+    return launch(scan_backward_kernel<Tr, W, U, ALIGNED, REGULAR, false, ACT>, blocks, threads, stream,
                   static_cast<const S*>(gates), static_cast<const S*>(states), static_cast<const S*>(grad_out),
                   static_cast<S*>(d_gates), static_cast<TokS*>(d_tokens), rows, T,
                   static_cast<SplitHeader*>(nullptr), static_cast<const S*>(initial), static_cast<S*>(d_initial), grid);
@@ -1406,13 +1460,13 @@ int64_t host_tiles_per_row(int64_t T, int64_t tile, bool regular, const Lead& at
     return (T + head + tile - 1) / tile;
 }
 
-template <class Tr, bool REV, bool REGULAR>
+template <class Tr, bool REV, bool REGULAR, int ACT>
 hipError_t launch_forward_split(const void* gates, const void* tokens, void* out, const void* initial, int64_t rows,
                                 int64_t T, int grid, int64_t ntiles, const Workspace& ws, hipStream_t stream) {
     using S = typename Tr::S;
     using TokS = typename Tr::TokS;
     constexpr int U = REGULAR ? Tuning<Tr>::U : Tuning<Tr>::UG;
-    auto kernel = scan_forward_kernel<Tr, kSplitWaves, U, REV, true, REGULAR, true>;
+    auto kernel = scan_forward_kernel<Tr, kSplitWaves, U, REV, true, REGULAR, true, ACT>;
     const unsigned resident = resident_workgroups(kernel, 64 * kSplitWaves);
     if (resident == 0) return hipErrorInvalidConfiguration;
     const hipError_t e = reset_split_table(ws, rows, ntiles, stream);
@@ -1423,14 +1477,14 @@ hipError_t launch_forward_split(const void* gates, const void* tokens, void* out
                   static_cast<SplitHeader*>(ws.ptr), static_cast<const S*>(initial), grid);
 }
 
-template <class Tr, bool REGULAR>
+template <class Tr, bool REGULAR, int ACT>
 hipError_t launch_backward_split(const void* gates, const void* states, const void* grad_out, void* d_gates,
                                  void* d_tokens, const void* initial, void* d_initial, int64_t rows, int64_t T,
                                  int grid, int64_t ntiles, const Workspace& ws, hipStream_t stream) {
     using S = typename Tr::S;
     using TokS = typename Tr::TokS;
     constexpr int U = REGULAR ? Tuning<Tr>::UB : Tuning<Tr>::UBG;
-    auto kernel = scan_backward_kernel<Tr, kSplitWaves, U, true, REGULAR, true>;
+    auto kernel = scan_backward_kernel<Tr, kSplitWaves, U, true, REGULAR, true, ACT>;
     const unsigned resident = resident_workgroups(kernel, 64 * kSplitWaves);
     if (resident == 0) return hipErrorInvalidConfiguration;
     const hipError_t e = reset_split_table(ws, rows, ntiles, stream);
@@ -1458,9 +1512,13 @@ Access choose_access(bool same_lead, int lead, int64_t T, int64_t tile) {
     return Access::kVector;
 }
 
+// Kernels with the sigmoid gate exist for the real dtypes, forward in time.
+template <class Tr>
+constexpr bool kHasSigmoid = std::is_same<typename Tr::V, float>::value;
+
 template <class Tr>
 int forward_typed(const void* gates, const void* tokens, void* out, const void* initial, int64_t rows, int64_t T,
-                  bool reverse, const Workspace& ws, hipStream_t stream) {
+                  bool reverse, int act, const Workspace& ws, hipStream_t stream) {
     constexpr int64_t kElem = (int64_t)sizeof(typename Tr::S);
     constexpr int64_t SUB = (int64_t)Tuning<Tr>::U * 64 * Tr::EPV;    // regular kernels
     constexpr int64_t SUBG = (int64_t)Tuning<Tr>::UG * 64 * Tr::EPV;  // kernels with masking code
@@ -1477,23 +1535,32 @@ int forward_typed(const void* gates, const void* tokens, void* out, const void* 
         const bool regular = lead == 0 && T % (SUB * kSplitWaves) == 0;
         const int64_t ntiles = host_tiles_per_row<Tr>(T, (regular ? SUB : SUBG) * kSplitWaves, regular, at);
         if (want_split(rows, ntiles) && workspace_fits(ws, rows, ntiles)) {
-#define ASCAN_FWD_SPLIT(REV, REG) \
-    launch_forward_split<Tr, REV, REG>(gates, tokens, out, initial, rows, T, at.grid, ntiles, ws, stream)
-            if (regular) {
-                err = reverse ? ASCAN_FWD_SPLIT(true, true) : ASCAN_FWD_SPLIT(false, true);
+#define ASCAN_FWD_SPLIT(REV, REG, ACT) \
+    launch_forward_split<Tr, REV, REG, ACT>(gates, tokens, out, initial, rows, T, at.grid, ntiles, ws, stream)
+            if (act == kGateSigmoid) {
+                if constexpr (kHasSigmoid<Tr>) {
+                    err = regular ? ASCAN_FWD_SPLIT(false, true, kGateSigmoid) : ASCAN_FWD_SPLIT(false, false, kGateSigmoid);
+                }
+            } else if (regular) {
+                err = reverse ? ASCAN_FWD_SPLIT(true, true, kGateIdentity) : ASCAN_FWD_SPLIT(false, true, kGateIdentity);
             } else {
-                err = reverse ? ASCAN_FWD_SPLIT(true, false) : ASCAN_FWD_SPLIT(false, false);
+                err = reverse ? ASCAN_FWD_SPLIT(true, false, kGateIdentity) : ASCAN_FWD_SPLIT(false, false, kGateIdentity);
             }
 #undef ASCAN_FWD_SPLIT
             return launch_status(err);
         }
     }
-#define ASCAN_FWD(WV, AL, REG)                                                                     \
-    do {                                                                                           \
-        if (reverse)                                                                               \
-            err = launch_forward<Tr, WV, true, AL, REG>(gates, tokens, out, initial, rows, T, at.grid, R, stream);  \
-        else                                                                                                       \
-            err = launch_forward<Tr, WV, false, AL, REG>(gates, tokens, out, initial, rows, T, at.grid, R, stream); \
+#define ASCAN_FWD_ARGS gates, tokens, out, initial, rows, T, at.grid, R, stream
+#define ASCAN_FWD(WV, AL, REG)                                                                  \
+    do {                                                                                        \
+        if (act == kGateSigmoid) {                                                              \
+            if constexpr (kHasSigmoid<Tr>)                                                      \
+                err = launch_forward<Tr, WV, false, AL, REG, kGateSigmoid>(ASCAN_FWD_ARGS);     \
+        } else if (reverse) {                                                                   \
+            err = launch_forward<Tr, WV, true, AL, REG, kGateIdentity>(ASCAN_FWD_ARGS);         \
+        } else {                                                                                \
+            err = launch_forward<Tr, WV, false, AL, REG, kGateIdentity>(ASCAN_FWD_ARGS);        \
+        }                                                                                       \
     } while (0)
 #define ASCAN_FWD_W(AL, REG)                            \
     switch (plan.waves_per_row) {                       \
@@ -1512,12 +1579,13 @@ int forward_typed(const void* gates, const void* tokens, void* out, const void* 
     }
 #undef ASCAN_FWD_W
 #undef ASCAN_FWD
+#undef ASCAN_FWD_ARGS
     return launch_status(err);
 }
 
 template <class Tr>
 int backward_typed(const void* gates, const void* states, const void* grad_out, void* d_gates, void* d_tokens,
-                   const void* initial, void* d_initial, int64_t rows, int64_t T, const Workspace& ws,
+                   const void* initial, void* d_initial, int64_t rows, int64_t T, int act, const Workspace& ws,
                    hipStream_t stream) {
     constexpr int64_t kElem = (int64_t)sizeof(typename Tr::S);
     constexpr int64_t SUB = (int64_t)Tuning<Tr>::UB * 64 * Tr::EPV;    // regular kernels
@@ -1535,16 +1603,30 @@ int backward_typed(const void* gates, const void* states, const void* grad_out, 
         const bool regular = lead == 0 && T % (SUB * kSplitWaves) == 0;
         const int64_t ntiles = host_tiles_per_row<Tr>(T, (regular ? SUB : SUBG) * kSplitWaves, regular, at);
         if (want_split(rows, ntiles) && workspace_fits(ws, rows, ntiles)) {
-            err = regular ? launch_backward_split<Tr, true>(gates, states, grad_out, d_gates, d_tokens, initial,
-                                                            d_initial, rows, T, at.grid, ntiles, ws, stream)
-                          : launch_backward_split<Tr, false>(gates, states, grad_out, d_gates, d_tokens, initial,
-                                                             d_initial, rows, T, at.grid, ntiles, ws, stream);
+#define ASCAN_BWD_SPLIT(REG, ACT)                                                                              \
+    launch_backward_split<Tr, REG, ACT>(gates, states, grad_out, d_gates, d_tokens, initial, d_initial, rows, T, \
+                                        at.grid, ntiles, ws, stream)
+            if (act == kGateSigmoid) {
+                if constexpr (kHasSigmoid<Tr>) {
+                    err = regular ? ASCAN_BWD_SPLIT(true, kGateSigmoid) : ASCAN_BWD_SPLIT(false, kGateSigmoid);
+                }
+            } else {
+                err = regular ? ASCAN_BWD_SPLIT(true, kGateIdentity) : ASCAN_BWD_SPLIT(false, kGateIdentity);
+            }
+#undef ASCAN_BWD_SPLIT
             return launch_status(err);
         }
     }
-#define ASCAN_BWD(WV, AL, REG) \
-    err = launch_backward<Tr, WV, AL, REG>(gates, states, grad_out, d_gates, d_tokens, initial, d_initial, rows, T, \
-                                           at.grid, R, stream)
+#define ASCAN_BWD_ARGS gates, states, grad_out, d_gates, d_tokens, initial, d_initial, rows, T, at.grid, R, stream
+#define ASCAN_BWD(WV, AL, REG)                                                              \
+    do {                                                                                    \
+        if (act == kGateSigmoid) {                                                          \
+            if constexpr (kHasSigmoid<Tr>)                                                  \
+                err = launch_backward<Tr, WV, AL, REG, kGateSigmoid>(ASCAN_BWD_ARGS);       \
+        } else {                                                                            \
+            err = launch_backward<Tr, WV, AL, REG, kGateIdentity>(ASCAN_BWD_ARGS);          \
+        }                                                                                   \
+    } while (0)
 #define ASCAN_BWD_W(AL, REG)                            \
     switch (plan.waves_per_row) {                       \
         case 1: ASCAN_BWD(1, AL, REG); break;           \
@@ -1562,6 +1644,7 @@ int backward_typed(const void* gates, const void* states, const void* grad_out, 
     }
 #undef ASCAN_BWD_W
 #undef ASCAN_BWD
+#undef ASCAN_BWD_ARGS
     return launch_status(err);
 }
 
@@ -1584,10 +1667,28 @@ bool element_aligned(const void* p, size_t es) { return (reinterpret_cast<uintpt
 // Largest row count one launch can address: gridDim.x is limited to 2^31-1.
 constexpr int64_t kMaxBlocks = 2147483647LL;
 
+// Calls fn with a value of the traits type that `dtype` selects.
+template <class Fn>
+int with_traits(int dtype, Fn fn) {
+    switch (dtype) {
+        case ASCAN_F32: return fn(TraitsF32{});
+        case ASCAN_BF16: return fn(TraitsBF16{});
+        case ASCAN_F16: return fn(TraitsF16{});
+        case ASCAN_C64: return fn(TraitsC64{});
+        default: return fn(TraitsC64RealTokens{});
+    }
+}
+
+bool activation_supported(int act, int dtype, bool reverse) {
+    if (act == kGateIdentity) return true;
+    return act == kGateSigmoid && !reverse && (dtype == ASCAN_F32 || dtype == ASCAN_BF16 || dtype == ASCAN_F16);
+}
+
 int forward_checked(const void* gates, const void* tokens, void* out, const void* initial, int64_t rows,
-                    int64_t seqlen, int dtype, int reverse, const Workspace& ws, void* stream) {
+                    int64_t seqlen, int dtype, int reverse, int act, const Workspace& ws, void* stream) {
     const size_t es = element_size(dtype);
     if (es == 0) return ASCAN_ERR_BAD_DTYPE;
+    if (!activation_supported(act, dtype, reverse != 0)) return ASCAN_ERR_BAD_ACTIVATION;
     if (rows < 0 || seqlen < 0 || rows > kMaxBlocks) return ASCAN_ERR_BAD_SHAPE;
     if (rows == 0 || seqlen == 0) return ASCAN_OK;
     if (!gates || !tokens || !out) return ASCAN_ERR_NULL_POINTER;
@@ -1595,21 +1696,17 @@ int forward_checked(const void* gates, const void* tokens, void* out, const void
         !element_aligned(initial, es))
         return ASCAN_ERR_MISALIGNED;
     hipStream_t s = static_cast<hipStream_t>(stream);
-    const bool rev = reverse != 0;
-    switch (dtype) {
-        case ASCAN_F32: return forward_typed<TraitsF32>(gates, tokens, out, initial, rows, seqlen, rev, ws, s);
-        case ASCAN_BF16: return forward_typed<TraitsBF16>(gates, tokens, out, initial, rows, seqlen, rev, ws, s);
-        case ASCAN_F16: return forward_typed<TraitsF16>(gates, tokens, out, initial, rows, seqlen, rev, ws, s);
-        case ASCAN_C64: return forward_typed<TraitsC64>(gates, tokens, out, initial, rows, seqlen, rev, ws, s);
-        default: return forward_typed<TraitsC64RealTokens>(gates, tokens, out, initial, rows, seqlen, rev, ws, s);
-    }
+    return with_traits(dtype, [&](auto traits) {
+        return forward_typed<decltype(traits)>(gates, tokens, out, initial, rows, seqlen, reverse != 0, act, ws, s);
+    });
 }
 
 int backward_checked(const void* gates, const void* states, const void* grad_out, void* d_gates, void* d_tokens,
-                     const void* initial, void* d_initial, int64_t rows, int64_t seqlen, int dtype,
+                     const void* initial, void* d_initial, int64_t rows, int64_t seqlen, int dtype, int act,
                      const Workspace& ws, void* stream) {
     const size_t es = element_size(dtype);
     if (es == 0) return ASCAN_ERR_BAD_DTYPE;
+    if (!activation_supported(act, dtype, false)) return ASCAN_ERR_BAD_ACTIVATION;
     if (rows < 0 || seqlen < 0 || rows > kMaxBlocks) return ASCAN_ERR_BAD_SHAPE;
     if (rows == 0 || seqlen == 0) return ASCAN_OK;
     if (!gates || !states || !grad_out || !d_gates || !d_tokens) return ASCAN_ERR_NULL_POINTER;
@@ -1618,23 +1715,10 @@ int backward_checked(const void* gates, const void* states, const void* grad_out
         !element_aligned(initial, es) || !element_aligned(d_initial, es))
         return ASCAN_ERR_MISALIGNED;
     hipStream_t s = static_cast<hipStream_t>(stream);
-    switch (dtype) {
-        case ASCAN_F32:
-            return backward_typed<TraitsF32>(gates, states, grad_out, d_gates, d_tokens, initial, d_initial, rows,
-                                             seqlen, ws, s);
-        case ASCAN_BF16:
-            return backward_typed<TraitsBF16>(gates, states, grad_out, d_gates, d_tokens, initial, d_initial, rows,
-                                             seqlen, ws, s);
-        case ASCAN_F16:
-            return backward_typed<TraitsF16>(gates, states, grad_out, d_gates, d_tokens, initial, d_initial, rows,
-                                             seqlen, ws, s);
-        case ASCAN_C64:
-            return backward_typed<TraitsC64>(gates, states, grad_out, d_gates, d_tokens, initial, d_initial, rows,
-                                             seqlen, ws, s);
-        default:
-            return backward_typed<TraitsC64RealTokens>(gates, states, grad_out, d_gates, d_tokens, initial,
-                                                       d_initial, rows, seqlen, ws, s);
-    }
+    return with_traits(dtype, [&](auto traits) {
+        return backward_typed<decltype(traits)>(gates, states, grad_out, d_gates, d_tokens, initial, d_initial, rows,
+                                                seqlen, act, ws, s);
+    });
 }
 
 }  // namespace
@@ -1643,13 +1727,14 @@ extern "C" {
 
 int ascan_forward(const void* gates, const void* tokens, void* out, int64_t rows, int64_t seqlen, int dtype,
                   int reverse, void* stream) {
-    return forward_checked(gates, tokens, out, nullptr, rows, seqlen, dtype, reverse, Workspace{nullptr, 0}, stream);
+    return forward_checked(gates, tokens, out, nullptr, rows, seqlen, dtype, reverse, ASCAN_GATE_IDENTITY,
+                           Workspace{nullptr, 0}, stream);
 }
 
 int ascan_backward(const void* gates, const void* states, const void* grad_out, void* d_gates, void* d_tokens,
                    int64_t rows, int64_t seqlen, int dtype, void* stream) {
     return backward_checked(gates, states, grad_out, d_gates, d_tokens, nullptr, nullptr, rows, seqlen, dtype,
-                            Workspace{nullptr, 0}, stream);
+                            ASCAN_GATE_IDENTITY, Workspace{nullptr, 0}, stream);
 }
 
 size_t ascan_workspace_bytes(int64_t rows, int64_t seqlen, int dtype) {
@@ -1667,7 +1752,7 @@ size_t ascan_workspace_bytes(int64_t rows, int64_t seqlen, int dtype) {
 
 int ascan_forward_split(const void* gates, const void* tokens, void* out, int64_t rows, int64_t seqlen, int dtype,
                         int reverse, void* workspace, size_t workspace_bytes, void* stream) {
-    return forward_checked(gates, tokens, out, nullptr, rows, seqlen, dtype, reverse,
+    return forward_checked(gates, tokens, out, nullptr, rows, seqlen, dtype, reverse, ASCAN_GATE_IDENTITY,
                            Workspace{workspace, workspace_bytes}, stream);
 }
 
@@ -1675,13 +1760,13 @@ int ascan_backward_split(const void* gates, const void* states, const void* grad
                          void* d_tokens, int64_t rows, int64_t seqlen, int dtype, void* workspace,
                          size_t workspace_bytes, void* stream) {
     return backward_checked(gates, states, grad_out, d_gates, d_tokens, nullptr, nullptr, rows, seqlen, dtype,
-                            Workspace{workspace, workspace_bytes}, stream);
+                            ASCAN_GATE_IDENTITY, Workspace{workspace, workspace_bytes}, stream);
 }
 
 int ascan_forward_from(const void* gates, const void* tokens, const void* initial, void* out, int64_t rows,
                        int64_t seqlen, int dtype, int reverse, void* workspace, size_t workspace_bytes,
                        void* stream) {
-    return forward_checked(gates, tokens, out, initial, rows, seqlen, dtype, reverse,
+    return forward_checked(gates, tokens, out, initial, rows, seqlen, dtype, reverse, ASCAN_GATE_IDENTITY,
                            Workspace{workspace, workspace_bytes}, stream);
 }
 
@@ -1689,7 +1774,20 @@ int ascan_backward_from(const void* gates, const void* states, const void* initi
                         void* d_gates, void* d_tokens, void* d_initial, int64_t rows, int64_t seqlen, int dtype,
                         void* workspace, size_t workspace_bytes, void* stream) {
     return backward_checked(gates, states, grad_out, d_gates, d_tokens, initial, d_initial, rows, seqlen, dtype,
-                            Workspace{workspace, workspace_bytes}, stream);
+                            ASCAN_GATE_IDENTITY, Workspace{workspace, workspace_bytes}, stream);
+}
+
+int ascan_forward_gated(const void* gate_inputs, const void* tokens, const void* initial, void* out, int64_t rows,
+                        int64_t seqlen, int dtype, int gate, void* workspace, size_t workspace_bytes, void* stream) {
+    return forward_checked(gate_inputs, tokens, out, initial, rows, seqlen, dtype, 0, gate,
+                           Workspace{workspace, workspace_bytes}, stream);
+}
+
+int ascan_backward_gated(const void* gate_inputs, const void* states, const void* initial, const void* grad_out,
+                         void* d_gate_inputs, void* d_tokens, void* d_initial, int64_t rows, int64_t seqlen,
+                         int dtype, int gate, void* workspace, size_t workspace_bytes, void* stream) {
+    return backward_checked(gate_inputs, states, grad_out, d_gate_inputs, d_tokens, initial, d_initial, rows, seqlen,
+                            dtype, gate, Workspace{workspace, workspace_bytes}, stream);
 }
 
 unsigned int ascan_workspace_timeouts(const void* workspace_header_copy) {
@@ -1704,6 +1802,8 @@ const char* ascan_status_string(int status) {
         case ASCAN_ERR_BAD_DTYPE: return "unsupported dtype: expecting float32, bfloat16, float16, complex64 or complex64 with float32 tokens";
         case ASCAN_ERR_MISALIGNED: return "a buffer is not aligned to its element size";
         case ASCAN_ERR_LAUNCH: return "the HIP runtime reported a launch error";
+        case ASCAN_ERR_BAD_ACTIVATION:
+            return "unsupported gate activation: expecting identity, or sigmoid with float32, bfloat16 or float16";
         default: return "unknown status";
     }
 }

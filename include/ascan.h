@@ -47,7 +47,7 @@
 extern "C" {
 #endif
 
-#define ASCAN_ABI_VERSION 3
+#define ASCAN_ABI_VERSION 4
 
 /* Element types of the tensors of a call. */
 enum ascan_dtype {
@@ -72,7 +72,14 @@ enum ascan_status {
     ASCAN_ERR_BAD_SHAPE     = 2, /* rows < 0, seqlen < 0, or rows too large for one grid */
     ASCAN_ERR_BAD_DTYPE     = 3, /* dtype is not an ascan_dtype (warp.cuh:390-391) */
     ASCAN_ERR_MISALIGNED    = 4, /* a pointer is not aligned to its element size */
-    ASCAN_ERR_LAUNCH        = 5  /* the HIP runtime refused the launch (see ascan_last_hip_error) */
+    ASCAN_ERR_LAUNCH        = 5, /* the HIP runtime refused the launch (see ascan_last_hip_error) */
+    ASCAN_ERR_BAD_ACTIVATION = 6 /* gate is not an ascan_gate, or not available for this dtype */
+};
+
+/* What the kernels make of the stored gate values (the *_gated entry points). */
+enum ascan_gate {
+    ASCAN_GATE_IDENTITY = 0, /* stored values are the gates: the reference's operator */
+    ASCAN_GATE_SIGMOID  = 1  /* gate = 1 / (1 + exp(-stored)); float32, bfloat16, float16 */
 };
 
 /*
@@ -166,6 +173,33 @@ int ascan_backward_from(const void* gates, const void* states, const void* initi
                         const void* grad_out, void* d_gates, void* d_tokens, void* d_initial,
                         int64_t rows, int64_t seqlen, int dtype,
                         void* workspace, size_t workspace_bytes, void* stream);
+
+/*
+ * Scans whose gates come out of a non-linearity, applied in registers: the
+ * caller passes the pre-activations and receives the gradient with respect to
+ * them, instead of running one elementwise pass that materialises the gates and
+ * another that turns d_gates into the gradient of the pre-activations (the
+ * linear-RNN layers that call the scan, README.md:8,42 of the reference,
+ * typically compute their gates with a sigmoid just before it).
+ *
+ *     gate[t]          = act(gate_inputs[t])
+ *     forward          : x[t] = gate[t] * x[t-1] + tokens[t],   x[-1] = initial (NULL: 0)
+ *     d_gate_inputs[t] = g[t] * x[t-1] * act'(gate_inputs[t])
+ *
+ * with g, d_tokens and d_initial as in ascan_backward_from.  No counterpart in
+ * the reference.  gate = ASCAN_GATE_IDENTITY makes these calls the *_from ones
+ * (forward in time only); ASCAN_GATE_SIGMOID needs a real dtype, else
+ * ASCAN_ERR_BAD_ACTIVATION.  The sigmoid is evaluated in fp32 with the
+ * hardware's exp2 and reciprocal (about 2 ulp).
+ */
+int ascan_forward_gated(const void* gate_inputs, const void* tokens, const void* initial, void* out,
+                        int64_t rows, int64_t seqlen, int dtype, int gate,
+                        void* workspace, size_t workspace_bytes, void* stream);
+
+int ascan_backward_gated(const void* gate_inputs, const void* states, const void* initial,
+                         const void* grad_out, void* d_gate_inputs, void* d_tokens, void* d_initial,
+                         int64_t rows, int64_t seqlen, int dtype, int gate,
+                         void* workspace, size_t workspace_bytes, void* stream);
 
 /* Static, human-readable text for an ascan_status code. */
 const char* ascan_status_string(int status);

@@ -11,6 +11,7 @@
  *   backward (complex) accelerated_scan/complex.py:79-92,113-115,141-147
  * Rows are independent; OpenMP runs them in parallel.
  */
+#include <math.h>
 #include <stdint.h>
 
 /* out[r,t] = g[r,t] * out[r,t-1] + x[r,t]   (reverse: t+1 in place of t-1) */
@@ -226,5 +227,48 @@ void seq_backward_from_c64(const float* g, const float* state, const float* init
             dinit[2 * r] = cr * ar - ci * ai;
             dinit[2 * r + 1] = cr * ai + ci * ar;
         }
+    }
+}
+
+/*
+ * Scans whose gates are the sigmoid of stored pre-activations, gradient with
+ * respect to the pre-activations (no counterpart in the reference, which is
+ * handed finished gates):
+ *   gate[t] = 1 / (1 + exp(-z[t])),  out[t] = gate[t] * out[t-1] + x[t],  out[-1] = init
+ *   dz[t]   = a[t] * state[t-1] * gate[t] * (1 - gate[t]),  dinit = gate[0] * a[0]
+ * Pinned by tests/test_oracle.py: torch autograd through the plain float64 loop
+ * with torch.sigmoid, the zero-start functions above on gates rounded to fp32,
+ * and closed forms (z = 0 gives the geometric series of ratio 1/2).
+ */
+static double sigmoid64(double z) { return 1.0 / (1.0 + exp(-z)); }
+
+void seq_forward_sigmoid_f32(const float* z, const float* x, const float* init, double* out, int64_t rows,
+                             int64_t T) {
+#pragma omp parallel for schedule(static)
+    for (int64_t r = 0; r < rows; ++r) {
+        double s = init ? (double)init[r] : 0.0;
+        for (int64_t t = 0; t < T; ++t) {
+            s = sigmoid64((double)z[r * T + t]) * s + (double)x[r * T + t];
+            out[r * T + t] = s;
+        }
+    }
+}
+
+void seq_backward_sigmoid_f32(const float* z, const float* state, const float* init, const float* dout, double* dz,
+                              double* dx, double* dinit, int64_t rows, int64_t T) {
+#pragma omp parallel for schedule(static)
+    for (int64_t r = 0; r < rows; ++r) {
+        const float* zr = z + r * T;
+        const float* sr = state + r * T;
+        const double x0 = init ? (double)init[r] : 0.0;
+        double a = 0.0;
+        for (int64_t t = T - 1; t >= 0; --t) {
+            const double gnext = (t + 1 < T) ? sigmoid64((double)zr[t + 1]) : 1.0;
+            a = (double)dout[r * T + t] + gnext * a;
+            dx[r * T + t] = a;
+            const double gate = sigmoid64((double)zr[t]);
+            dz[r * T + t] = a * ((t > 0) ? (double)sr[t - 1] : x0) * gate * (1.0 - gate);
+        }
+        if (dinit) dinit[r] = (T > 0) ? sigmoid64((double)zr[0]) * a : 0.0;
     }
 }

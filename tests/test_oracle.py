@@ -310,3 +310,48 @@ def test_from_vs_autograd_of_loop(T, cplx):
     np.testing.assert_allclose(dt, dt_ref.numpy(), rtol=1e-12, atol=1e-12)
     np.testing.assert_allclose(di, di_ref.numpy(), rtol=1e-12, atol=1e-12)
     np.testing.assert_allclose(dg, dg_ref.numpy(), rtol=1e-5, atol=1e-5)  # states rounded to fp32 before the multiply
+
+
+# ---------------------------------------------------------------------------
+# Sigmoid-gated scans (oracle functions *_sigmoid)
+# ---------------------------------------------------------------------------
+@pytest.mark.parametrize("T", [1, 2, 9, 64])
+@pytest.mark.parametrize("with_initial", [False, True])
+def test_sigmoid_vs_autograd_of_loop(T, with_initial):
+    gen = torch.Generator().manual_seed(400 + T)
+    logits = 3.0 * torch.randn(2, 2, T, generator=gen)
+    tokens, grad_out = (torch.randn(2, 2, T, generator=gen) for _ in range(2))
+    initial = torch.randn(2, 2, generator=gen) if with_initial else torch.zeros(2, 2)
+    zw, tw, iw = (t.double().requires_grad_(True) for t in (logits, tokens, initial))
+    out = _loop_scan_from(torch.sigmoid(zw), tw, iw)
+    dz_ref, dt_ref, di_ref = torch.autograd.grad(out, (zw, tw, iw), grad_out.double())
+    init_arg = initial.numpy() if with_initial else None
+    fwd = seqscan.forward_sigmoid(logits.numpy(), tokens.numpy(), init_arg)
+    np.testing.assert_allclose(fwd, out.detach().numpy(), rtol=1e-12, atol=1e-12)
+    dz, dt, di = seqscan.backward_sigmoid(logits.numpy(), fwd.astype(np.float32), grad_out.numpy(), init_arg)
+    np.testing.assert_allclose(dt, dt_ref.numpy(), rtol=1e-12, atol=1e-12)
+    np.testing.assert_allclose(di, di_ref.numpy(), rtol=1e-12, atol=1e-12)
+    np.testing.assert_allclose(dz, dz_ref.numpy(), rtol=1e-5, atol=1e-5)  # states rounded to fp32 before the multiply
+
+
+def test_sigmoid_vs_plain_scan_of_rounded_gates_and_closed_form():
+    gen = torch.Generator().manual_seed(17)
+    logits = 2.0 * torch.randn(3, 4, 200, generator=gen)
+    tokens, grad_out = (torch.randn(3, 4, 200, generator=gen) for _ in range(2))
+    gates = torch.sigmoid(logits.double())
+    fwd = seqscan.forward_sigmoid(logits.numpy(), tokens.numpy())
+    plain = seqscan.forward(gates.float().numpy(), tokens.numpy())
+    np.testing.assert_allclose(fwd, plain, rtol=1e-5, atol=1e-5)  # gates rounded to fp32 on one side
+    states = fwd.astype(np.float32)
+    dz, dx, _ = seqscan.backward_sigmoid(logits.numpy(), states, grad_out.numpy())
+    dg, dx_plain = seqscan.backward(gates.float().numpy(), states, grad_out.numpy())
+    np.testing.assert_allclose(dx, dx_plain, rtol=1e-5, atol=1e-5)
+    np.testing.assert_allclose(dz, dg * (gates * (1 - gates)).numpy(), rtol=1e-5, atol=1e-5)
+    # z = 0: every gate is 1/2, unit tokens give 2 - 2^-t
+    T = 30
+    out = seqscan.forward_sigmoid(np.zeros((1, 1, T), np.float32), np.ones((1, 1, T), np.float32))
+    np.testing.assert_allclose(out[0, 0], 2.0 - 0.5 ** np.arange(T), rtol=1e-15)
+    # saturated gates: z = +40 is a running sum, z = -40 returns the tokens
+    x = tokens[:1, :1, :50].numpy()
+    np.testing.assert_allclose(seqscan.forward_sigmoid(np.full_like(x, 40.0), x), np.cumsum(x.astype(np.float64), -1), rtol=1e-12, atol=1e-12)
+    np.testing.assert_allclose(seqscan.forward_sigmoid(np.full_like(x, -40.0), x), x, rtol=1e-12, atol=1e-12)
