@@ -60,7 +60,7 @@ def main():
                 out = ref.scan(gates, tokens, reverse=reverse)
         data[f"{name}.out"] = out.numpy().copy()
 
-    # BASELINE config 1: fp32 (1, 64, 1024), U(0,1) gates and tokens.
+    # The smallest benchmark configuration: fp32 (1, 64, 1024), U(0,1) gates and tokens.
     real_case("cfg1_fwd", 3407, (1, 64, 1024))
     real_case("pow2_rev", 4, (2, 3, 256), reverse=True)
     real_case("pad_fwd", 42, (2, 3, 1000))            # padded to 1024 with (1, 0)

@@ -275,7 +275,7 @@ def test_unaligned_base_pointer(dtype, offsets, rows, T):
 
 
 # ---------------------------------------------------------------------------
-# BASELINE configurations
+# The five benchmark configurations (shapes and dtypes the reference is quoted on)
 # ---------------------------------------------------------------------------
 def test_config1_cpu_plumbing(golden):
     """fp32 (1, 64, 1024), U(0,1): GPU against the CPU tree scan and the recorded reference output."""
