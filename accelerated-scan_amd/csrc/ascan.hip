@@ -863,27 +863,142 @@ __device__ __forceinline__ void exchange_carries_split(const V (&totA)[U], const
 }
 
 // ---------------------------------------------------------------------------
+// Packed rows: short rows, many of them.  One workgroup per row would leave
+// most lanes idle (a row of 16 elements occupies 4 lanes of one wave), so a
+// workgroup scans a group of consecutive rows -- one contiguous stretch of
+// memory -- as a single long row with a "cut" in front of every row: at a row's
+// first element the gate is replaced by 0, which annihilates whatever the scan
+// carries in from the row before, and gate * x[-1] is added to the token.  All
+// of the tiling, masking and carry code is shared with the one-row-per-
+// workgroup mode; the cuts are applied to the unpacked vectors.
+//   rel  position of an element relative to the first element of the group;
+//   the element is the first of its row when rel % T == 0, the last when
+//   rel % T == T - 1, and belongs to row rel / T of the group.
+// The initial states of the rows a wave's sub-tile touches are staged in LDS by
+// one coalesced read, so the cuts need no per-lane global loads.
+// ---------------------------------------------------------------------------
+template <class Tr>
+struct Cuts {
+    int T;          // row length
+    float inv_T;    // 1 / T
+    int len;        // elements in the group
+    int first_row;  // of the rows staged in `stage`, relative to the group
+    const typename Tr::S* stage;  // their initial states (LDS), or null
+};
+
+// Row and position-in-row of element `rel` (exact for the magnitudes that occur:
+// |rel| < 2^21, T < 2^21).
+__device__ __forceinline__ void split_position(int rel, int T, float inv_T, int& row, int& pos) {
+    row = (int)__builtin_floorf(((float)rel + 0.5f) * inv_T);
+    pos = rel - row * T;
+}
+
+// Forward / reverse scan: at the element that starts the recurrence of its row
+// (first in time order), token += gate * x_start and gate = 0.
+template <class Tr, bool REV>
+__device__ __forceinline__ void cut_rows(typename Tr::V (&g)[Tr::EPV], typename Tr::V (&t)[Tr::EPV], int rel0,
+                                         const Cuts<Tr>& cuts) {
+    using V = typename Tr::V;
+    int row, pos;
+    split_position(rel0, cuts.T, cuts.inv_T, row, pos);
+#pragma unroll
+    for (int e = 0; e < Tr::EPV; ++e) {
+        const bool valid = (unsigned)(rel0 + e) < (unsigned)cuts.len;
+        const bool cut = valid && pos == (REV ? cuts.T - 1 : 0);
+        V start = vzero<V>();
+        if (cuts.stage != nullptr && cut) start = Tr::load1(cuts.stage + (row - cuts.first_row));
+        t[e] = vselect(cut, vfma(g[e], start, t[e]), t[e]);
+        g[e] = vselect(cut, vzero<V>(), g[e]);
+        if (++pos == cuts.T) {
+            pos = 0;
+            ++row;
+        }
+    }
+}
+
+// Backward scan: `after[e]` is the gate that follows element e in its row and
+// `before[e]` the state that precedes it; at a row's last element nothing
+// follows (0), at its first the state before it is the row's initial state.
+// is_first[e] / row_of[e] tell the caller where to put the gradient of that
+// initial state.
+template <class Tr>
+__device__ __forceinline__ void cut_rows_backward(typename Tr::V (&after)[Tr::EPV], typename Tr::V (&before)[Tr::EPV],
+                                                  bool (&is_first)[Tr::EPV], int (&row_of)[Tr::EPV], int rel0,
+                                                  const Cuts<Tr>& cuts) {
+    using V = typename Tr::V;
+    int row, pos;
+    split_position(rel0, cuts.T, cuts.inv_T, row, pos);
+#pragma unroll
+    for (int e = 0; e < Tr::EPV; ++e) {
+        const bool valid = (unsigned)(rel0 + e) < (unsigned)cuts.len;
+        const bool first = valid && pos == 0;
+        const bool last = valid && pos == cuts.T - 1;
+        V start = vzero<V>();
+        if (cuts.stage != nullptr && first) start = Tr::load1(cuts.stage + (row - cuts.first_row));
+        before[e] = vselect(first, start, before[e]);
+        after[e] = vselect(last, vzero<V>(), after[e]);
+        is_first[e] = first;
+        row_of[e] = row;
+        if (++pos == cuts.T) {
+            pos = 0;
+            ++row;
+        }
+    }
+}
+
+// Stages the initial states of the rows that the sub-tile [sub_rel, sub_rel+sub)
+// touches (positions relative to the group) into the wave's LDS area.
+template <class Tr>
+__device__ __forceinline__ Cuts<Tr> stage_row_starts(const typename Tr::S* __restrict__ initial_of_group, int T,
+                                                     int len, int sub_rel, int sub, typename Tr::S* stage, int lane) {
+    Cuts<Tr> cuts;
+    cuts.T = T;
+    cuts.inv_T = 1.0f / (float)T;
+    cuts.len = len;
+    cuts.first_row = 0;
+    cuts.stage = nullptr;
+    if (initial_of_group != nullptr) {
+        const int rel_first = sub_rel > 0 ? sub_rel : 0;
+        const int rel_last = sub_rel + sub - 1 < len - 1 ? sub_rel + sub - 1 : len - 1;
+        if (rel_first <= rel_last) {  // wave-uniform
+            cuts.first_row = rel_first / T;
+            const int count = rel_last / T - cuts.first_row + 1;  // at most `sub`
+            for (int i = lane; i < count; i += 64) stage[i] = initial_of_group[cuts.first_row + i];
+        }
+        cuts.stage = stage;
+        __syncthreads();  // makes the staged values visible to the other lanes
+    }
+    return cuts;
+}
+
+// ---------------------------------------------------------------------------
 // Forward kernel (REV = false) and plain reverse scan (REV = true).
 // A workgroup holds R rows x W waves per row (R = blockDim.x / 64 / W); the
 // rows of a workgroup are adjacent in memory, so with W*R = 16 one tile step
 // of the workgroup covers one contiguous span of 16 sub-tiles.
 // ---------------------------------------------------------------------------
-template <class Tr, int W, int U, bool REV, bool ALIGNED, bool REGULAR, bool SPLIT, int ACT>
+template <class Tr, int W, int U, bool REV, bool ALIGNED, bool REGULAR, bool SPLIT, int ACT, bool PACKED>
 __global__ void __launch_bounds__(64 * kMaxWavesPerBlock)
     scan_forward_kernel(const typename Tr::S* __restrict__ gates, const typename Tr::TokS* __restrict__ tokens,
                         typename Tr::S* __restrict__ out, int64_t rows, int64_t T, SplitHeader* split,
-                        const typename Tr::S* __restrict__ initial, int G) {
+                        const typename Tr::S* __restrict__ initial, int G, int group) {
     using S = typename Tr::S;
     using V = typename Tr::V;
     constexpr int EPV = Tr::EPV;
     constexpr int64_t SUB = (int64_t)U * 64 * EPV;
     constexpr int64_t TILE = SUB * W;
+    static_assert(!PACKED || (!SPLIT && !REGULAR), "packed rows use the general kernels, one group per workgroup");
 
     const int lane = threadIdx.x & 63;
-    // rows start at the same misalignment when T is a multiple of the grid spacing
-    const int head = REGULAR ? 0 : (ALIGNED ? (T % G == 0 ? row_lead<Tr>(gates, G) : G - 1) : 0);
-    const int64_t ntiles = tiles_per_row(T, TILE, head);
+    // Packed rows: this workgroup scans rows [first_row, first_row + nrows) as one row of `len` elements.
+    const int64_t first_row = PACKED ? (int64_t)blockIdx.x * group : 0;
+    const int64_t len = PACKED ? (rows - first_row < group ? rows - first_row : (int64_t)group) * T : T;
+    const int64_t longest = PACKED ? (int64_t)group * T : T;
+    // rows start at the same misalignment when their length is a multiple of the grid spacing
+    const int head = REGULAR ? 0 : (ALIGNED ? (longest % G == 0 ? row_lead<Tr>(gates, G) : G - 1) : 0);
+    const int64_t ntiles = tiles_per_row(longest, TILE, head);
     __shared__ V slots_all[W == 1 ? 1 : 2 * kSlotsPerBuffer];
+    __shared__ S stage_all[PACKED ? W * SUB : 1];
     // Split rows: a fixed set of co-resident workgroups walks over all (row,
     // tile) pairs in order, all tiles of row 0 first; what is in flight at any
     // time is one contiguous stretch of memory, and a workgroup only ever waits
@@ -899,20 +1014,25 @@ __global__ void __launch_bounds__(64 * kMaxWavesPerBlock)
         k_end = k_begin + 1;
         w = threadIdx.x >> 6;
         slot_base = 0;
+    } else if constexpr (PACKED) {
+        row = first_row;
+        w = threadIdx.x >> 6;
+        slot_base = 0;
     } else {
         if (!locate_wave<W>(rows, ntiles, row, w, slot_base)) return;  // wave-uniform
     }
     V* slots = slots_all + (W == 1 ? 0 : slot_base);
 
     const int64_t lo = (ALIGNED && !REGULAR) ? row_lead<Tr>(gates + row * T, G) : 0;
-    const int64_t hi = lo + T;
+    const int64_t hi = lo + len;
     const S* __restrict__ grow = gates + row * T - lo;
     const typename Tr::TokS* __restrict__ trow = tokens + row * T - lo;
     S* __restrict__ orow = out + row * T - lo;
 
     // state the row starts from (one element per row; absent = zero); a split
-    // row needs it in its first tile only
-    const V row_start = (initial != nullptr && (!SPLIT || k_begin == 0)) ? Tr::load1(initial + row) : vzero<V>();
+    // row needs it in its first tile only; packed rows take theirs at the cuts
+    const V row_start =
+        (!PACKED && initial != nullptr && (!SPLIT || k_begin == 0)) ? Tr::load1(initial + row) : vzero<V>();
     V carry = row_start;
 
     // Position of this wave's sub-tile in tile step k.
@@ -932,6 +1052,12 @@ __global__ void __launch_bounds__(64 * kMaxWavesPerBlock)
         const S* __restrict__ gsub = grow + sub_base;
         const typename Tr::TokS* __restrict__ tsub = trow + sub_base;
         S* __restrict__ osub = orow + sub_base;
+
+        Cuts<Tr> cuts;
+        if constexpr (PACKED) {
+            cuts = stage_row_starts<Tr>(initial != nullptr ? initial + first_row : nullptr, (int)T, (int)len,
+                                        (int)(sub_base - lo), (int)SUB, stage_all + w * SUB, lane);
+        }
 
         u32x4_t graw[U], traw[U];
         if (touches) {
@@ -957,6 +1083,7 @@ __global__ void __launch_bounds__(64 * kMaxWavesPerBlock)
             Tr::unpack(graw[j], g);
             activate<ACT>(g);
             Tr::unpack(traw[j], t);
+            if constexpr (PACKED) cut_rows<Tr, REV>(g, t, (int)(sub_base - lo) + vec_offset<U, EPV, REV>(j, lane), cuts);
             constexpr int e0 = REV ? EPV - 1 : 0;
             V A = g[e0];
             V X = t[e0];
@@ -992,6 +1119,7 @@ __global__ void __launch_bounds__(64 * kMaxWavesPerBlock)
             Tr::unpack(graw[j], g);
             activate<ACT>(g);
             Tr::unpack(traw[j], t);
+            if constexpr (PACKED) cut_rows<Tr, REV>(g, t, (int)(sub_base - lo) + vec_offset<U, EPV, REV>(j, lane), cuts);
             V x = vfma(exA[j], c, exX[j]);  // state entering this lane's vector
             c = vfma(totA[j], c, totX[j]);  // state entering the next block
             V o[EPV];
@@ -1028,23 +1156,30 @@ __global__ void __launch_bounds__(64 * kMaxWavesPerBlock)
 // Fused backward kernel: reverse-time scan over gate[t+1] producing d_tokens,
 // and d_gates[t] = d_tokens[t] * conj(x[t-1]) in the same pass.
 // ---------------------------------------------------------------------------
-template <class Tr, int W, int U, bool ALIGNED, bool REGULAR, bool SPLIT, int ACT>
+template <class Tr, int W, int U, bool ALIGNED, bool REGULAR, bool SPLIT, int ACT, bool PACKED>
 __global__ void __launch_bounds__(64 * kMaxWavesPerBlock)
     scan_backward_kernel(const typename Tr::S* __restrict__ gates, const typename Tr::S* __restrict__ states,
                          const typename Tr::S* __restrict__ grad_out, typename Tr::S* __restrict__ d_gates,
                          typename Tr::TokS* __restrict__ d_tokens, int64_t rows, int64_t T, SplitHeader* split,
-                         const typename Tr::S* __restrict__ initial, typename Tr::S* __restrict__ d_initial, int G) {
+                         const typename Tr::S* __restrict__ initial, typename Tr::S* __restrict__ d_initial, int G,
+                         int group) {
     using S = typename Tr::S;
     using V = typename Tr::V;
     constexpr int EPV = Tr::EPV;
     constexpr int64_t SUB = (int64_t)U * 64 * EPV;
     constexpr int64_t TILE = SUB * W;
+    static_assert(!PACKED || (!SPLIT && !REGULAR), "packed rows use the general kernels, one group per workgroup");
 
     const int lane = threadIdx.x & 63;
-    // rows start at the same misalignment when T is a multiple of the grid spacing
-    const int head = REGULAR ? 0 : (ALIGNED ? (T % G == 0 ? row_lead<Tr>(gates, G) : G - 1) : 0);
-    const int64_t ntiles = tiles_per_row(T, TILE, head);
+    // Packed rows: this workgroup scans rows [first_row, first_row + nrows) as one row of `len` elements.
+    const int64_t first_row = PACKED ? (int64_t)blockIdx.x * group : 0;
+    const int64_t len = PACKED ? (rows - first_row < group ? rows - first_row : (int64_t)group) * T : T;
+    const int64_t longest = PACKED ? (int64_t)group * T : T;
+    // rows start at the same misalignment when their length is a multiple of the grid spacing
+    const int head = REGULAR ? 0 : (ALIGNED ? (longest % G == 0 ? row_lead<Tr>(gates, G) : G - 1) : 0);
+    const int64_t ntiles = tiles_per_row(longest, TILE, head);
     __shared__ V slots_all[W == 1 ? 1 : 2 * kSlotsPerBuffer];
+    __shared__ S stage_all[PACKED ? W * SUB : 1];
     // Split rows: a fixed set of co-resident workgroups walks over all (row,
     // tile) pairs in order, all tiles of row 0 first; what is in flight at any
     // time is one contiguous stretch of memory, and a workgroup only ever waits
@@ -1060,13 +1195,17 @@ __global__ void __launch_bounds__(64 * kMaxWavesPerBlock)
         k_end = k_begin + 1;
         w = threadIdx.x >> 6;
         slot_base = 0;
+    } else if constexpr (PACKED) {
+        row = first_row;
+        w = threadIdx.x >> 6;
+        slot_base = 0;
     } else {
         if (!locate_wave<W>(rows, ntiles, row, w, slot_base)) return;  // wave-uniform
     }
     V* slots = slots_all + (W == 1 ? 0 : slot_base);
 
     const int64_t lo = (ALIGNED && !REGULAR) ? row_lead<Tr>(gates + row * T, G) : 0;
-    const int64_t hi = lo + T;
+    const int64_t hi = lo + len;
     const S* __restrict__ arow = gates + row * T - lo;
     const S* __restrict__ xrow = states + row * T - lo;
     const S* __restrict__ drow = grad_out + row * T - lo;
@@ -1105,7 +1244,12 @@ __global__ void __launch_bounds__(64 * kMaxWavesPerBlock)
         // x[-1], the state the forward scan started from (absent = zero), is
         // needed by the sub-tile that holds the row's first element
         V x_start = vzero<V>();
-        if (initial != nullptr && sub_base <= lo && lo < sub_end) x_start = Tr::load1(initial + row);  // wave-uniform
+        if (!PACKED && initial != nullptr && sub_base <= lo && lo < sub_end) x_start = Tr::load1(initial + row);  // wave-uniform
+        Cuts<Tr> cuts;  // packed rows take their initial states at the cuts instead
+        if constexpr (PACKED) {
+            cuts = stage_row_starts<Tr>(initial != nullptr ? initial + first_row : nullptr, (int)T, (int)len,
+                                        (int)(sub_base - lo), (int)SUB, stage_all + w * SUB, lane);
+        }
 
         u32x4_t araw[U], draw[U], xraw[U];
         if (touches) {
@@ -1172,11 +1316,24 @@ __global__ void __launch_bounds__(64 * kMaxWavesPerBlock)
             a_next[j] = shift_up1(a[0], hi_edge);
             x_prev[j] = shift_down1(x[EPV - 1], lo_edge);
 
-            V A = vconj(a_next[j]);
+            // after[e]: the gate that follows element e; before[e]: the state that precedes it
+            V after[EPV], before[EPV];
+#pragma unroll
+            for (int e = 0; e < EPV; ++e) {
+                after[e] = e < EPV - 1 ? a[e + 1] : a_next[j];
+                before[e] = e > 0 ? x[e - 1] : x_prev[j];
+            }
+            if constexpr (PACKED) {
+                bool is_first[EPV];
+                int row_of[EPV];
+                cut_rows_backward<Tr>(after, before, is_first, row_of,
+                                      (int)(sub_base - lo) + vec_offset<U, EPV, true>(j, lane), cuts);
+            }
+            V A = vconj(after[EPV - 1]);
             V X = d[EPV - 1];
 #pragma unroll
             for (int e = EPV - 2; e >= 0; --e) {
-                const V ga = vconj(a[e + 1]);
+                const V ga = vconj(after[e]);
                 X = vfma(ga, X, d[e]);
                 A = vmul(A, ga);
             }
@@ -1209,20 +1366,38 @@ __global__ void __launch_bounds__(64 * kMaxWavesPerBlock)
             Tr::unpack(xraw[j], x);
             V gr = vfma(exA[j], c, exX[j]);  // g entering this lane's vector from above
             c = vfma(totA[j], c, totX[j]);
+            const int off = vec_offset<U, EPV, true>(j, lane);
+            V after[EPV], before[EPV];
+#pragma unroll
+            for (int e = 0; e < EPV; ++e) {
+                after[e] = e < EPV - 1 ? a[e + 1] : a_next[j];
+                before[e] = e > 0 ? x[e - 1] : x_prev[j];
+            }
+            bool is_first[EPV];
+            int row_of[EPV];
+            if constexpr (PACKED) {
+                cut_rows_backward<Tr>(after, before, is_first, row_of, (int)(sub_base - lo) + off, cuts);
+            }
             V dt[EPV], dg[EPV];
 #pragma unroll
             for (int e = EPV - 1; e >= 0; --e) {
-                const V ga = vconj(e < EPV - 1 ? a[e + 1] : a_next[j]);
-                const V xs = vconj(e > 0 ? x[e - 1] : x_prev[j]);
-                gr = vfma(ga, gr, d[e]);
+                gr = vfma(vconj(after[e]), gr, d[e]);
                 dt[e] = gr;
-                dg[e] = vmul(gr, xs);
+                dg[e] = vmul(gr, vconj(before[e]));
                 if constexpr (ACT != kGateIdentity) dg[e] = vmul(dg[e], gate_slope<ACT>(a[e]));
             }
-            const int off = vec_offset<U, EPV, true>(j, lane);
             if (touches) {
                 store_tok_vec<Tr, ALIGNED, FULL>(dtsub, off, win, dt);
                 store_vec<Tr, ALIGNED, FULL>(dgsub, off, win, dg);
+            }
+            if constexpr (PACKED) {
+                // gradient of each row's initial state, conj(gate[0]) * g[0], from the lane that holds the row's start
+                if (d_initial != nullptr) {
+#pragma unroll
+                    for (int e = 0; e < EPV; ++e) {
+                        if (is_first[e]) Tr::store1(d_initial + first_row + row_of[e], vmul(vconj(a[e]), dt[e]));
+                    }
+                }
             }
         }
 
@@ -1246,7 +1421,7 @@ __global__ void __launch_bounds__(64 * kMaxWavesPerBlock)
         }
     }
     // after the last tile step the carry is g at position 0 of the first tile
-    if constexpr (!SPLIT) {
+    if constexpr (!SPLIT && !PACKED) {
         if (d_initial != nullptr && w == 0) store_start_gradient(carry);  // wave-uniform
     }
     }  // visits
@@ -1362,9 +1537,9 @@ hipError_t launch_forward(const void* gates, const void* tokens, void* out, cons
     constexpr int U = REGULAR ? Tuning<Tr>::U : Tuning<Tr>::UG;
     const unsigned blocks = (unsigned)((rows + rows_per_block - 1) / rows_per_block);
     const unsigned threads = 64u * W * rows_per_block;
-    return launch(scan_forward_kernel<Tr, W, U, REV, ALIGNED, REGULAR, false, ACT>, blocks, threads, stream,
+    return launch(scan_forward_kernel<Tr, W, U, REV, ALIGNED, REGULAR, false, ACT, false>, blocks, threads, stream,
                   static_cast<const S*>(gates), static_cast<const TokS*>(tokens), static_cast<S*>(out), rows, T,
-                  static_cast<SplitHeader*>(nullptr), static_cast<const S*>(initial), grid);
+                  static_cast<SplitHeader*>(nullptr), static_cast<const S*>(initial), grid, 0);
 }
 
 template <class Tr, int W, bool ALIGNED, bool REGULAR, int ACT>
@@ -1376,10 +1551,10 @@ hipError_t launch_backward(const void* gates, const void* states, const void* gr
     constexpr int U = REGULAR ? Tuning<Tr>::UB : Tuning<Tr>::UBG;
     const unsigned blocks = (unsigned)((rows + rows_per_block - 1) / rows_per_block);
     const unsigned threads = 64u * W * rows_per_block;
-    return launch(scan_backward_kernel<Tr, W, U, ALIGNED, REGULAR, false, ACT>, blocks, threads, stream,
+    return launch(scan_backward_kernel<Tr, W, U, ALIGNED, REGULAR, false, ACT, false>, blocks, threads, stream,
                   static_cast<const S*>(gates), static_cast<const S*>(states), static_cast<const S*>(grad_out),
                   static_cast<S*>(d_gates), static_cast<TokS*>(d_tokens), rows, T,
-                  static_cast<SplitHeader*>(nullptr), static_cast<const S*>(initial), static_cast<S*>(d_initial), grid);
+                  static_cast<SplitHeader*>(nullptr), static_cast<const S*>(initial), static_cast<S*>(d_initial), grid, 0);
 }
 
 // Caller-provided table for split rows (may be absent).
@@ -1466,7 +1641,7 @@ hipError_t launch_forward_split(const void* gates, const void* tokens, void* out
     using S = typename Tr::S;
     using TokS = typename Tr::TokS;
     constexpr int U = REGULAR ? Tuning<Tr>::U : Tuning<Tr>::UG;
-    auto kernel = scan_forward_kernel<Tr, kSplitWaves, U, REV, true, REGULAR, true, ACT>;
+    auto kernel = scan_forward_kernel<Tr, kSplitWaves, U, REV, true, REGULAR, true, ACT, false>;
     const unsigned resident = resident_workgroups(kernel, 64 * kSplitWaves);
     if (resident == 0) return hipErrorInvalidConfiguration;
     const hipError_t e = reset_split_table(ws, rows, ntiles, stream);
@@ -1474,7 +1649,7 @@ hipError_t launch_forward_split(const void* gates, const void* tokens, void* out
     const int64_t tiles = rows * ntiles;
     return launch(kernel, (unsigned)(tiles < resident ? tiles : resident), 64u * kSplitWaves, stream,
                   static_cast<const S*>(gates), static_cast<const TokS*>(tokens), static_cast<S*>(out), rows, T,
-                  static_cast<SplitHeader*>(ws.ptr), static_cast<const S*>(initial), grid);
+                  static_cast<SplitHeader*>(ws.ptr), static_cast<const S*>(initial), grid, 0);
 }
 
 template <class Tr, bool REGULAR, int ACT>
@@ -1484,7 +1659,7 @@ hipError_t launch_backward_split(const void* gates, const void* states, const vo
     using S = typename Tr::S;
     using TokS = typename Tr::TokS;
     constexpr int U = REGULAR ? Tuning<Tr>::UB : Tuning<Tr>::UBG;
-    auto kernel = scan_backward_kernel<Tr, kSplitWaves, U, true, REGULAR, true, ACT>;
+    auto kernel = scan_backward_kernel<Tr, kSplitWaves, U, true, REGULAR, true, ACT, false>;
     const unsigned resident = resident_workgroups(kernel, 64 * kSplitWaves);
     if (resident == 0) return hipErrorInvalidConfiguration;
     const hipError_t e = reset_split_table(ws, rows, ntiles, stream);
@@ -1493,7 +1668,70 @@ hipError_t launch_backward_split(const void* gates, const void* states, const vo
     return launch(kernel, (unsigned)(tiles < resident ? tiles : resident), 64u * kSplitWaves, stream,
                   static_cast<const S*>(gates), static_cast<const S*>(states), static_cast<const S*>(grad_out),
                   static_cast<S*>(d_gates), static_cast<TokS*>(d_tokens), rows, T,
-                  static_cast<SplitHeader*>(ws.ptr), static_cast<const S*>(initial), static_cast<S*>(d_initial), grid);
+                  static_cast<SplitHeader*>(ws.ptr), static_cast<const S*>(initial), static_cast<S*>(d_initial), grid, 0);
+}
+
+// Packed-row policy.  Rows shorter than kPackedMaxRowBytes (of states) are
+// scanned in groups, one group per 4-wave workgroup; a group fills one tile of
+// the general kernel, counting the lead of its first element, and when possible
+// is a whole number of 128-byte lines long so that every group starts on the
+// grid like the first.  ASCAN_PACKED_MAX_ROW_BYTES overrides the limit (0
+// switches packing off), read once.
+constexpr int kPackedWaves = 4;
+constexpr int64_t kPackedMaxRowBytesDefault = 2048;
+
+int64_t packed_max_row_bytes() {
+    static const int64_t v = [] {
+        const char* s = getenv("ASCAN_PACKED_MAX_ROW_BYTES");
+        return s ? (int64_t)atoll(s) : kPackedMaxRowBytesDefault;
+    }();
+    return v;
+}
+
+int64_t gcd64(int64_t a, int64_t b) {
+    while (b != 0) {
+        const int64_t t = a % b;
+        a = b;
+        b = t;
+    }
+    return a;
+}
+
+// Rows per group for rows of T elements, tiles of `tile` elements and a grid of
+// `grid` elements; 0 when rows of this length are not packed.
+int packed_group(int64_t rows, int64_t T, int64_t element_bytes, int64_t tile, int grid) {
+    if (rows < 2 || T * element_bytes >= packed_max_row_bytes()) return 0;
+    int64_t group = (tile - grid) / T;
+    if (group < 2) return 0;
+    const int64_t whole_lines = grid / gcd64(T, grid);  // rows per whole number of grid cells
+    if (group >= whole_lines) group -= group % whole_lines;
+    return (int)group;
+}
+
+template <class Tr, bool REV, bool ALIGNED, int ACT>
+hipError_t launch_forward_packed(const void* gates, const void* tokens, void* out, const void* initial, int64_t rows,
+                                 int64_t T, int grid, int group, hipStream_t stream) {
+    using S = typename Tr::S;
+    using TokS = typename Tr::TokS;
+    const unsigned blocks = (unsigned)((rows + group - 1) / group);
+    return launch(scan_forward_kernel<Tr, kPackedWaves, Tuning<Tr>::UG, REV, ALIGNED, false, false, ACT, true>, blocks,
+                  64u * kPackedWaves, stream, static_cast<const S*>(gates), static_cast<const TokS*>(tokens),
+                  static_cast<S*>(out), rows, T, static_cast<SplitHeader*>(nullptr), static_cast<const S*>(initial),
+                  grid, group);
+}
+
+template <class Tr, bool ALIGNED, int ACT>
+hipError_t launch_backward_packed(const void* gates, const void* states, const void* grad_out, void* d_gates,
+                                  void* d_tokens, const void* initial, void* d_initial, int64_t rows, int64_t T,
+                                  int grid, int group, hipStream_t stream) {
+    using S = typename Tr::S;
+    using TokS = typename Tr::TokS;
+    const unsigned blocks = (unsigned)((rows + group - 1) / group);
+    return launch(scan_backward_kernel<Tr, kPackedWaves, Tuning<Tr>::UBG, ALIGNED, false, false, ACT, true>, blocks,
+                  64u * kPackedWaves, stream, static_cast<const S*>(gates), static_cast<const S*>(states),
+                  static_cast<const S*>(grad_out), static_cast<S*>(d_gates), static_cast<TokS*>(d_tokens), rows, T,
+                  static_cast<SplitHeader*>(nullptr), static_cast<const S*>(initial), static_cast<S*>(d_initial), grid,
+                  group);
 }
 
 // Memory-access flavour of a launch.
@@ -1531,6 +1769,21 @@ int forward_typed(const void* gates, const void* tokens, void* out, const void* 
     if (access != Access::kRegular) plan = choose_plan(T, SUBG, kElem);
     const int R = plan.rows_per_block;
     hipError_t err = hipSuccess;
+    if (const int group = packed_group(rows, T, kElem, SUBG * kPackedWaves, same_lead ? at.grid : 1)) {
+#define ASCAN_FWD_PACKED(REV, AL, ACT) \
+    launch_forward_packed<Tr, REV, AL, ACT>(gates, tokens, out, initial, rows, T, at.grid, group, stream)
+        if (act == kGateSigmoid) {
+            if constexpr (kHasSigmoid<Tr>) {
+                err = same_lead ? ASCAN_FWD_PACKED(false, true, kGateSigmoid) : ASCAN_FWD_PACKED(false, false, kGateSigmoid);
+            }
+        } else if (same_lead) {
+            err = reverse ? ASCAN_FWD_PACKED(true, true, kGateIdentity) : ASCAN_FWD_PACKED(false, true, kGateIdentity);
+        } else {
+            err = reverse ? ASCAN_FWD_PACKED(true, false, kGateIdentity) : ASCAN_FWD_PACKED(false, false, kGateIdentity);
+        }
+#undef ASCAN_FWD_PACKED
+        return launch_status(err);
+    }
     if (same_lead && ws.ptr != nullptr) {
         const bool regular = lead == 0 && T % (SUB * kSplitWaves) == 0;
         const int64_t ntiles = host_tiles_per_row<Tr>(T, (regular ? SUB : SUBG) * kSplitWaves, regular, at);
@@ -1599,6 +1852,20 @@ int backward_typed(const void* gates, const void* states, const void* grad_out, 
     if (access != Access::kRegular) plan = choose_plan(T, SUBG, kElem);
     const int R = plan.rows_per_block;
     hipError_t err = hipSuccess;
+    if (const int group = packed_group(rows, T, kElem, SUBG * kPackedWaves, same_lead ? at.grid : 1)) {
+#define ASCAN_BWD_PACKED(AL, ACT)                                                                                  \
+    launch_backward_packed<Tr, AL, ACT>(gates, states, grad_out, d_gates, d_tokens, initial, d_initial, rows, T, \
+                                        at.grid, group, stream)
+        if (act == kGateSigmoid) {
+            if constexpr (kHasSigmoid<Tr>) {
+                err = same_lead ? ASCAN_BWD_PACKED(true, kGateSigmoid) : ASCAN_BWD_PACKED(false, kGateSigmoid);
+            }
+        } else {
+            err = same_lead ? ASCAN_BWD_PACKED(true, kGateIdentity) : ASCAN_BWD_PACKED(false, kGateIdentity);
+        }
+#undef ASCAN_BWD_PACKED
+        return launch_status(err);
+    }
     if (same_lead && ws.ptr != nullptr) {
         const bool regular = lead == 0 && T % (SUB * kSplitWaves) == 0;
         const int64_t ntiles = host_tiles_per_row<Tr>(T, (regular ? SUB : SUBG) * kSplitWaves, regular, at);

@@ -97,9 +97,16 @@ def test_tile_and_wave_boundaries(dtype, with_initial, rows, T):
 
 
 @pytest.mark.parametrize("dtype", DTYPES, ids=IDS)
+@pytest.mark.parametrize("with_initial", [False, True], ids=["zero-start", "initial"])
+@pytest.mark.parametrize("rows,T", [(100000, 1), (4099, 2), (1000, 7), (777, 33), (5000, 64), (999, 255), (301, 500)])
+def test_short_rows_in_groups(dtype, with_initial, rows, T):
+    _run_and_compare(rows, T, dtype, seed=rows + T, what="short rows", with_initial=with_initial)
+
+
+@pytest.mark.parametrize("dtype", DTYPES, ids=IDS)
 @pytest.mark.parametrize("offsets", [(1, 1, 1), (3, 3, 3), (1, 0, 2), (1, 9, 17)],
                          ids=["same1", "same3", "mixed", "same-mod-8"])
-@pytest.mark.parametrize("rows,T", [(6, 2048), (3, 40000), (2050, 1031), (4, 7)])
+@pytest.mark.parametrize("rows,T", [(6, 2048), (3, 40000), (2050, 1031), (4, 7), (3000, 37)])
 def test_unaligned_base_pointer(dtype, offsets, rows, T):
     _run_and_compare(rows, T, dtype, seed=9, what="offset views", with_initial=True, offsets=offsets)
 

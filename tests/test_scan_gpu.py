@@ -237,7 +237,7 @@ def test_unaligned_rows(dtype, rows, T):
 @pytest.mark.parametrize("dtype", ALL_DTYPES, ids=ALL_IDS)
 @pytest.mark.parametrize("offsets", [(1, 1, 1), (3, 3, 3), (1, 0, 2), (1, 9, 17), (4, 12, 8)],
                          ids=["same1", "same3", "mixed", "same-mod-8", "multiples-of-4"])
-@pytest.mark.parametrize("rows,T", [(6, 2048), (3, 40000), (2050, 1031)])
+@pytest.mark.parametrize("rows,T", [(6, 2048), (3, 40000), (2050, 1031), (3000, 37)])
 def test_unaligned_base_pointer(dtype, offsets, rows, T):
     """Views with a storage offset: base pointers off the 16-byte grid.  Equal
     offsets keep the vectorised kernels (rows are addressed from the 128-byte
@@ -272,6 +272,17 @@ def test_unaligned_base_pointer(dtype, offsets, rows, T):
         k = t.storage_offset()
         whole = torch.empty(0, dtype=t.dtype, device=DEVICE).set_(t.untyped_storage())
         assert whole[:k].abs().sum().item() == 0 and whole[k + rows * T:].abs().sum().item() == 0
+
+
+@pytest.mark.parametrize("dtype", ALL_DTYPES, ids=ALL_IDS)
+@pytest.mark.parametrize("rows,T", [(100000, 1), (4099, 2), (3001, 3), (1000, 7), (777, 33), (5000, 64), (1234, 100),
+                                    (999, 255), (640, 256), (2, 200), (301, 500)])
+def test_short_rows_in_groups(dtype, rows, T):
+    """Rows shorter than 2 KiB are scanned in groups of consecutive rows with a
+    cut in front of every row: many groups, a last group that is not full, row
+    lengths below, at and above the vector width."""
+    gates, tokens, grad_out = _truth_inputs(rows, T, dtype, seed=rows + T)
+    _check_against_truth(gates, tokens, grad_out, dtype, what="short rows")
 
 
 # ---------------------------------------------------------------------------

@@ -122,9 +122,18 @@ def test_tile_and_wave_boundaries(dtype, rows, T):
 
 
 @pytest.mark.parametrize("dtype", ALL_DTYPES, ids=ALL_IDS)
+@pytest.mark.parametrize("rows,T", [(100000, 1), (4099, 2), (3001, 3), (1000, 7), (777, 33), (5000, 64), (1234, 100),
+                                    (999, 255), (640, 256), (2, 200), (301, 500)])
+def test_short_rows_in_groups(dtype, rows, T):
+    """Short rows scanned in groups: every row takes its own initial state at its
+    cut and returns the gradient of it."""
+    _run_and_compare(rows, T, dtype, seed=rows + T, what="short rows")
+
+
+@pytest.mark.parametrize("dtype", ALL_DTYPES, ids=ALL_IDS)
 @pytest.mark.parametrize("offsets", [(1, 1, 1), (3, 3, 3), (1, 0, 2), (1, 9, 17), (4, 12, 8)],
                          ids=["same1", "same3", "mixed", "same-mod-8", "multiples-of-4"])
-@pytest.mark.parametrize("rows,T", [(6, 2048), (3, 40000), (2050, 1031), (4, 7)])
+@pytest.mark.parametrize("rows,T", [(6, 2048), (3, 40000), (2050, 1031), (4, 7), (3000, 37)])
 def test_unaligned_base_pointer(dtype, offsets, rows, T):
     _run_and_compare(rows, T, dtype, seed=9, what="offset views", offsets=offsets)
 
