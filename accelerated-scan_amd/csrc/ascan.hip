@@ -39,6 +39,7 @@
 #include <stdint.h>
 #include <stdlib.h>
 
+#include <atomic>
 #include <type_traits>
 
 #include "ascan.h"
@@ -650,13 +651,18 @@ __device__ __forceinline__ void exchange_carries(const V (&totA)[U], const V (&t
 //   * it then walks back over the earlier tiles of its row, folding aggregates
 //     until it meets a tile whose inclusive state P is already published;
 //   * it publishes its own inclusive state and finishes the tile.
-// The launch has no more workgroups than the GPU can hold at once, and
-// workgroup b takes tiles b, b + G, b + 2G, ... of the row-major list of all
-// tiles, so the earliest unfinished tile is always being worked on by a resident
-// workgroup and depends only on finished ones (a ticket counter was tried
-// first: one device-wide atomic per tile costs ~0.1 us and serialises the
-// launch).  Each wait is bounded by a wall-clock limit set by the host; a wait
-// that runs out poisons the result with NaN and is counted in the header.
+// Tiles are handed out by ticket: every row has a counter, and a workgroup
+// takes the next tile of a row with one fetch-add on it (moving on to the next
+// row when a row has no tiles left).  A tile is therefore only ever waited for
+// by workgroups that started after its owner did: progress never depends on a
+// workgroup that has not been dispatched yet, whatever else is running on the
+// GPU, and the launch size (what an idle GPU holds at once) is a matter of
+// speed only.  One counter per row keeps the fetch-adds of different rows
+// apart (measured: ~11 ns each on one address, concurrent across addresses).
+// Each wait is nevertheless bounded by a limit set by the host; a wait that
+// runs out poisons the result with NaN and is counted in the header.  Waiting
+// time is summed from clock differences capped at 10 us each, so a stretch
+// during which the whole kernel was not running does not count.
 // ---------------------------------------------------------------------------
 struct SplitHeader {
     unsigned long long reserved0;
@@ -665,6 +671,15 @@ struct SplitHeader {
     unsigned int reserved[11];
 };
 static_assert(sizeof(SplitHeader) == 64, "header is 64 bytes");
+
+// One ticket counter per row, each on a cache line of its own.
+struct alignas(64) SplitTicket {
+    unsigned long long next;  // scan-order index of the next tile to hand out
+    unsigned long long pad[7];
+};
+static_assert(sizeof(SplitTicket) == 64, "ticket line is 64 bytes");
+
+constexpr unsigned long long kWaitStepCap = 1000;  // 10 us in 100 MHz ticks
 
 // One record per (row, tile).  Every field is a 64-bit word holding an fp32
 // payload in its low half and a tag in its high half (0 = not written yet,
@@ -724,9 +739,91 @@ __global__ void split_reset_kernel(uint32_t* words, size_t nwords, unsigned long
     }
 }
 
-// The records follow the header.
-__device__ __forceinline__ SplitRecord* split_records(SplitHeader* header) {
-    return reinterpret_cast<SplitRecord*>(header + 1);
+// Layout of the table: header, one ticket line per row, one record per (row, tile).
+__device__ __forceinline__ SplitTicket* split_tickets(SplitHeader* header) {
+    return reinterpret_cast<SplitTicket*>(header + 1);
+}
+__device__ __forceinline__ SplitRecord* split_records(SplitHeader* header, int64_t rows) {
+    return reinterpret_cast<SplitRecord*>(split_tickets(header) + rows);
+}
+
+// A workgroup's place in the hand-out of tiles: the row it is taking tiles from
+// and the ticket it has already drawn for its next tile (drawn while the
+// current tile's loads are in flight, so that the fetch-add's latency is off
+// the critical path).  Meaningful in wave 0 only.
+struct SplitWalk {
+    int64_t row;
+    unsigned long long drawn;  // valid when has_drawn
+    bool has_drawn;
+};
+
+__device__ __forceinline__ unsigned long long draw_ticket(SplitTicket* ticket, int lane) {
+    unsigned long long t = 0;
+    if (lane == 0) t = __hip_atomic_fetch_add(&ticket->next, 1ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    return t;  // lane 0 holds the ticket
+}
+__device__ __forceinline__ unsigned long long from_lane0(unsigned long long v) {
+    return ((unsigned long long)(unsigned)__builtin_amdgcn_readfirstlane((int)(v >> 32)) << 32) |
+           (unsigned)__builtin_amdgcn_readfirstlane((int)v);
+}
+
+// Hands the workgroup its next tile: the next tile of the row it is on if that
+// row has one left, else of the next row (cyclically) that does.  Returns false
+// when no row has tiles left.  All threads of the workgroup call it together
+// and get the same answer; `mailbox` is two words of LDS.
+__device__ __forceinline__ bool take_split_tile(SplitHeader* header, int64_t rows, int64_t ntiles, SplitWalk& walk,
+                                                int64_t& row, int64_t& k, long long* mailbox) {
+    if (threadIdx.x < 64) {  // wave 0
+        const int lane = threadIdx.x;
+        SplitTicket* tickets = split_tickets(header);
+        long long got_row = -1, got_k = -1;
+        for (;;) {
+            unsigned long long ticket;
+            if (walk.has_drawn) {
+                ticket = from_lane0(walk.drawn);
+                walk.has_drawn = false;
+            } else {
+                // first row at or after walk.row, cyclically, that still has tiles: 64 rows per look
+                long long found = -1;
+                for (int64_t base = 0; base < rows && found < 0; base += 64) {
+                    const int64_t idx = base + lane;
+                    bool has = false;
+                    if (idx < rows) {
+                        const int64_t r = walk.row + idx < rows ? walk.row + idx : walk.row + idx - rows;
+                        has = __hip_atomic_load(&tickets[r].next, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) <
+                              (unsigned long long)ntiles;
+                    }
+                    const unsigned long long mask = __ballot(has);
+                    if (mask) found = base + (long long)__builtin_ctzll(mask);
+                }
+                if (found < 0) break;  // nothing left anywhere
+                walk.row = walk.row + found < rows ? walk.row + found : walk.row + found - rows;
+                ticket = from_lane0(draw_ticket(&tickets[walk.row], lane));
+            }
+            if (ticket < (unsigned long long)ntiles) {
+                got_row = walk.row;
+                got_k = (long long)ticket;
+                if (ticket + 1 < (unsigned long long)ntiles) {  // draw the next one now; it is read at the next call
+                    walk.drawn = draw_ticket(&tickets[walk.row], lane);
+                    walk.has_drawn = true;
+                }
+                break;
+            }
+            // the row ran out (another workgroup took its last tile): look again
+        }
+        if (lane == 0) {
+            mailbox[0] = got_row;
+            mailbox[1] = got_k;
+        }
+    }
+    __syncthreads();
+    const long long got_row = mailbox[0];
+    const long long got_k = mailbox[1];
+    __syncthreads();  // the mailbox may be rewritten by the next call
+    if (got_row < 0) return false;
+    row = got_row;
+    k = got_k;
+    return true;
 }
 
 __device__ __forceinline__ float read_lane_at(float v, int lane) {
@@ -769,7 +866,7 @@ __device__ __forceinline__ V split_look_back(SplitHeader* header, SplitRecord* m
             V A = vone<V>(), X = vzero<V>();
             if (active) {
                 SplitRecord* prev = mine + q * stride;
-                const unsigned long long t0 = __builtin_amdgcn_s_memrealtime();
+                unsigned long long waited = 0, last = __builtin_amdgcn_s_memrealtime();
                 for (;;) {
                     V P, Aq, Xq;
                     if (peek(prev->p, P)) {
@@ -785,7 +882,10 @@ __device__ __forceinline__ V split_look_back(SplitHeader* header, SplitRecord* m
                         seen = 1;
                         break;
                     }
-                    if (__builtin_amdgcn_s_memrealtime() - t0 > limit) break;
+                    const unsigned long long now = __builtin_amdgcn_s_memrealtime();
+                    waited += now - last < kWaitStepCap ? now - last : kWaitStepCap;
+                    last = now;
+                    if (waited > limit) break;
                     __builtin_amdgcn_s_sleep(1);
                 }
             }
@@ -999,21 +1099,23 @@ __global__ void __launch_bounds__(64 * kMaxWavesPerBlock)
     const int64_t ntiles = tiles_per_row(longest, TILE, head);
     __shared__ V slots_all[W == 1 ? 1 : 2 * kSlotsPerBuffer];
     __shared__ S stage_all[PACKED ? W * SUB : 1];
-    // Split rows: a fixed set of co-resident workgroups walks over all (row,
-    // tile) pairs in order, all tiles of row 0 first; what is in flight at any
-    // time is one contiguous stretch of memory, and a workgroup only ever waits
-    // for tiles that resident workgroups are already working on.
-    const int64_t visits = SPLIT ? rows * ntiles : 1;
-    for (int64_t visit = SPLIT ? blockIdx.x : 0; visit < visits; visit += SPLIT ? gridDim.x : 1) {
+    // Split rows: the workgroups take tiles by ticket, row by row, until none
+    // is left; a workgroup only ever waits for tiles whose owners started before it.
+    __shared__ long long split_mailbox[2];
+    SplitWalk walk;  // starts at row blockIdx % rows
+    walk.row = SPLIT ? (int64_t)(blockIdx.x % rows) : 0;
+    walk.has_drawn = false;
+    for (bool first_visit = true;; first_visit = false) {
     int64_t row;
     int w, slot_base;
     int64_t k_begin = 0, k_end = ntiles;
     if constexpr (SPLIT) {
-        row = visit / ntiles;
-        k_begin = visit - row * ntiles;
+        if (!take_split_tile(split, rows, ntiles, walk, row, k_begin, split_mailbox)) break;
         k_end = k_begin + 1;
         w = threadIdx.x >> 6;
         slot_base = 0;
+    } else if (!first_visit) {
+        break;
     } else if constexpr (PACKED) {
         row = first_row;
         w = threadIdx.x >> 6;
@@ -1102,7 +1204,7 @@ __global__ void __launch_bounds__(64 * kMaxWavesPerBlock)
 
         V c;
         if constexpr (SPLIT) {
-            exchange_carries_split<V, W, U>(totA, totX, c, slots, w, lane, split, split_records(split) + row * ntiles, 1, k,
+            exchange_carries_split<V, W, U>(totA, totX, c, slots, w, lane, split, split_records(split, rows) + row * ntiles, 1, k,
                                             row_start);
         } else {
             exchange_carries<V, W, U>(totA, totX, carry, c, slots, (int)(k & 1), w, lane);
@@ -1180,21 +1282,23 @@ __global__ void __launch_bounds__(64 * kMaxWavesPerBlock)
     const int64_t ntiles = tiles_per_row(longest, TILE, head);
     __shared__ V slots_all[W == 1 ? 1 : 2 * kSlotsPerBuffer];
     __shared__ S stage_all[PACKED ? W * SUB : 1];
-    // Split rows: a fixed set of co-resident workgroups walks over all (row,
-    // tile) pairs in order, all tiles of row 0 first; what is in flight at any
-    // time is one contiguous stretch of memory, and a workgroup only ever waits
-    // for tiles that resident workgroups are already working on.
-    const int64_t visits = SPLIT ? rows * ntiles : 1;
-    for (int64_t visit = SPLIT ? blockIdx.x : 0; visit < visits; visit += SPLIT ? gridDim.x : 1) {
+    // Split rows: the workgroups take tiles by ticket, row by row, until none
+    // is left; a workgroup only ever waits for tiles whose owners started before it.
+    __shared__ long long split_mailbox[2];
+    SplitWalk walk;  // starts at row blockIdx % rows
+    walk.row = SPLIT ? (int64_t)(blockIdx.x % rows) : 0;
+    walk.has_drawn = false;
+    for (bool first_visit = true;; first_visit = false) {
     int64_t row;
     int w, slot_base;
     int64_t k_begin = 0, k_end = ntiles;
     if constexpr (SPLIT) {
-        row = visit / ntiles;
-        k_begin = visit - row * ntiles;
+        if (!take_split_tile(split, rows, ntiles, walk, row, k_begin, split_mailbox)) break;
         k_end = k_begin + 1;
         w = threadIdx.x >> 6;
         slot_base = 0;
+    } else if (!first_visit) {
+        break;
     } else if constexpr (PACKED) {
         row = first_row;
         w = threadIdx.x >> 6;
@@ -1346,7 +1450,7 @@ __global__ void __launch_bounds__(64 * kMaxWavesPerBlock)
 
         V c;
         if constexpr (SPLIT) {
-            exchange_carries_split<V, W, U>(totA, totX, c, slots, w, lane, split, split_records(split) + row * ntiles, 1, k,
+            exchange_carries_split<V, W, U>(totA, totX, c, slots, w, lane, split, split_records(split, rows) + row * ntiles, 1, k,
                                             vzero<V>());
         } else {
             exchange_carries<V, W, U>(totA, totX, carry, c, slots, (int)(k & 1), w, lane);
@@ -1592,7 +1696,8 @@ unsigned long long split_wait_limit() {
 bool want_split(int64_t rows, int64_t ntiles) { return rows <= split_max_rows() && ntiles >= 8; }
 
 size_t split_bytes(int64_t rows, int64_t ntiles) {
-    return sizeof(SplitHeader) + (size_t)rows * (size_t)ntiles * sizeof(SplitRecord);
+    return sizeof(SplitHeader) + (size_t)rows * sizeof(SplitTicket) +
+           (size_t)rows * (size_t)ntiles * sizeof(SplitRecord);
 }
 
 bool workspace_fits(const Workspace& ws, int64_t rows, int64_t ntiles) {
@@ -1614,18 +1719,20 @@ unsigned resident_workgroups(K kernel, int threads) {
     int device = 0;
     if (hipGetDevice(&device) != hipSuccess) return 0;
     constexpr int kMaxDevices = 64;
-    static unsigned cache[kMaxDevices] = {};  // 0 = not queried yet; one array per kernel instantiation
+    static std::atomic<unsigned> cache[kMaxDevices];  // 0 = not queried yet; one array per kernel instantiation
     if (device < 0 || device >= kMaxDevices) return 0;
-    if (cache[device] == 0) {
+    unsigned known = cache[device].load(std::memory_order_relaxed);
+    if (known == 0) {
         int per_cu = 0, cus = 0;
         if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, kernel, threads, 0) != hipSuccess ||
             hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, device) != hipSuccess ||
             per_cu <= 0 || cus <= 0) {
             return 0;
         }
-        cache[device] = (unsigned)per_cu * (unsigned)cus;
+        known = (unsigned)per_cu * (unsigned)cus;
+        cache[device].store(known, std::memory_order_relaxed);
     }
-    return cache[device];
+    return known;
 }
 
 // Tiles per row as the kernels count them (tiles_per_row on the device).

@@ -125,12 +125,15 @@ int ascan_backward(const void* gates, const void* states, const void* grad_out,
  *                          has completed.  NULL or a too-small buffer selects
  *                          the plain path.
  *
- * A workgroup waits for the workgroups of earlier tiles; tiles are handed out
- * in order, so those are always running already.  Every wait is bounded
- * (2 s by default); a wait that runs out writes NaN into the affected tile
- * and is counted: copy the first 64 bytes of the workspace to the host after
- * the stream has completed and pass them to ascan_workspace_timeouts (0 = all
- * waits were served).
+ * A workgroup waits for the workgroups of earlier tiles.  Tiles are handed out
+ * in order by a ticket counter per row, so the owner of a tile that is waited
+ * for has always started already: progress does not depend on how much of the
+ * GPU the call gets, and concurrent calls (each with its own workspace) are
+ * fine.  Every wait is bounded all the same (2 s of running time by default);
+ * a wait that runs out writes NaN into the affected tile and is counted: copy
+ * the first 64 bytes of the workspace to the host after the stream has
+ * completed and pass them to ascan_workspace_timeouts (0 = all waits were
+ * served).
  */
 size_t ascan_workspace_bytes(int64_t rows, int64_t seqlen, int dtype);
 

@@ -644,6 +644,47 @@ def test_split_matches_unsplit_and_autograd_path():
     assert _rel_err(dg, t_dg) <= 1e-5
 
 
+def test_split_calls_on_two_streams_at_once():
+    """Two split scans in flight together, each on its own stream with its own
+    table: tiles are handed out by ticket, so neither depends on workgroups the
+    other keeps from being dispatched.  Results equal those of the calls run
+    alone and no wait runs out."""
+    from accelerated_scan import _abi
+
+    lib = _abi.load()
+    rows, T = 8, 1 << 21
+    gen = torch.Generator().manual_seed(5)
+    inputs = []
+    for _ in range(2):
+        g = torch.rand(1, rows, T, generator=gen).to(DEVICE)
+        x = torch.randn(1, rows, T, generator=gen).to(DEVICE)
+        inputs.append((g, x))
+    nbytes = lib.ascan_workspace_bytes(rows, T, 0)
+    assert nbytes > 0
+    alone = []
+    for g, x in inputs:
+        out = torch.empty_like(g)
+        _abi.forward(g, x, out, False)
+        alone.append(out)
+    torch.cuda.synchronize()
+
+    streams = [torch.cuda.Stream(), torch.cuda.Stream()]
+    tables = [torch.empty(nbytes, dtype=torch.uint8, device=DEVICE) for _ in streams]
+    outs = [torch.empty_like(g) for g, _ in inputs]
+    for s in streams:
+        s.wait_stream(torch.cuda.current_stream())
+    for _ in range(8):  # interleaved launches keep both streams busy at the same time
+        for (g, x), out, table, s in zip(inputs, outs, tables, streams):
+            with torch.cuda.stream(s):
+                _abi.forward(g, x, out, False, workspace=table)
+    for s in streams:
+        torch.cuda.current_stream().wait_stream(s)
+    torch.cuda.synchronize()
+    for out, ref, table in zip(outs, alone, tables):
+        torch.testing.assert_close(out, ref, rtol=2e-6, atol=1e-6)
+        assert _abi.workspace_timeouts(table) == 0
+
+
 def test_split_wait_limit_is_an_exit_not_a_hang():
     """With the wait limit forced to zero from the host every workgroup still
     finishes; tiles whose predecessor was not ready are poisoned with NaN and
