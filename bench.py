@@ -39,8 +39,8 @@ HBM_PEAK_GBPS = 8000.0  # MI355X HBM3E, published peak
 # (FETCH_SIZE x 2.000 + WRITE_SIZE x 1.000 KiB, factors from a plain copy of
 # known size; summaries in profiles/).
 MEASURED_TRAFFIC_BYTES = {
-    ((8, 1536, 65536), "fp32"): (4721995 * 2 + 6292184) * 1024,
-    ((8, 1536, 65536), "bf16"): (2367212 * 2 + 3146553) * 1024,
+    ((8, 1536, 65536), "fp32"): (4721940 * 2 + 6292153) * 1024,
+    ((8, 1536, 65536), "bf16"): (2366704 * 2 + 3146428) * 1024,
 }
 
 
