@@ -1,0 +1,297 @@
+// The fused backward kernel.
+
+#ifndef ASCAN_BACKWARD_KERNEL_H_
+#define ASCAN_BACKWARD_KERNEL_H_
+
+#include <type_traits>
+
+#include "access.h"
+#include "carry.h"
+#include "gate.h"
+#include "packed.h"
+#include "split.h"
+
+namespace ascan {
+namespace {
+
+// ---------------------------------------------------------------------------
+// Fused backward kernel: reverse-time scan over gate[t+1] producing d_tokens,
+// and d_gates[t] = d_tokens[t] * conj(x[t-1]) in the same pass.
+// ---------------------------------------------------------------------------
+template <class Tr, int W, int U, bool ALIGNED, bool REGULAR, bool SPLIT, int ACT, bool PACKED>
+__global__ void __launch_bounds__(64 * kMaxWavesPerBlock)
+    scan_backward_kernel(const typename Tr::S* __restrict__ gates, const typename Tr::S* __restrict__ states,
+                         const typename Tr::S* __restrict__ grad_out, typename Tr::S* __restrict__ d_gates,
+                         typename Tr::TokS* __restrict__ d_tokens, int64_t rows, int64_t T, SplitHeader* split,
+                         const typename Tr::S* __restrict__ initial, typename Tr::S* __restrict__ d_initial, int G,
+                         int group) {
+    using S = typename Tr::S;
+    using V = typename Tr::V;
+    constexpr int EPV = Tr::EPV;
+    constexpr int64_t SUB = (int64_t)U * 64 * EPV;
+    constexpr int64_t TILE = SUB * W;
+    static_assert(!PACKED || (!SPLIT && !REGULAR), "packed rows use the general kernels, one group per workgroup");
+
+    const int lane = threadIdx.x & 63;
+    // Packed rows: this workgroup scans rows [first_row, first_row + nrows) as one row of `len` elements.
+    const int64_t first_row = PACKED ? (int64_t)blockIdx.x * group : 0;
+    const int64_t len = PACKED ? (rows - first_row < group ? rows - first_row : (int64_t)group) * T : T;
+    const int64_t longest = PACKED ? (int64_t)group * T : T;
+    // rows start at the same misalignment when their length is a multiple of the grid spacing
+    const int head = REGULAR ? 0 : (ALIGNED ? (longest % G == 0 ? row_lead<Tr>(gates, G) : G - 1) : 0);
+    const int64_t ntiles = tiles_per_row(longest, TILE, head);
+    __shared__ V slots_all[W == 1 ? 1 : 2 * kSlotsPerBuffer];
+    __shared__ S stage_all[PACKED ? W * SUB : 1];
+    // Split rows: the workgroups take tiles by ticket, row by row, until none
+    // is left; a workgroup only ever waits for tiles whose owners started before it.
+    __shared__ long long split_mailbox[2];
+    SplitWalk walk;  // starts at row blockIdx % rows
+    walk.row = SPLIT ? (int64_t)(blockIdx.x % rows) : 0;
+    walk.has_drawn = false;
+    for (bool first_visit = true;; first_visit = false) {
+    int64_t row;
+    int w, slot_base;
+    int64_t k_begin = 0, k_end = ntiles;
+    if constexpr (SPLIT) {
+        if (!take_split_tile(split, rows, ntiles, walk, row, k_begin, split_mailbox)) break;
+        k_end = k_begin + 1;
+        w = threadIdx.x >> 6;
+        slot_base = 0;
+    } else if (!first_visit) {
+        break;
+    } else if constexpr (PACKED) {
+        row = first_row;
+        w = threadIdx.x >> 6;
+        slot_base = 0;
+    } else {
+        if (!locate_wave<W>(rows, ntiles, row, w, slot_base)) return;  // wave-uniform
+    }
+    V* slots = slots_all + (W == 1 ? 0 : slot_base);
+
+    const int64_t lo = (ALIGNED && !REGULAR) ? row_lead<Tr>(gates + row * T, G) : 0;
+    const int64_t hi = lo + len;
+    const S* __restrict__ arow = gates + row * T - lo;
+    const S* __restrict__ xrow = states + row * T - lo;
+    const S* __restrict__ drow = grad_out + row * T - lo;
+    S* __restrict__ dgrow = d_gates + row * T - lo;
+    typename Tr::TokS* __restrict__ dtrow = d_tokens + row * T - lo;
+
+    V carry = vzero<V>();
+
+    // Gradient of x[-1], conj(gate[0]) * g[0], from g at position 0 of the row's
+    // first tile.  Positions below the row's first element (position lo) carry
+    // gate 1 and grad_out 0, so with lo > 0 that g already is the gradient;
+    // with lo == 0 the last factor is still missing.
+    auto store_start_gradient = [&](V g_low) {
+        if (lo == 0) g_low = vmul(vconj(activate1<ACT>(Tr::load1(arow))), g_low);
+        if (lane == 0) Tr::store1(d_initial + row, g_low);
+    };
+
+    // Position of this wave's sub-tile in tile step k (reverse time).
+    auto sub_tile_base = [&](int64_t k) {
+        const int64_t tile = ntiles - 1 - k;
+        return tile * TILE + (int64_t)(W - 1 - w) * SUB;
+    };
+    // One tile step of this wave; FULL as in the forward kernel.
+    auto tile_step = [&](int64_t k, auto full_tag) {
+        constexpr bool FULL = decltype(full_tag)::value;
+        const int64_t sub_base = sub_tile_base(k);
+        const int64_t sub_end = sub_base + SUB;
+        const Window win = make_window(lo, hi, sub_base);
+        const bool touches = FULL || (win.hi > 0 && win.lo < SUB);  // wave-uniform
+        const S* __restrict__ asub = arow + sub_base;
+        const S* __restrict__ dsub = drow + sub_base;
+        const S* __restrict__ xsub = xrow + sub_base;
+        S* __restrict__ dgsub = dgrow + sub_base;
+        typename Tr::TokS* __restrict__ dtsub = dtrow + sub_base;
+
+        // x[-1], the state the forward scan started from (absent = zero), is
+        // needed by the sub-tile that holds the row's first element
+        V x_start = vzero<V>();
+        if (!PACKED && initial != nullptr && sub_base <= lo && lo < sub_end) x_start = Tr::load1(initial + row);  // wave-uniform
+        Cuts<Tr> cuts;  // packed rows take their initial states at the cuts instead
+        if constexpr (PACKED) {
+            cuts = stage_row_starts<Tr>(initial != nullptr ? initial + first_row : nullptr, (int)T, (int)len,
+                                        (int)(sub_base - lo), (int)SUB, stage_all + w * SUB, lane);
+        }
+
+        u32x4_t araw[U], draw[U], xraw[U];
+        if (touches) {
+#pragma unroll
+            for (int j = 0; j < U; ++j) {
+                const int off = vec_offset<U, EPV, true>(j, lane);
+                araw[j] = load_raw<Tr, ALIGNED, FULL>(asub, off, win, identity_gate<ACT, V>());
+                draw[j] = load_raw<Tr, ALIGNED, FULL>(dsub, off, win, vzero<V>());
+                xraw[j] = load_raw<Tr, ALIGNED, FULL>(xsub, off, win, x_start);
+            }
+        } else {
+#pragma unroll
+            for (int j = 0; j < U; ++j) {
+                araw[j] = fill_raw<Tr>(identity_gate<ACT, V>());
+                draw[j] = fill_raw<Tr>(vzero<V>());
+                xraw[j] = fill_raw<Tr>(x_start);
+            }
+        }
+
+        // The two elements just outside the sub-tile: gate at sub_end and x at
+        // sub_base-1.  Addresses are clamped into the row so the loads are
+        // unconditional; out-of-row positions take the identity gate and x[-1].
+        V a_edge, x_edge;
+        {
+            const int64_t ia = sub_end < hi ? (sub_end > lo ? sub_end : lo) : hi - 1;
+            int64_t ix = sub_base - 1;
+            ix = ix < lo ? lo : (ix < hi ? ix : hi - 1);
+            const V av = activate1<ACT>(Tr::load1(arow + ia));
+            const V xv = Tr::load1(xrow + ix);
+            a_edge = vselect(sub_end >= lo && sub_end < hi, av, vone<V>());
+            x_edge = vselect(sub_base - 1 >= lo && sub_base - 1 < hi, xv, x_start);
+        }
+
+        // Pass 1.  Gates are needed one element later (gate[t+1]) and states one
+        // element earlier (x[t-1]).  In scan order the vector at the next higher
+        // address belongs to lane-1 and the one at the next lower address to
+        // lane+1, so each block needs one value from each neighbour: a_next (the
+        // first gate of the vector above) and x_prev (the last state of the
+        // vector below).
+        V a_next[U], x_prev[U];
+        V totA[U], totX[U], exA[U], exX[U];
+#pragma unroll
+        for (int j = 0; j < U; ++j) {
+            V a[EPV], d[EPV], x[EPV];
+            Tr::unpack(araw[j], a);
+            activate<ACT>(a);
+            Tr::unpack(draw[j], d);
+            Tr::unpack(xraw[j], x);
+            V hi_edge, lo_edge;
+            if (j == 0) {
+                hi_edge = a_edge;
+            } else {
+                V above[EPV];
+                Tr::unpack(araw[j > 0 ? j - 1 : 0], above);
+                hi_edge = read_lane<63>(activate1<ACT>(above[0]));
+            }
+            if (j == U - 1) {
+                lo_edge = x_edge;
+            } else {
+                V below[EPV];
+                Tr::unpack(xraw[j < U - 1 ? j + 1 : j], below);
+                lo_edge = read_lane<0>(below[EPV - 1]);
+            }
+            a_next[j] = shift_up1(a[0], hi_edge);
+            x_prev[j] = shift_down1(x[EPV - 1], lo_edge);
+
+            // after[e]: the gate that follows element e; before[e]: the state that precedes it
+            V after[EPV], before[EPV];
+#pragma unroll
+            for (int e = 0; e < EPV; ++e) {
+                after[e] = e < EPV - 1 ? a[e + 1] : a_next[j];
+                before[e] = e > 0 ? x[e - 1] : x_prev[j];
+            }
+            if constexpr (PACKED) {
+                bool is_first[EPV];
+                int row_of[EPV];
+                cut_rows_backward<Tr>(after, before, is_first, row_of,
+                                      (int)(sub_base - lo) + vec_offset<U, EPV, true>(j, lane), cuts);
+            }
+            V A = vconj(after[EPV - 1]);
+            V X = d[EPV - 1];
+#pragma unroll
+            for (int e = EPV - 2; e >= 0; --e) {
+                const V ga = vconj(after[e]);
+                X = vfma(ga, X, d[e]);
+                A = vmul(A, ga);
+            }
+            wave_scan_inclusive(A, X);
+            totA[j] = read_lane<63>(A);
+            totX[j] = read_lane<63>(X);
+            exA[j] = shift_up1(A, vone<V>());
+            exX[j] = shift_up1(X, vzero<V>());
+        }
+
+        V c;
+        if constexpr (SPLIT) {
+            exchange_carries_split<V, W, U>(totA, totX, c, slots, w, lane, split, split_records(split, rows) + row * ntiles, 1, k,
+                                            vzero<V>());
+        } else {
+            exchange_carries<V, W, U>(totA, totX, carry, c, slots, (int)(k & 1), w, lane);
+        }
+        // Pass 2: the plain reverse recurrence and the gate gradient.
+#pragma unroll
+        for (int j = 0; j < U; ++j) {
+            if constexpr (Tr::kNarrow) {
+                forget_unpacked(araw[j]);
+                forget_unpacked(draw[j]);
+                forget_unpacked(xraw[j]);
+            }
+            V a[EPV], d[EPV], x[EPV];
+            Tr::unpack(araw[j], a);
+            activate<ACT>(a);
+            Tr::unpack(draw[j], d);
+            Tr::unpack(xraw[j], x);
+            V gr = vfma(exA[j], c, exX[j]);  // g entering this lane's vector from above
+            c = vfma(totA[j], c, totX[j]);
+            const int off = vec_offset<U, EPV, true>(j, lane);
+            V after[EPV], before[EPV];
+#pragma unroll
+            for (int e = 0; e < EPV; ++e) {
+                after[e] = e < EPV - 1 ? a[e + 1] : a_next[j];
+                before[e] = e > 0 ? x[e - 1] : x_prev[j];
+            }
+            bool is_first[EPV];
+            int row_of[EPV];
+            if constexpr (PACKED) {
+                cut_rows_backward<Tr>(after, before, is_first, row_of, (int)(sub_base - lo) + off, cuts);
+            }
+            V dt[EPV], dg[EPV];
+#pragma unroll
+            for (int e = EPV - 1; e >= 0; --e) {
+                gr = vfma(vconj(after[e]), gr, d[e]);
+                dt[e] = gr;
+                dg[e] = vmul(gr, vconj(before[e]));
+                if constexpr (ACT != kGateIdentity) dg[e] = vmul(dg[e], gate_slope<ACT>(a[e]));
+            }
+            if (touches) {
+                store_tok_vec<Tr, ALIGNED, FULL>(dtsub, off, win, dt);
+                store_vec<Tr, ALIGNED, FULL>(dgsub, off, win, dg);
+            }
+            if constexpr (PACKED) {
+                // gradient of each row's initial state, conj(gate[0]) * g[0], from the lane that holds the row's start
+                if (d_initial != nullptr) {
+#pragma unroll
+                    for (int e = 0; e < EPV; ++e) {
+                        if (is_first[e]) Tr::store1(d_initial + first_row + row_of[e], vmul(vconj(a[e]), dt[e]));
+                    }
+                }
+            }
+        }
+
+        // A split row's last tile step ends at the row's first element: after
+        // pass 2, c is g at the lowest position of this wave's sub-tile.
+        if constexpr (SPLIT) {
+            if (d_initial != nullptr && k == ntiles - 1 && w == W - 1) store_start_gradient(c);  // wave-uniform
+        }
+    };
+
+    for (int64_t k = k_begin; k < k_end; ++k) {
+        if constexpr (REGULAR) {
+            tile_step(k, std::true_type{});
+        } else {
+            const int64_t sub_base = sub_tile_base(k);
+            if (sub_base >= lo && sub_base + SUB <= hi) {  // wave-uniform
+                tile_step(k, std::true_type{});
+            } else {
+                tile_step(k, std::false_type{});
+            }
+        }
+    }
+    // after the last tile step the carry is g at position 0 of the first tile
+    if constexpr (!SPLIT && !PACKED) {
+        if (d_initial != nullptr && w == 0) store_start_gradient(carry);  // wave-uniform
+    }
+    }  // visits
+}
+
+}  // namespace
+}  // namespace ascan
+
+#endif  // ASCAN_BACKWARD_KERNEL_H_

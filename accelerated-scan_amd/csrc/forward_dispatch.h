@@ -1,0 +1,145 @@
+// Chooses and launches the forward kernel of a call for one dtype.
+#ifndef ASCAN_FORWARD_DISPATCH_H_
+#define ASCAN_FORWARD_DISPATCH_H_
+
+#include "forward_kernel.h"
+#include "policy.h"
+
+namespace ascan {
+namespace {
+
+template <class Tr, int W, bool REV, bool ALIGNED, bool REGULAR, int ACT>
+hipError_t launch_forward(const void* gates, const void* tokens, void* out, const void* initial, int64_t rows,
+                          int64_t T, int grid, int rows_per_block, hipStream_t stream) {
+    using S = typename Tr::S;
+    using TokS = typename Tr::TokS;
+    constexpr int U = REGULAR ? Tuning<Tr>::U : Tuning<Tr>::UG;
+    const unsigned blocks = (unsigned)((rows + rows_per_block - 1) / rows_per_block);
+    const unsigned threads = 64u * W * rows_per_block;
+    return launch(scan_forward_kernel<Tr, W, U, REV, ALIGNED, REGULAR, false, ACT, false>, blocks, threads, stream,
+                  static_cast<const S*>(gates), static_cast<const TokS*>(tokens), static_cast<S*>(out), rows, T,
+                  static_cast<SplitHeader*>(nullptr), static_cast<const S*>(initial), grid, 0);
+}
+
+template <class Tr, bool REV, bool REGULAR, int ACT>
+hipError_t launch_forward_split(const void* gates, const void* tokens, void* out, const void* initial, int64_t rows,
+                                int64_t T, int grid, int64_t ntiles, const Workspace& ws, hipStream_t stream) {
+    using S = typename Tr::S;
+    using TokS = typename Tr::TokS;
+    constexpr int U = REGULAR ? Tuning<Tr>::U : Tuning<Tr>::UG;
+    auto kernel = scan_forward_kernel<Tr, kSplitWaves, U, REV, true, REGULAR, true, ACT, false>;
+    const unsigned resident = resident_workgroups(kernel, 64 * kSplitWaves);
+    if (resident == 0) return hipErrorInvalidConfiguration;
+    const hipError_t e = reset_split_table(ws, rows, ntiles, stream);
+    if (e != hipSuccess) return e;
+    const int64_t tiles = rows * ntiles;
+    return launch(kernel, (unsigned)(tiles < resident ? tiles : resident), 64u * kSplitWaves, stream,
+                  static_cast<const S*>(gates), static_cast<const TokS*>(tokens), static_cast<S*>(out), rows, T,
+                  static_cast<SplitHeader*>(ws.ptr), static_cast<const S*>(initial), grid, 0);
+}
+
+template <class Tr, bool REV, bool ALIGNED, int ACT>
+hipError_t launch_forward_packed(const void* gates, const void* tokens, void* out, const void* initial, int64_t rows,
+                                 int64_t T, int grid, int group, hipStream_t stream) {
+    using S = typename Tr::S;
+    using TokS = typename Tr::TokS;
+    const unsigned blocks = (unsigned)((rows + group - 1) / group);
+    return launch(scan_forward_kernel<Tr, kPackedWaves, Tuning<Tr>::UG, REV, ALIGNED, false, false, ACT, true>, blocks,
+                  64u * kPackedWaves, stream, static_cast<const S*>(gates), static_cast<const TokS*>(tokens),
+                  static_cast<S*>(out), rows, T, static_cast<SplitHeader*>(nullptr), static_cast<const S*>(initial),
+                  grid, group);
+}
+
+template <class Tr>
+int forward_typed(const void* gates, const void* tokens, void* out, const void* initial, int64_t rows, int64_t T,
+                  bool reverse, int act, const Workspace& ws, hipStream_t stream) {
+    constexpr int64_t kElem = (int64_t)sizeof(typename Tr::S);
+    constexpr int64_t SUB = (int64_t)Tuning<Tr>::U * 64 * Tr::EPV;    // regular kernels
+    constexpr int64_t SUBG = (int64_t)Tuning<Tr>::UG * 64 * Tr::EPV;  // kernels with masking code
+    Plan plan = choose_plan(T, SUB, kElem);
+    const void* const state_like[] = {gates, out};
+    const Lead at = find_lead<Tr>(state_like, tokens);
+    const bool same_lead = at.same;
+    const int lead = at.lead;
+    const Access access = choose_access(same_lead, lead, T, SUB * plan.waves_per_row);
+    if (access != Access::kRegular) plan = choose_plan(T, SUBG, kElem);
+    const int R = plan.rows_per_block;
+    hipError_t err = hipSuccess;
+    if (const int group = packed_group(rows, T, kElem, SUBG * kPackedWaves, same_lead ? at.grid : 1)) {
+#define ASCAN_FWD_PACKED(REV, AL, ACT) \
+    launch_forward_packed<Tr, REV, AL, ACT>(gates, tokens, out, initial, rows, T, at.grid, group, stream)
+        if (act == kGateSigmoid) {
+            if constexpr (kHasSigmoid<Tr>) {
+                err = same_lead ? ASCAN_FWD_PACKED(false, true, kGateSigmoid) : ASCAN_FWD_PACKED(false, false, kGateSigmoid);
+            }
+        } else if (same_lead) {
+            err = reverse ? ASCAN_FWD_PACKED(true, true, kGateIdentity) : ASCAN_FWD_PACKED(false, true, kGateIdentity);
+        } else {
+            err = reverse ? ASCAN_FWD_PACKED(true, false, kGateIdentity) : ASCAN_FWD_PACKED(false, false, kGateIdentity);
+        }
+#undef ASCAN_FWD_PACKED
+        return launch_status(err);
+    }
+    if (same_lead && ws.ptr != nullptr) {
+        const bool regular = lead == 0 && T % (SUB * kSplitWaves) == 0;
+        const int64_t ntiles = host_tiles_per_row<Tr>(T, (regular ? SUB : SUBG) * kSplitWaves, regular, at);
+        if (want_split(rows, ntiles) && workspace_fits(ws, rows, ntiles)) {
+#define ASCAN_FWD_SPLIT(REV, REG, ACT) \
+    launch_forward_split<Tr, REV, REG, ACT>(gates, tokens, out, initial, rows, T, at.grid, ntiles, ws, stream)
+            if (act == kGateSigmoid) {
+                if constexpr (kHasSigmoid<Tr>) {
+                    err = regular ? ASCAN_FWD_SPLIT(false, true, kGateSigmoid) : ASCAN_FWD_SPLIT(false, false, kGateSigmoid);
+                }
+            } else if (regular) {
+                err = reverse ? ASCAN_FWD_SPLIT(true, true, kGateIdentity) : ASCAN_FWD_SPLIT(false, true, kGateIdentity);
+            } else {
+                err = reverse ? ASCAN_FWD_SPLIT(true, false, kGateIdentity) : ASCAN_FWD_SPLIT(false, false, kGateIdentity);
+            }
+#undef ASCAN_FWD_SPLIT
+            return launch_status(err);
+        }
+    }
+#define ASCAN_FWD_ARGS gates, tokens, out, initial, rows, T, at.grid, R, stream
+#define ASCAN_FWD(WV, AL, REG)                                                                  \
+    do {                                                                                        \
+        if (act == kGateSigmoid) {                                                              \
+            if constexpr (kHasSigmoid<Tr>)                                                      \
+                err = launch_forward<Tr, WV, false, AL, REG, kGateSigmoid>(ASCAN_FWD_ARGS);     \
+        } else if (reverse) {                                                                   \
+            err = launch_forward<Tr, WV, true, AL, REG, kGateIdentity>(ASCAN_FWD_ARGS);         \
+        } else {                                                                                \
+            err = launch_forward<Tr, WV, false, AL, REG, kGateIdentity>(ASCAN_FWD_ARGS);        \
+        }                                                                                       \
+    } while (0)
+#define ASCAN_FWD_W(AL, REG)                            \
+    switch (plan.waves_per_row) {                       \
+        case 1: ASCAN_FWD(1, AL, REG); break;           \
+        case 2: ASCAN_FWD(2, AL, REG); break;           \
+        case 4: ASCAN_FWD(4, AL, REG); break;           \
+        case 8: ASCAN_FWD(8, AL, REG); break;           \
+        default: ASCAN_FWD(16, AL, REG); break;         \
+    }
+    if (access == Access::kRegular) {
+        ASCAN_FWD_W(true, true);
+    } else if (access == Access::kVector) {
+        ASCAN_FWD_W(true, false);
+    } else {
+        ASCAN_FWD_W(false, false);
+    }
+#undef ASCAN_FWD_W
+#undef ASCAN_FWD
+#undef ASCAN_FWD_ARGS
+    return launch_status(err);
+}
+
+}  // namespace
+}  // namespace ascan
+
+// Defines ascan::NAME, the forward entry of one dtype, in the including file.
+#define ASCAN_DEFINE_FORWARD(NAME, TRAITS)                                                              \
+    int ascan::NAME(const ascan::ForwardCall& c) {                                                      \
+        return ascan::forward_typed<ascan::TRAITS>(c.gates, c.tokens, c.out, c.initial, c.rows, c.seqlen, \
+                                                   c.reverse, c.gate, c.workspace, c.stream);           \
+    }
+
+#endif  // ASCAN_FORWARD_DISPATCH_H_

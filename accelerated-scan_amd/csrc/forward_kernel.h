@@ -1,0 +1,203 @@
+// The forward / reverse scan kernel.
+
+#ifndef ASCAN_FORWARD_KERNEL_H_
+#define ASCAN_FORWARD_KERNEL_H_
+
+#include <type_traits>
+
+#include "access.h"
+#include "carry.h"
+#include "gate.h"
+#include "packed.h"
+#include "split.h"
+
+namespace ascan {
+namespace {
+
+// ---------------------------------------------------------------------------
+// Forward kernel (REV = false) and plain reverse scan (REV = true).
+// A workgroup holds R rows x W waves per row (R = blockDim.x / 64 / W); the
+// rows of a workgroup are adjacent in memory, so with W*R = 16 one tile step
+// of the workgroup covers one contiguous span of 16 sub-tiles.
+// ---------------------------------------------------------------------------
+template <class Tr, int W, int U, bool REV, bool ALIGNED, bool REGULAR, bool SPLIT, int ACT, bool PACKED>
+__global__ void __launch_bounds__(64 * kMaxWavesPerBlock)
+    scan_forward_kernel(const typename Tr::S* __restrict__ gates, const typename Tr::TokS* __restrict__ tokens,
+                        typename Tr::S* __restrict__ out, int64_t rows, int64_t T, SplitHeader* split,
+                        const typename Tr::S* __restrict__ initial, int G, int group) {
+    using S = typename Tr::S;
+    using V = typename Tr::V;
+    constexpr int EPV = Tr::EPV;
+    constexpr int64_t SUB = (int64_t)U * 64 * EPV;
+    constexpr int64_t TILE = SUB * W;
+    static_assert(!PACKED || (!SPLIT && !REGULAR), "packed rows use the general kernels, one group per workgroup");
+
+    const int lane = threadIdx.x & 63;
+    // Packed rows: this workgroup scans rows [first_row, first_row + nrows) as one row of `len` elements.
+    const int64_t first_row = PACKED ? (int64_t)blockIdx.x * group : 0;
+    const int64_t len = PACKED ? (rows - first_row < group ? rows - first_row : (int64_t)group) * T : T;
+    const int64_t longest = PACKED ? (int64_t)group * T : T;
+    // rows start at the same misalignment when their length is a multiple of the grid spacing
+    const int head = REGULAR ? 0 : (ALIGNED ? (longest % G == 0 ? row_lead<Tr>(gates, G) : G - 1) : 0);
+    const int64_t ntiles = tiles_per_row(longest, TILE, head);
+    __shared__ V slots_all[W == 1 ? 1 : 2 * kSlotsPerBuffer];
+    __shared__ S stage_all[PACKED ? W * SUB : 1];
+    // Split rows: the workgroups take tiles by ticket, row by row, until none
+    // is left; a workgroup only ever waits for tiles whose owners started before it.
+    __shared__ long long split_mailbox[2];
+    SplitWalk walk;  // starts at row blockIdx % rows
+    walk.row = SPLIT ? (int64_t)(blockIdx.x % rows) : 0;
+    walk.has_drawn = false;
+    for (bool first_visit = true;; first_visit = false) {
+    int64_t row;
+    int w, slot_base;
+    int64_t k_begin = 0, k_end = ntiles;
+    if constexpr (SPLIT) {
+        if (!take_split_tile(split, rows, ntiles, walk, row, k_begin, split_mailbox)) break;
+        k_end = k_begin + 1;
+        w = threadIdx.x >> 6;
+        slot_base = 0;
+    } else if (!first_visit) {
+        break;
+    } else if constexpr (PACKED) {
+        row = first_row;
+        w = threadIdx.x >> 6;
+        slot_base = 0;
+    } else {
+        if (!locate_wave<W>(rows, ntiles, row, w, slot_base)) return;  // wave-uniform
+    }
+    V* slots = slots_all + (W == 1 ? 0 : slot_base);
+
+    const int64_t lo = (ALIGNED && !REGULAR) ? row_lead<Tr>(gates + row * T, G) : 0;
+    const int64_t hi = lo + len;
+    const S* __restrict__ grow = gates + row * T - lo;
+    const typename Tr::TokS* __restrict__ trow = tokens + row * T - lo;
+    S* __restrict__ orow = out + row * T - lo;
+
+    // state the row starts from (one element per row; absent = zero); a split
+    // row needs it in its first tile only; packed rows take theirs at the cuts
+    const V row_start =
+        (!PACKED && initial != nullptr && (!SPLIT || k_begin == 0)) ? Tr::load1(initial + row) : vzero<V>();
+    V carry = row_start;
+
+    // Position of this wave's sub-tile in tile step k.
+    auto sub_tile_base = [&](int64_t k) {
+        const int64_t tile = REV ? (ntiles - 1 - k) : k;
+        return tile * TILE + (int64_t)(REV ? (W - 1 - w) : w) * SUB;
+    };
+    // One tile step of this wave.  FULL (a compile-time flag) says that the
+    // wave's sub-tile lies entirely inside the row: that copy of the body has no
+    // masking code.  The other copy serves the (at most two) ragged tiles of a
+    // row; it exists only in the kernels for arbitrary row starts and lengths.
+    auto tile_step = [&](int64_t k, auto full_tag) {
+        constexpr bool FULL = decltype(full_tag)::value;
+        const int64_t sub_base = sub_tile_base(k);
+        const Window win = make_window(lo, hi, sub_base);
+        const bool touches = FULL || (win.hi > 0 && win.lo < SUB);  // wave-uniform
+        const S* __restrict__ gsub = grow + sub_base;
+        const typename Tr::TokS* __restrict__ tsub = trow + sub_base;
+        S* __restrict__ osub = orow + sub_base;
+
+        Cuts<Tr> cuts;
+        if constexpr (PACKED) {
+            cuts = stage_row_starts<Tr>(initial != nullptr ? initial + first_row : nullptr, (int)T, (int)len,
+                                        (int)(sub_base - lo), (int)SUB, stage_all + w * SUB, lane);
+        }
+
+        u32x4_t graw[U], traw[U];
+        if (touches) {
+#pragma unroll
+            for (int j = 0; j < U; ++j) {
+                const int off = vec_offset<U, EPV, REV>(j, lane);
+                graw[j] = load_raw<Tr, ALIGNED, FULL>(gsub, off, win, identity_gate<ACT, V>());
+                traw[j] = load_tok_raw<Tr, ALIGNED, FULL>(tsub, off, win, vzero<V>());
+            }
+        } else {
+#pragma unroll
+            for (int j = 0; j < U; ++j) {
+                graw[j] = fill_raw<Tr>(identity_gate<ACT, V>());
+                traw[j] = fill_raw<Tr>(vzero<V>());
+            }
+        }
+
+        // Pass 1: fold each vector into one (A, X) pair and scan the pairs.
+        V totA[U], totX[U], exA[U], exX[U];
+#pragma unroll
+        for (int j = 0; j < U; ++j) {
+            V g[EPV], t[EPV];
+            Tr::unpack(graw[j], g);
+            activate<ACT>(g);
+            Tr::unpack(traw[j], t);
+            if constexpr (PACKED) cut_rows<Tr, REV>(g, t, (int)(sub_base - lo) + vec_offset<U, EPV, REV>(j, lane), cuts);
+            constexpr int e0 = REV ? EPV - 1 : 0;
+            V A = g[e0];
+            V X = t[e0];
+#pragma unroll
+            for (int i = 1; i < EPV; ++i) {
+                const int e = REV ? EPV - 1 - i : i;
+                X = vfma(g[e], X, t[e]);
+                A = vmul(A, g[e]);
+            }
+            wave_scan_inclusive(A, X);
+            totA[j] = read_lane<63>(A);
+            totX[j] = read_lane<63>(X);
+            exA[j] = shift_up1(A, vone<V>());
+            exX[j] = shift_up1(X, vzero<V>());
+        }
+
+        V c;
+        if constexpr (SPLIT) {
+            exchange_carries_split<V, W, U>(totA, totX, c, slots, w, lane, split, split_records(split, rows) + row * ntiles, 1, k,
+                                            row_start);
+        } else {
+            exchange_carries<V, W, U>(totA, totX, carry, c, slots, (int)(k & 1), w, lane);
+        }
+
+        // Pass 2: the plain recurrence from the state entering each lane.
+#pragma unroll
+        for (int j = 0; j < U; ++j) {
+            if constexpr (Tr::kNarrow) {
+                forget_unpacked(graw[j]);
+                forget_unpacked(traw[j]);
+            }
+            V g[EPV], t[EPV];
+            Tr::unpack(graw[j], g);
+            activate<ACT>(g);
+            Tr::unpack(traw[j], t);
+            if constexpr (PACKED) cut_rows<Tr, REV>(g, t, (int)(sub_base - lo) + vec_offset<U, EPV, REV>(j, lane), cuts);
+            V x = vfma(exA[j], c, exX[j]);  // state entering this lane's vector
+            c = vfma(totA[j], c, totX[j]);  // state entering the next block
+            V o[EPV];
+#pragma unroll
+            for (int i = 0; i < EPV; ++i) {
+                const int e = REV ? EPV - 1 - i : i;
+                x = vfma(g[e], x, t[e]);
+                o[e] = x;
+            }
+            const int off = vec_offset<U, EPV, REV>(j, lane);
+            if (touches) store_vec<Tr, ALIGNED, FULL>(osub, off, win, o);
+        }
+    };
+
+    // (Issuing the loads of step k+1 before the arithmetic of step k was tried
+    // and measured no faster: the memory system is already saturated by the
+    // other workgroups.)
+    for (int64_t k = k_begin; k < k_end; ++k) {
+        if constexpr (REGULAR) {
+            tile_step(k, std::true_type{});
+        } else {
+            const int64_t sub_base = sub_tile_base(k);
+            if (sub_base >= lo && sub_base + SUB <= hi) {  // wave-uniform
+                tile_step(k, std::true_type{});
+            } else {
+                tile_step(k, std::false_type{});
+            }
+        }
+    }
+    }  // visits
+}
+
+}  // namespace
+}  // namespace ascan
+
+#endif  // ASCAN_FORWARD_KERNEL_H_

@@ -1,0 +1,255 @@
+// Host-side policy shared by the forward and the backward dispatch: tile sizes,
+// launch geometry, where the tensors sit on the alignment grid, and when rows
+// are split over workgroups or packed into groups.
+#ifndef ASCAN_POLICY_H_
+#define ASCAN_POLICY_H_
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+#include <stdlib.h>
+
+#include <atomic>
+#include <type_traits>
+
+#include "ascan.h"
+#include "dispatch.h"
+#include "split.h"
+#include "traits.h"
+
+namespace ascan {
+namespace {
+
+// Blocks (64 vectors = 1 KiB of a tensor each) per wave and tile step:
+//   U / UB    forward / backward kernels of regular shapes: 4 KiB of each
+//             tensor per wave, except the complex backward kernel (its three
+//             inputs plus complex temporaries would spill);
+//   UG / UBG  the same for the kernels that carry masking code (rows of
+//             arbitrary start and length), which need registers for the masks.
+template <class Tr> struct Tuning;
+template <> struct Tuning<TraitsF32> { static constexpr int U = 4, UG = 4, UB = 4, UBG = 2; };
+template <> struct Tuning<TraitsBF16> { static constexpr int U = 4, UG = 2, UB = 4, UBG = 2; };
+template <> struct Tuning<TraitsF16> { static constexpr int U = 4, UG = 2, UB = 4, UBG = 2; };
+template <> struct Tuning<TraitsC64> { static constexpr int U = 4, UG = 4, UB = 2, UBG = 2; };
+template <> struct Tuning<TraitsC64RealTokens> : Tuning<TraitsC64> {};
+
+// Launch geometry: W waves per row, R rows per workgroup (W*R <= 16).
+struct Plan {
+    int waves_per_row;
+    int rows_per_block;
+};
+
+int env_int(const char* name) {
+    const char* s = getenv(name);
+    return s ? atoi(s) : 0;
+}
+
+// Optional overrides for tuning runs, read once per process:
+// ASCAN_WAVES_PER_ROW in {1,2,4,8,16}, ASCAN_ROWS_PER_BLOCK in {1,2,4,8,16}.
+const Plan& forced_plan() {
+    static const Plan p = [] {
+        auto pow2 = [](int n) { return (n == 1 || n == 2 || n == 4 || n == 8 || n == 16) ? n : 0; };
+        return Plan{pow2(env_int("ASCAN_WAVES_PER_ROW")), pow2(env_int("ASCAN_ROWS_PER_BLOCK"))};
+    }();
+    return p;
+}
+
+// Measured on MI355X: what counts is how few rows are being streamed at any
+// one time.  With every wave on its own row the memory system sees thousands
+// of concurrent streams and tops out near 5.0 TB/s; with 16 waves marching
+// along one row it reaches the 5.7-6.1 TB/s of a plain linear sweep.  So a row
+// gets as many waves as it has sub-tiles (up to 16).  Short rows keep small
+// workgroups (256 threads, several rows each): packing more short rows into
+// one large workgroup measured slower.
+Plan choose_plan(int64_t T, int64_t sub, int64_t element_bytes) {
+    const Plan& forced = forced_plan();
+    // one wave per 4 KiB of row, but never more waves than sub-tiles
+    int w = 1;
+    while (w < kMaxWavesPerBlock && (int64_t)w * 4096 < T * element_bytes && (int64_t)w * sub < T) w *= 2;
+    if (forced.waves_per_row) w = forced.waves_per_row;
+    int r = w >= 4 ? 1 : 4 / w;
+    if (forced.rows_per_block) r = forced.rows_per_block;
+    if (w * r > kMaxWavesPerBlock) r = kMaxWavesPerBlock / w;
+    return Plan{w, r};
+}
+
+// Offset of an address from the grid boundary below it, in elements of
+// `elem_bytes` bytes; boundaries are `grid` elements apart.  Tensors whose first
+// elements have the same lead line up vector by vector, row by row.
+int lead_of(const void* p, size_t elem_bytes, int grid) {
+    return (int)((reinterpret_cast<uintptr_t>(p) / elem_bytes) % (unsigned)grid);
+}
+
+// The grid rows are addressed from (elements between boundaries) and where the
+// call's tensors sit on it.
+struct Lead {
+    int grid;   // 128 bytes of states when all tensors agree there, else one 16-byte vector
+    int lead;   // of the first tensor
+    bool same;  // all tensors share `lead` on `grid`
+};
+
+template <class Tr, size_t N>
+Lead find_lead(const void* const (&state_like)[N], const void* token_like) {
+    constexpr size_t kElem = sizeof(typename Tr::S);
+    for (int grid : {(int)(128 / kElem), Tr::EPV}) {
+        const int lead = lead_of(state_like[0], kElem, grid);
+        bool same = lead_of(token_like, sizeof(typename Tr::TokS), grid) == lead;
+        for (size_t i = 1; i < N; ++i) same = same && lead_of(state_like[i], kElem, grid) == lead;
+        if (same || grid == Tr::EPV) return Lead{grid, lead, same};
+    }
+    return Lead{Tr::EPV, 0, false};  // not reached
+}
+
+// Launches through hipLaunchKernel so that the launch's own status comes back
+// (the <<<>>> form reports through the thread's sticky last-error slot, which
+// may hold an error of the caller's).
+template <class... Args>
+hipError_t launch(void (*kernel)(Args...), unsigned blocks, unsigned threads, hipStream_t stream, Args... args) {
+    void* argv[] = {static_cast<void*>(&args)...};
+    return hipLaunchKernel(reinterpret_cast<const void*>(kernel), dim3(blocks), dim3(threads), argv, 0, stream);
+}
+
+inline int launch_status(hipError_t e) {
+    if (e != hipSuccess) {
+        g_last_hip_error = (int)e;
+        return ASCAN_ERR_LAUNCH;
+    }
+    return ASCAN_OK;
+}
+
+
+// Split-row policy.  A call is split when its rows alone would leave most
+// compute units without a workgroup and every row has several tiles.  Split
+// tiles are small (4 waves) so that several workgroups share a compute unit
+// and overlap each other's loads, waits and stores.
+constexpr int kSplitWaves = 4;
+constexpr int64_t kSplitMaxRowsDefault = 128;
+
+int64_t split_max_rows() {
+    static const int64_t v = [] {
+        const char* s = getenv("ASCAN_SPLIT_MAX_ROWS");
+        return s ? (int64_t)atoll(s) : kSplitMaxRowsDefault;
+    }();
+    return v;
+}
+
+// Longest single wait of a workgroup for an earlier tile, in 100 MHz ticks
+// (default 2 s; ASCAN_SPLIT_WAIT_US overrides, read once).
+unsigned long long split_wait_limit() {
+    static const unsigned long long v = [] {
+        const char* s = getenv("ASCAN_SPLIT_WAIT_US");
+        const unsigned long long us = s ? strtoull(s, nullptr, 10) : 2000000ull;
+        return us * 100ull;
+    }();
+    return v;
+}
+
+bool want_split(int64_t rows, int64_t ntiles) { return rows <= split_max_rows() && ntiles >= 8; }
+
+size_t split_bytes(int64_t rows, int64_t ntiles) {
+    return sizeof(SplitHeader) + (size_t)rows * sizeof(SplitTicket) +
+           (size_t)rows * (size_t)ntiles * sizeof(SplitRecord);
+}
+
+bool workspace_fits(const Workspace& ws, int64_t rows, int64_t ntiles) {
+    return ws.ptr != nullptr && (reinterpret_cast<uintptr_t>(ws.ptr) % alignof(SplitRecord)) == 0 &&
+           ws.bytes >= split_bytes(rows, ntiles);
+}
+
+hipError_t reset_split_table(const Workspace& ws, int64_t rows, int64_t ntiles, hipStream_t stream) {
+    const size_t nwords = split_bytes(rows, ntiles) / sizeof(uint32_t);
+    const unsigned blocks = (unsigned)((nwords + 255) / 256);
+    return launch(split_reset_kernel, blocks, 256u, stream, static_cast<uint32_t*>(ws.ptr), nwords,
+                  split_wait_limit());
+}
+
+// Number of workgroups of `kernel` (of `threads` threads, no dynamic LDS) the
+// current device holds at one time.  Queried once per kernel and device.
+template <class K>
+unsigned resident_workgroups(K kernel, int threads) {
+    int device = 0;
+    if (hipGetDevice(&device) != hipSuccess) return 0;
+    constexpr int kMaxDevices = 64;
+    static std::atomic<unsigned> cache[kMaxDevices];  // 0 = not queried yet; one array per kernel instantiation
+    if (device < 0 || device >= kMaxDevices) return 0;
+    unsigned known = cache[device].load(std::memory_order_relaxed);
+    if (known == 0) {
+        int per_cu = 0, cus = 0;
+        if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, kernel, threads, 0) != hipSuccess ||
+            hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, device) != hipSuccess ||
+            per_cu <= 0 || cus <= 0) {
+            return 0;
+        }
+        known = (unsigned)per_cu * (unsigned)cus;
+        cache[device].store(known, std::memory_order_relaxed);
+    }
+    return known;
+}
+
+// Tiles per row as the kernels count them (tiles_per_row on the device).
+template <class Tr>
+int64_t host_tiles_per_row(int64_t T, int64_t tile, bool regular, const Lead& at) {
+    const int head = regular ? 0 : (T % at.grid == 0 ? at.lead : at.grid - 1);
+    return (T + head + tile - 1) / tile;
+}
+
+// Packed-row policy.  Rows shorter than kPackedMaxRowBytes (of states) are
+// scanned in groups, one group per 4-wave workgroup; a group fills one tile of
+// the general kernel, counting the lead of its first element, and when possible
+// is a whole number of 128-byte lines long so that every group starts on the
+// grid like the first.  ASCAN_PACKED_MAX_ROW_BYTES overrides the limit (0
+// switches packing off), read once.
+constexpr int kPackedWaves = 4;
+constexpr int64_t kPackedMaxRowBytesDefault = 2048;
+
+int64_t packed_max_row_bytes() {
+    static const int64_t v = [] {
+        const char* s = getenv("ASCAN_PACKED_MAX_ROW_BYTES");
+        return s ? (int64_t)atoll(s) : kPackedMaxRowBytesDefault;
+    }();
+    return v;
+}
+
+int64_t gcd64(int64_t a, int64_t b) {
+    while (b != 0) {
+        const int64_t t = a % b;
+        a = b;
+        b = t;
+    }
+    return a;
+}
+
+// Rows per group for rows of T elements, tiles of `tile` elements and a grid of
+// `grid` elements; 0 when rows of this length are not packed.
+int packed_group(int64_t rows, int64_t T, int64_t element_bytes, int64_t tile, int grid) {
+    if (rows < 2 || T * element_bytes >= packed_max_row_bytes()) return 0;
+    int64_t group = (tile - grid) / T;
+    if (group < 2) return 0;
+    const int64_t whole_lines = grid / gcd64(T, grid);  // rows per whole number of grid cells
+    if (group >= whole_lines) group -= group % whole_lines;
+    return (int)group;
+}
+
+// Memory-access flavour of a launch.
+//   kRegular    : every row starts on a grid boundary and is a whole number
+//                 of tiles long, so every sub-tile is full: the kernel carries
+//                 no masking code at all (the common case: T a power of two).
+//   kVector     : all tensors share one offset from the grid; rows may start
+//                 anywhere and have any length.  Whole-vector accesses except
+//                 where a vector straddles a row end.
+//   kElementwise: tensors at different offsets inside a 16-byte vector.
+enum class Access { kRegular, kVector, kElementwise };
+
+Access choose_access(bool same_lead, int lead, int64_t T, int64_t tile) {
+    if (!same_lead) return Access::kElementwise;
+    if (lead == 0 && T % tile == 0) return Access::kRegular;
+    return Access::kVector;
+}
+
+// Kernels with the sigmoid gate exist for the real dtypes, forward in time.
+template <class Tr>
+constexpr bool kHasSigmoid = std::is_same<typename Tr::V, float>::value;
+
+}  // namespace
+}  // namespace ascan
+
+#endif  // ASCAN_POLICY_H_

@@ -21,7 +21,7 @@ HERE = Path(__file__).resolve().parent
 
 class BuildWithLibrary(build_py):
     def run(self):
-        subprocess.run(["make", "-C", str(HERE)], check=True)
+        subprocess.run(["make", "-j8", "-C", str(HERE)], check=True)
         header_dir = HERE / "accelerated_scan" / "include"
         header_dir.mkdir(exist_ok=True)
         shutil.copy2(HERE.parent / "include" / "ascan.h", header_dir / "ascan.h")

@@ -49,6 +49,9 @@ extern "C" {
 
 #define ASCAN_ABI_VERSION 4
 
+/* Marks the exported entry points (the library is built with hidden visibility). */
+#define ASCAN_API __attribute__((visibility("default")))
+
 /* Element types of the tensors of a call. */
 enum ascan_dtype {
     ASCAN_F32  = 0, /* float                                   (warp.cuh:388) */
@@ -89,7 +92,7 @@ enum ascan_gate {
  * reverse != 0 runs the recurrence from t = seqlen-1 down to 0 with the
  * un-shifted gates (the `reverse` argument of warp.cuh:395).
  */
-int ascan_forward(const void* gates, const void* tokens, void* out,
+ASCAN_API int ascan_forward(const void* gates, const void* tokens, void* out,
                   int64_t rows, int64_t seqlen, int dtype, int reverse,
                   void* stream);
 
@@ -100,7 +103,7 @@ int ascan_forward(const void* gates, const void* tokens, void* out,
  * gradient; d_gates and d_tokens receive the two gradients.  One fused
  * reverse-time pass: 3 tensors read, 2 written.
  */
-int ascan_backward(const void* gates, const void* states, const void* grad_out,
+ASCAN_API int ascan_backward(const void* gates, const void* states, const void* grad_out,
                    void* d_gates, void* d_tokens,
                    int64_t rows, int64_t seqlen, int dtype,
                    void* stream);
@@ -135,18 +138,18 @@ int ascan_backward(const void* gates, const void* states, const void* grad_out,
  * completed and pass them to ascan_workspace_timeouts (0 = all waits were
  * served).
  */
-size_t ascan_workspace_bytes(int64_t rows, int64_t seqlen, int dtype);
+ASCAN_API size_t ascan_workspace_bytes(int64_t rows, int64_t seqlen, int dtype);
 
-int ascan_forward_split(const void* gates, const void* tokens, void* out,
+ASCAN_API int ascan_forward_split(const void* gates, const void* tokens, void* out,
                         int64_t rows, int64_t seqlen, int dtype, int reverse,
                         void* workspace, size_t workspace_bytes, void* stream);
 
-int ascan_backward_split(const void* gates, const void* states, const void* grad_out,
+ASCAN_API int ascan_backward_split(const void* gates, const void* states, const void* grad_out,
                          void* d_gates, void* d_tokens,
                          int64_t rows, int64_t seqlen, int dtype,
                          void* workspace, size_t workspace_bytes, void* stream);
 
-unsigned int ascan_workspace_timeouts(const void* workspace_header_copy);
+ASCAN_API unsigned int ascan_workspace_timeouts(const void* workspace_header_copy);
 
 /*
  * Scans that start from a given state, for callers that process a long
@@ -168,11 +171,11 @@ unsigned int ascan_workspace_timeouts(const void* workspace_header_copy);
  *
  * With initial == NULL and d_initial == NULL these calls are the *_split ones.
  */
-int ascan_forward_from(const void* gates, const void* tokens, const void* initial, void* out,
+ASCAN_API int ascan_forward_from(const void* gates, const void* tokens, const void* initial, void* out,
                        int64_t rows, int64_t seqlen, int dtype, int reverse,
                        void* workspace, size_t workspace_bytes, void* stream);
 
-int ascan_backward_from(const void* gates, const void* states, const void* initial,
+ASCAN_API int ascan_backward_from(const void* gates, const void* states, const void* initial,
                         const void* grad_out, void* d_gates, void* d_tokens, void* d_initial,
                         int64_t rows, int64_t seqlen, int dtype,
                         void* workspace, size_t workspace_bytes, void* stream);
@@ -195,23 +198,23 @@ int ascan_backward_from(const void* gates, const void* states, const void* initi
  * ASCAN_ERR_BAD_ACTIVATION.  The sigmoid is evaluated in fp32 with the
  * hardware's exp2 and reciprocal (about 2 ulp).
  */
-int ascan_forward_gated(const void* gate_inputs, const void* tokens, const void* initial, void* out,
+ASCAN_API int ascan_forward_gated(const void* gate_inputs, const void* tokens, const void* initial, void* out,
                         int64_t rows, int64_t seqlen, int dtype, int gate,
                         void* workspace, size_t workspace_bytes, void* stream);
 
-int ascan_backward_gated(const void* gate_inputs, const void* states, const void* initial,
+ASCAN_API int ascan_backward_gated(const void* gate_inputs, const void* states, const void* initial,
                          const void* grad_out, void* d_gate_inputs, void* d_tokens, void* d_initial,
                          int64_t rows, int64_t seqlen, int dtype, int gate,
                          void* workspace, size_t workspace_bytes, void* stream);
 
 /* Static, human-readable text for an ascan_status code. */
-const char* ascan_status_string(int status);
+ASCAN_API const char* ascan_status_string(int status);
 
 /* hipError_t (as int) recorded by the calling thread's last ASCAN_ERR_LAUNCH. */
-int ascan_last_hip_error(void);
+ASCAN_API int ascan_last_hip_error(void);
 
 /* ASCAN_ABI_VERSION the library was built with. */
-int ascan_abi_version(void);
+ASCAN_API int ascan_abi_version(void);
 
 #ifdef __cplusplus
 }
