@@ -141,7 +141,7 @@ int ascan_backward(const void* gates, const void* states, const void* grad_out, 
 size_t ascan_workspace_bytes(int64_t rows, int64_t seqlen, int dtype) {
     const size_t es = element_size(dtype);
     if (es == 0 || rows <= 0 || seqlen <= 0) return 0;
-    // the smallest split tile any kernel uses for this dtype: 4 waves x 2 blocks x 64 vectors
+    // the smallest split tile any kernel uses for this dtype: 2 blocks of 64 vectors per wave
     const int64_t epv = 16 / (int64_t)es;
     const int64_t tile = (int64_t)kSplitWaves * 2 * 64 * epv;
     // rows are addressed from the 128-byte boundary below their first element at most

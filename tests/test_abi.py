@@ -80,7 +80,7 @@ def test_workspace_sizing_and_split_entry_validation():
     # few long rows: header (64 bytes) + one 64-byte ticket line per row
     # + one 64-byte record per (row, smallest tile)
     nbytes = lib.ascan_workspace_bytes(4, 1 << 20, 0)
-    assert nbytes == 64 + 4 * 64 + 4 * ((1 << 20) // 2048 + 1) * 64
+    assert nbytes == 64 + 4 * 64 + 4 * ((1 << 20) // 8192 + 1) * 64
     assert lib.ascan_workspace_bytes(4, 1 << 20, 1) < nbytes  # 16-bit tiles hold more elements
     # the split entry points validate like the plain ones, before touching the GPU
     assert lib.ascan_forward_split(p, p, p, 1, 4, 7, 0, None, 0, None) == 3

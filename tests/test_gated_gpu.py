@@ -112,7 +112,7 @@ def test_unaligned_base_pointer(dtype, offsets, rows, T):
 
 
 @pytest.mark.parametrize("dtype", DTYPES, ids=IDS)
-@pytest.mark.parametrize("rows,T", [(1, 1 << 20), (3, 300000), (64, 65536), (128, 32768 + 8), (5, 99999)])
+@pytest.mark.parametrize("rows,T", [(1, 1 << 20), (3, 300000), (64, 65536), (128, 65536 + 8), (5, 99999)])
 def test_split_rows(dtype, rows, T):
     from accelerated_scan import _abi
 

@@ -592,7 +592,7 @@ def test_linearity_and_concatenation():
 # Split rows: few rows, long sequences, several workgroups per row
 # ---------------------------------------------------------------------------
 @pytest.mark.parametrize("dtype", ALL_DTYPES, ids=ALL_IDS)
-@pytest.mark.parametrize("rows,T", [(1, 1 << 20), (3, 300000), (64, 65536), (128, 32768 + 8), (5, 99999), (2, 16384 * 3)])
+@pytest.mark.parametrize("rows,T", [(1, 1 << 20), (3, 300000), (64, 65536), (128, 65536 + 8), (5, 99999), (2, 16384 * 3)])
 def test_split_rows(dtype, rows, T):
     """The table-passing kernels (one workgroup per tile) against the fp64 loops,
     and no wait may have run out."""
