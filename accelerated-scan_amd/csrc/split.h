@@ -19,8 +19,8 @@ namespace {
 //     until it meets a tile whose inclusive state P is already published;
 //   * it publishes its own inclusive state and finishes the tile.
 // Tiles are handed out by ticket: every row has a counter, and a workgroup
-// takes the next tile of a row with one fetch-add on it (moving on to the next
-// row when a row has no tiles left).  A tile is therefore only ever waited for
+// takes the next tile of the row it serves with one fetch-add on it.  A tile
+// is therefore only ever waited for
 // by workgroups that started after its owner did: progress never depends on a
 // workgroup that has not been dispatched yet, whatever else is running on the
 // GPU, and the launch size (what an idle GPU holds at once) is a matter of
@@ -134,39 +134,25 @@ __device__ __forceinline__ unsigned long long from_lane0(unsigned long long v) {
            (unsigned)__builtin_amdgcn_readfirstlane((int)v);
 }
 
-// Hands the workgroup its next tile: the next tile of the row it is on if that
-// row has one left, else of the next row (cyclically) that does.  Returns false
-// when no row has tiles left.  All threads of the workgroup call it together
-// and get the same answer; `mailbox` is two words of LDS.
+// Hands the workgroup its next tile.  Workgroup b serves row b % rows -- with
+// fewer rows than workgroups several workgroups share a row and draw its tiles
+// in turn -- and, when that row has no tiles left, the rows b + G, b + 2G, ...
+// (G = workgroups in the launch), so every row is served whatever G is.
+// (Letting idle workgroups look for tiles in other rows was tried: near the end
+// hundreds of them draw from the few counters that still have tiles, and the
+// owners' own draws queue behind them.)  Returns false when the workgroup has
+// nothing left to do.  All threads of the workgroup call it together and get
+// the same answer; `mailbox` is two words of LDS.
 __device__ __forceinline__ bool take_split_tile(SplitHeader* header, int64_t rows, int64_t ntiles, SplitWalk& walk,
                                                 int64_t& row, int64_t& k, long long* mailbox) {
     if (threadIdx.x < 64) {  // wave 0
         const int lane = threadIdx.x;
         SplitTicket* tickets = split_tickets(header);
         long long got_row = -1, got_k = -1;
-        for (;;) {
-            unsigned long long ticket;
-            if (walk.has_drawn) {
-                ticket = from_lane0(walk.drawn);
-                walk.has_drawn = false;
-            } else {
-                // first row at or after walk.row, cyclically, that still has tiles: 64 rows per look
-                long long found = -1;
-                for (int64_t base = 0; base < rows && found < 0; base += 64) {
-                    const int64_t idx = base + lane;
-                    bool has = false;
-                    if (idx < rows) {
-                        const int64_t r = walk.row + idx < rows ? walk.row + idx : walk.row + idx - rows;
-                        has = __hip_atomic_load(&tickets[r].next, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) <
-                              (unsigned long long)ntiles;
-                    }
-                    const unsigned long long mask = __ballot(has);
-                    if (mask) found = base + (long long)__builtin_ctzll(mask);
-                }
-                if (found < 0) break;  // nothing left anywhere
-                walk.row = walk.row + found < rows ? walk.row + found : walk.row + found - rows;
-                ticket = from_lane0(draw_ticket(&tickets[walk.row], lane));
-            }
+        while (walk.row < rows) {
+            const unsigned long long ticket =
+                from_lane0(walk.has_drawn ? walk.drawn : draw_ticket(&tickets[walk.row], lane));
+            walk.has_drawn = false;
             if (ticket < (unsigned long long)ntiles) {
                 got_row = walk.row;
                 got_k = (long long)ticket;
@@ -176,7 +162,7 @@ __device__ __forceinline__ bool take_split_tile(SplitHeader* header, int64_t row
                 }
                 break;
             }
-            // the row ran out (another workgroup took its last tile): look again
+            walk.row += gridDim.x;  // this row is handed out completely
         }
         if (lane == 0) {
             mailbox[0] = got_row;
