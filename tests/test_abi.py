@@ -36,8 +36,8 @@ def test_library_exports_every_declared_symbol():
 def test_abi_version_and_status_strings():
     lib = _abi.load()
     assert lib.ascan_abi_version() == _abi.ABI_VERSION
-    texts = {lib.ascan_status_string(i).decode() for i in range(6)}
-    assert len(texts) == 6 and "ok" in texts
+    texts = {lib.ascan_status_string(i).decode() for i in range(7)}
+    assert len(texts) == 7 and "ok" in texts
     assert lib.ascan_status_string(99).decode() == "unknown status"
 
 
@@ -48,6 +48,10 @@ def test_argument_validation_returns_codes():
     # unknown dtype
     assert lib.ascan_forward(p, p, p, 1, 4, 7, 0, None) == 3
     assert lib.ascan_backward(p, p, p, p, p, 1, 4, -1, None) == 3
+    # unknown gate activation, or one the dtype does not have
+    assert lib.ascan_forward_gated(p, p, None, p, 1, 4, 0, 5, None, 0, None) == 6
+    assert lib.ascan_forward_gated(p, p, None, p, 1, 4, 3, 1, None, 0, None) == 6
+    assert lib.ascan_backward_gated(p, p, None, p, p, p, None, 1, 4, 4, 1, None, 0, None) == 6
     # negative sizes, too many rows
     assert lib.ascan_forward(p, p, p, -1, 4, 0, 0, None) == 2
     assert lib.ascan_forward(p, p, p, 1, -4, 0, 0, None) == 2
