@@ -150,6 +150,29 @@ def test_split_rows(dtype, rows, T):
     _run_and_compare(rows, T, dtype, seed=rows, what="split")
 
 
+def _random_cases(n, seed, n_dtypes):
+    """Seeded random (dtype, rows, T, offsets): short rows in groups, rows of every
+    tile count, few long rows; equal offsets for all tensors in 7 of 10 cases."""
+    rng = np.random.RandomState(seed)
+    cases = []
+    for i in range(n):
+        dtype_index = int(rng.randint(n_dtypes))
+        rows = int(np.exp(rng.uniform(0, np.log(3000)))) if rng.rand() < 0.7 else int(rng.randint(1, 9))
+        max_T = max(2, min(200000, 6_000_000 // rows))
+        T = int(np.exp(rng.uniform(0, np.log(max_T))))
+        k = int(rng.randint(0, 4))
+        offsets = (k, k, k) if rng.rand() < 0.7 else tuple(int(v) for v in rng.randint(0, 4, size=3))
+        cases.append((i, dtype_index, rows, T, offsets))
+    return cases
+
+
+@pytest.mark.parametrize("case", _random_cases(60, seed=20240611, n_dtypes=len(ALL_DTYPES)),
+                         ids=lambda c: f"{c[0]}-{ALL_IDS[c[1]]}-{c[2]}x{c[3]}")
+def test_random_shapes_and_offsets(case):
+    _, dtype_index, rows, T, offsets = case
+    _run_and_compare(rows, T, ALL_DTYPES[dtype_index], seed=rows * 7919 + T, what=f"random case {case}", offsets=offsets)
+
+
 def test_null_initial_and_null_gradient_through_the_c_abi():
     """ascan_*_from with initial == NULL is the zero-start scan; d_initial == NULL is allowed."""
     from accelerated_scan import _abi
