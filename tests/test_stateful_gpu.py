@@ -97,10 +97,10 @@ def _run_and_compare(rows, T, dtype, seed, what, offsets=(0, 0, 0)):
     og, ox, oo = offsets
     shape = (1, rows, T)
     g, x, d = _offset_copy(gates, shape, og), _offset_copy(tokens, shape, ox), _offset_copy(grad_out, shape, oo)
-    init = initial.to(DEVICE).reshape(1, rows)
+    init = _offset_copy(initial, (1, rows), 1)  # one state per row; only element alignment is required
     out, rev = _offset_copy(torch.zeros_like(gates), shape, oo), _offset_copy(torch.zeros_like(gates), shape, og)
     dg, dx = _offset_copy(torch.zeros_like(gates), shape, ox), _offset_copy(torch.zeros_like(tokens), shape, oo)
-    di = torch.full_like(init, float("nan"))
+    di = _offset_copy(torch.full_like(initial, float("nan")), (1, rows), 3)
     _abi.forward(g, x, out, False, initial=init)
     _abi.forward(g, x, rev, True, initial=init)
     _abi.backward(g, out, d, dg, dx, initial=init, d_initial=di)
