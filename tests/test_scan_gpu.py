@@ -766,7 +766,7 @@ def test_random_shapes_and_offsets(case):
 # ---------------------------------------------------------------------------
 # HIP graph capture: the entry points allocate nothing and use no memset
 # ---------------------------------------------------------------------------
-@pytest.mark.parametrize("rows,T", [(300, 20000), (4, 1 << 19)], ids=["plain", "split"])
+@pytest.mark.parametrize("rows,T", [(300, 20000), (4, 1 << 19), (50000, 24)], ids=["plain", "split", "packed"])
 def test_graph_capture_and_replay(rows, T):
     """Forward + backward captured once into a graph, replayed with new inputs;
     every replay is compared with the eager result of the same inputs."""
