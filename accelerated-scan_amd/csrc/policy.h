@@ -60,11 +60,35 @@ const Plan& forced_plan() {
 // gets as many waves as it has sub-tiles (up to 16).  Short rows keep small
 // workgroups (256 threads, several rows each): packing more short rows into
 // one large workgroup measured slower.
-Plan choose_plan(int64_t T, int64_t sub, int64_t element_bytes) {
+//
+// `trim`: a row is scanned in whole tiles of w sub-tiles, and when its last
+// tile would be mostly empty fewer waves per row leave fewer wave slots idle
+// (20000 bf16 elements in tiles of 16384: the second tile is a fifth full).  The
+// kernels for 16-bit storage, which run one large workgroup per compute unit,
+// gain from a narrower plan when more than 30 % of the slots would idle (bf16
+// backward at T = 20000: 0.65 -> 0.46 ms; below that waste they lose ~5 %); the
+// fp32 and complex kernels, which have other workgroups to fill the gaps, lose
+// up to 10 % and keep w.
+Plan choose_plan(int64_t T, int64_t sub, int64_t element_bytes, bool trim) {
     const Plan& forced = forced_plan();
     // one wave per 4 KiB of row, but never more waves than sub-tiles
     int w = 1;
     while (w < kMaxWavesPerBlock && (int64_t)w * 4096 < T * element_bytes && (int64_t)w * sub < T) w *= 2;
+    if (trim) {
+        // wave slots (of `sub` elements each) a row occupies over all its tile steps
+        auto slots = [&](int waves) { return (T + (int64_t)waves * sub - 1) / ((int64_t)waves * sub) * waves; };
+        if (slots(w) * sub * 10 > T * 13) {
+            int best = w;
+            for (int v = w / 2; v >= 1; v /= 2) {
+                if (slots(v) * sub * 100 <= T * 115) {  // the widest plan that wastes at most 15 %
+                    best = v;
+                    break;
+                }
+                if (slots(v) < slots(best)) best = v;
+            }
+            w = best;
+        }
+    }
     if (forced.waves_per_row) w = forced.waves_per_row;
     int r = w >= 4 ? 1 : 4 / w;
     if (forced.rows_per_block) r = forced.rows_per_block;
