@@ -67,9 +67,9 @@ int backward_typed(const void* gates, const void* states, const void* grad_out, 
     const Lead at = find_lead<Tr>(state_like, d_tokens);
     const bool same_lead = at.same;
     const int lead = at.lead;
-    Plan plan = choose_plan(T, SUB, kElem, Tr::kNarrow);
+    Plan plan = choose_plan(T, SUB, kElem, kTrimPlan<Tr>);
     const Access access = choose_access(same_lead, lead, T, SUB * plan.waves_per_row);
-    if (access != Access::kRegular) plan = choose_plan(T, SUBG, kElem, Tr::kNarrow);
+    if (access != Access::kRegular) plan = choose_plan(T, SUBG, kElem, kTrimPlan<Tr>);
     const int R = plan.rows_per_block;
     hipError_t err = hipSuccess;
     if (const int group = packed_group(rows, T, kElem, SUBG * kPackedWaves, same_lead ? at.grid : 1)) {

@@ -56,13 +56,13 @@ int forward_typed(const void* gates, const void* tokens, void* out, const void* 
     constexpr int64_t kElem = (int64_t)sizeof(typename Tr::S);
     constexpr int64_t SUB = (int64_t)Tuning<Tr>::U * 64 * Tr::EPV;    // regular kernels
     constexpr int64_t SUBG = (int64_t)Tuning<Tr>::UG * 64 * Tr::EPV;  // kernels with masking code
-    Plan plan = choose_plan(T, SUB, kElem, Tr::kNarrow);
+    Plan plan = choose_plan(T, SUB, kElem, kTrimPlan<Tr>);
     const void* const state_like[] = {gates, out};
     const Lead at = find_lead<Tr>(state_like, tokens);
     const bool same_lead = at.same;
     const int lead = at.lead;
     const Access access = choose_access(same_lead, lead, T, SUB * plan.waves_per_row);
-    if (access != Access::kRegular) plan = choose_plan(T, SUBG, kElem, Tr::kNarrow);
+    if (access != Access::kRegular) plan = choose_plan(T, SUBG, kElem, kTrimPlan<Tr>);
     const int R = plan.rows_per_block;
     hipError_t err = hipSuccess;
     if (const int group = packed_group(rows, T, kElem, SUBG * kPackedWaves, same_lead ? at.grid : 1)) {

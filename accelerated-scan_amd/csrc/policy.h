@@ -64,11 +64,13 @@ const Plan& forced_plan() {
 // `trim`: a row is scanned in whole tiles of w sub-tiles, and when its last
 // tile would be mostly empty fewer waves per row leave fewer wave slots idle
 // (20000 bf16 elements in tiles of 16384: the second tile is a fifth full).  The
-// kernels for 16-bit storage, which run one large workgroup per compute unit,
-// gain from a narrower plan when more than 30 % of the slots would idle (bf16
-// backward at T = 20000: 0.65 -> 0.46 ms; below that waste they lose ~5 %); the
-// fp32 and complex kernels, which have other workgroups to fill the gaps, lose
-// up to 10 % and keep w.
+// 16-bit and the complex kernels gain from a narrower plan when more than 30 %
+// of the slots would idle (bf16 backward at T = 20000: 0.65 -> 0.46 ms,
+// complex64 forward at T = 4500: 0.152 -> 0.121 ms; below that waste they lose
+// ~5 %); the fp32 kernels lose up to 10 % at every waste and keep w.
+template <class Tr>
+constexpr bool kTrimPlan = Tr::kNarrow || !std::is_same<typename Tr::V, float>::value;
+
 Plan choose_plan(int64_t T, int64_t sub, int64_t element_bytes, bool trim) {
     const Plan& forced = forced_plan();
     // one wave per 4 KiB of row, but never more waves than sub-tiles
