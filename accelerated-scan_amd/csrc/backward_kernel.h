@@ -198,10 +198,10 @@ __global__ void __launch_bounds__(64 * kMaxWavesPerBlock)
 #pragma unroll
             for (int e = EPV - 2; e >= 0; --e) {
                 const V ga = vconj(after[e]);
-                X = vfma(ga, X, d[e]);
-                A = vmul(A, ga);
+                X = carry_in<PACKED>(ga, X, d[e]);
+                A = gate_product<PACKED>(A, ga);
             }
-            wave_scan_inclusive(A, X);
+            wave_scan_inclusive<PACKED>(A, X);
             totA[j] = read_lane<63>(A);
             totX[j] = read_lane<63>(X);
             exA[j] = shift_up1(A, vone<V>());
@@ -213,7 +213,7 @@ __global__ void __launch_bounds__(64 * kMaxWavesPerBlock)
             exchange_carries_split<V, W, U>(totA, totX, c, slots, w, lane, split, split_records(split, rows) + row * ntiles, 1, k,
                                             vzero<V>());
         } else {
-            exchange_carries<V, W, U>(totA, totX, carry, c, slots, (int)(k & 1), w, lane);
+            exchange_carries<V, W, U, PACKED>(totA, totX, carry, c, slots, (int)(k & 1), w, lane);
         }
         // Pass 2: the plain reverse recurrence and the gate gradient.
 #pragma unroll
@@ -228,8 +228,8 @@ __global__ void __launch_bounds__(64 * kMaxWavesPerBlock)
             activate<ACT>(a);
             Tr::unpack(draw[j], d);
             Tr::unpack(xraw[j], x);
-            V gr = vfma(exA[j], c, exX[j]);  // g entering this lane's vector from above
-            c = vfma(totA[j], c, totX[j]);
+            V gr = carry_in<PACKED>(exA[j], c, exX[j]);  // g entering this lane's vector from above
+            c = carry_in<PACKED>(totA[j], c, totX[j]);
             const int off = vec_offset<U, EPV, true>(j, lane);
             V after[EPV], before[EPV];
 #pragma unroll
@@ -245,7 +245,7 @@ __global__ void __launch_bounds__(64 * kMaxWavesPerBlock)
             V dt[EPV], dg[EPV];
 #pragma unroll
             for (int e = EPV - 1; e >= 0; --e) {
-                gr = vfma(vconj(after[e]), gr, d[e]);
+                gr = carry_in<PACKED>(vconj(after[e]), gr, d[e]);
                 dt[e] = gr;
                 dg[e] = vmul(gr, vconj(before[e]));
                 if constexpr (ACT != kGateIdentity) dg[e] = vmul(dg[e], gate_slope<ACT>(a[e]));

@@ -37,23 +37,25 @@ __device__ __forceinline__ bool locate_wave(int64_t rows, int64_t ntiles, int64_
 //         carry          state entering the tile (wave-uniform, same in all waves)
 // Output: c              state entering block 0 of this wave
 //         carry          state entering the next tile
+// RESET: a total with a gate product of exactly zero discards the incoming state
+// (see carry_in).
 // With W > 1 the W waves of a row exchange their sub-tile totals through
 // `slots`, the row's W entries of one of two buffers selected by `parity`.
-template <class V, int W, int U>
+template <class V, int W, int U, bool RESET>
 __device__ __forceinline__ void exchange_carries(const V (&totA)[U], const V (&totX)[U], V& carry, V& c,
                                                  V* slots, int parity, int w, int lane) {
     if constexpr (W == 1) {
         c = carry;
         V n = carry;
 #pragma unroll
-        for (int j = 0; j < U; ++j) n = vfma(totA[j], n, totX[j]);
+        for (int j = 0; j < U; ++j) n = carry_in<RESET>(totA[j], n, totX[j]);
         carry = n;
     } else {
         V TA = totA[0], TX = totX[0];
 #pragma unroll
         for (int j = 1; j < U; ++j) {
-            TX = vfma(TX, totA[j], totX[j]);
-            TA = vmul(TA, totA[j]);
+            TX = carry_in<RESET>(totA[j], TX, totX[j]);
+            TA = gate_product<RESET>(TA, totA[j]);
         }
         V* buf = slots + parity * kSlotsPerBuffer;
         if (lane == 0) {
@@ -68,7 +70,7 @@ __device__ __forceinline__ void exchange_carries(const V (&totA)[U], const V (&t
             const V Ai = buf[2 * i];
             const V Xi = buf[2 * i + 1];
             mine = vselect(i == w, run, mine);
-            run = vfma(Ai, run, Xi);
+            run = carry_in<RESET>(Ai, run, Xi);
         }
         c = mine;
         carry = run;

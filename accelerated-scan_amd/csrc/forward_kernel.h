@@ -135,10 +135,10 @@ __global__ void __launch_bounds__(64 * kMaxWavesPerBlock)
 #pragma unroll
             for (int i = 1; i < EPV; ++i) {
                 const int e = REV ? EPV - 1 - i : i;
-                X = vfma(g[e], X, t[e]);
-                A = vmul(A, g[e]);
+                X = carry_in<PACKED>(g[e], X, t[e]);
+                A = gate_product<PACKED>(A, g[e]);
             }
-            wave_scan_inclusive(A, X);
+            wave_scan_inclusive<PACKED>(A, X);
             totA[j] = read_lane<63>(A);
             totX[j] = read_lane<63>(X);
             exA[j] = shift_up1(A, vone<V>());
@@ -150,7 +150,7 @@ __global__ void __launch_bounds__(64 * kMaxWavesPerBlock)
             exchange_carries_split<V, W, U>(totA, totX, c, slots, w, lane, split, split_records(split, rows) + row * ntiles, 1, k,
                                             row_start);
         } else {
-            exchange_carries<V, W, U>(totA, totX, carry, c, slots, (int)(k & 1), w, lane);
+            exchange_carries<V, W, U, PACKED>(totA, totX, carry, c, slots, (int)(k & 1), w, lane);
         }
 
         // Pass 2: the plain recurrence from the state entering each lane.
@@ -165,13 +165,13 @@ __global__ void __launch_bounds__(64 * kMaxWavesPerBlock)
             activate<ACT>(g);
             Tr::unpack(traw[j], t);
             if constexpr (PACKED) cut_rows<Tr, REV>(g, t, (int)(sub_base - lo) + vec_offset<U, EPV, REV>(j, lane), cuts);
-            V x = vfma(exA[j], c, exX[j]);  // state entering this lane's vector
-            c = vfma(totA[j], c, totX[j]);  // state entering the next block
+            V x = carry_in<PACKED>(exA[j], c, exX[j]);  // state entering this lane's vector
+            c = carry_in<PACKED>(totA[j], c, totX[j]);  // state entering the next block
             V o[EPV];
 #pragma unroll
             for (int i = 0; i < EPV; ++i) {
                 const int e = REV ? EPV - 1 - i : i;
-                x = vfma(g[e], x, t[e]);
+                x = carry_in<PACKED>(g[e], x, t[e]);
                 o[e] = x;
             }
             const int off = vec_offset<U, EPV, REV>(j, lane);

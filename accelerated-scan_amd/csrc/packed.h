@@ -14,7 +14,9 @@ namespace {
 // workgroup scans a group of consecutive rows -- one contiguous stretch of
 // memory -- as a single long row with a "cut" in front of every row: at a row's
 // first element the gate is replaced by 0, which annihilates whatever the scan
-// carries in from the row before, and gate * x[-1] is added to the token.  All
+// carries in from the row before (the scan's combine steps treat a gate of
+// exactly zero as a reset, so that even a non-finite state stops at the cut),
+// and gate * x[-1] is added to the token.  All
 // of the tiling, masking and carry code is shared with the one-row-per-
 // workgroup mode; the cuts are applied to the unpacked vectors.
 //   rel  position of an element relative to the first element of the group;

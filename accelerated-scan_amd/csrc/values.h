@@ -81,23 +81,50 @@ __device__ __forceinline__ cfloat dpp_move(cfloat old, cfloat src) {
 }
 
 // One Kogge-Stone step of the pair scan: (Ap, Xp) o (A, X) = (Ap*A, Xp*A + X).
-template <int CTRL, int ROW_MASK, class V>
+// The two halves of the scan operator, (A_l, X_l) o (A_r, X_r) =
+// (A_l * A_r, A_r * X_l + X_r).  With RESET a gate of exactly zero discards
+// what comes from the left even when that is not finite (0 * inf would be NaN):
+// kernels that scan several rows as one, with a zero gate in front of each row,
+// use it so that an overflowing row cannot reach into its neighbour.
+__device__ __forceinline__ bool is_zero(float a) { return a == 0.0f; }
+__device__ __forceinline__ bool is_zero(cfloat a) { return a.re == 0.0f && a.im == 0.0f; }
+
+template <bool RESET, class V>
+__device__ __forceinline__ V carry_in(V gate, V from_left, V local) {
+    const V r = vfma(gate, from_left, local);
+    if constexpr (RESET) {
+        return vselect(is_zero(gate), local, r);
+    } else {
+        return r;
+    }
+}
+template <bool RESET, class V>
+__device__ __forceinline__ V gate_product(V left, V right) {
+    const V r = vmul(left, right);
+    if constexpr (RESET) {
+        return vselect(is_zero(right), right, r);
+    } else {
+        return r;
+    }
+}
+
+template <int CTRL, int ROW_MASK, bool RESET, class V>
 __device__ __forceinline__ void scan_step(V& A, V& X) {
     const V Ap = dpp_move<CTRL, ROW_MASK>(vone<V>(), A);
     const V Xp = dpp_move<CTRL, ROW_MASK>(vzero<V>(), X);
-    X = vfma(Xp, A, X);
-    A = vmul(Ap, A);
+    X = carry_in<RESET>(A, Xp, X);
+    A = gate_product<RESET>(Ap, A);
 }
 
 // Inclusive scan of the 64 (A, X) pairs of a wave, ascending lane order.
-template <class V>
+template <bool RESET, class V>
 __device__ __forceinline__ void wave_scan_inclusive(V& A, V& X) {
-    scan_step<kRowShr1, 0xF>(A, X);
-    scan_step<kRowShr2, 0xF>(A, X);
-    scan_step<kRowShr4, 0xF>(A, X);
-    scan_step<kRowShr8, 0xF>(A, X);
-    scan_step<kRowBcast15, 0xA>(A, X);  // lane 15 of rows 0,2 -> rows 1,3
-    scan_step<kRowBcast31, 0xC>(A, X);  // lane 31 -> rows 2,3
+    scan_step<kRowShr1, 0xF, RESET>(A, X);
+    scan_step<kRowShr2, 0xF, RESET>(A, X);
+    scan_step<kRowShr4, 0xF, RESET>(A, X);
+    scan_step<kRowShr8, 0xF, RESET>(A, X);
+    scan_step<kRowBcast15, 0xA, RESET>(A, X);  // lane 15 of rows 0,2 -> rows 1,3
+    scan_step<kRowBcast31, 0xC, RESET>(A, X);  // lane 31 -> rows 2,3
 }
 
 // Lane l receives v of lane l-1; lane 0 receives `edge`.

@@ -285,6 +285,46 @@ def test_short_rows_in_groups(dtype, rows, T):
     _check_against_truth(gates, tokens, grad_out, dtype, what="short rows")
 
 
+@pytest.mark.parametrize("dtype", ALL_DTYPES, ids=ALL_IDS)
+@pytest.mark.parametrize("rows,T", [(300, 40), (50, 1), (64, 5), (33, 300), (5, 5000)])
+def test_rows_stay_independent_when_one_overflows(dtype, rows, T):
+    """One row whose states and gradients overflow to inf / NaN leaves every
+    other row exactly as it is without that row: also where several rows are
+    scanned as one (short rows), a non-finite state must stop at the row's end."""
+    from accelerated_scan import _abi
+
+    gates, tokens, grad_out = _truth_inputs(rows, T, dtype, seed=rows + T)
+    bad = rows // 2
+    huge = 6.0e4 if dtype == torch.float16 else 1.0e30
+
+    def run(poison):
+        g, x, d = gates.clone(), tokens.clone(), grad_out.clone()
+        if poison:
+            g[bad] = huge
+            x[bad] = huge
+            d[bad] = huge
+        g, x, d = (t.to(DEVICE).reshape(1, rows, T) for t in (g, x, d))
+        out, rev, dg = torch.empty_like(g), torch.empty_like(g), torch.empty_like(g)
+        dx = torch.empty_like(x)
+        _abi.forward(g, x, out, False)
+        _abi.forward(g, x, rev, True)
+        _abi.backward(g, out, d, dg, dx)
+        torch.cuda.synchronize()
+        return out, rev, dg, dx
+
+    clean = run(False)
+    dirty = run(True)
+    keep = torch.ones(rows, dtype=torch.bool)
+    keep[bad] = False
+    if T > 1:  # the poisoned row did overflow
+        assert not torch.isfinite(torch.view_as_real(dirty[0][0, bad]) if dirty[0].is_complex() else dirty[0][0, bad]).all()
+    for name, a, b in zip(("out", "reverse", "d_gates", "d_tokens"), clean, dirty):
+        a, b = a[0].cpu()[keep], b[0].cpu()[keep]
+        if a.is_complex():
+            a, b = torch.view_as_real(a), torch.view_as_real(b)
+        assert torch.equal(a, b), name
+
+
 # ---------------------------------------------------------------------------
 # The five benchmark configurations (shapes and dtypes the reference is quoted on)
 # ---------------------------------------------------------------------------
