@@ -325,6 +325,78 @@ def test_rows_stay_independent_when_one_overflows(dtype, rows, T):
         assert torch.equal(a, b), name
 
 
+def _check_rows_against_truth(g, x, d, out, dg, dx, row_ids, dtype, what):
+    """Selected rows of (1, rows, T) device tensors against the fp64 loops."""
+    tol = _tolerance(dtype)
+    for r in row_ids:
+        gr, xr, dr = (t[0, r].cpu().unsqueeze(0) for t in (g, x, d))
+        t_out = seqscan.forward(_np32(gr), _np32(xr))
+        t_dg, t_dx = seqscan.backward(_np32(gr), _np32(out[0, r].cpu().unsqueeze(0)), _np32(dr))
+        for name, got, want in (("out", out, t_out), ("d_tokens", dx, t_dx), ("d_gates", dg, t_dg)):
+            got = _np32(got[0, r].cpu().unsqueeze(0))
+            scale = max(1.0, float(np.abs(want).max()))
+            np.testing.assert_allclose(got, want, rtol=tol["rtol"], atol=tol["atol"] * scale,
+                                       err_msg=f"{what} {name} row {r}")
+
+
+@pytest.mark.parametrize("rows,T,dtype", [(40000, 60000, torch.bfloat16), (36_000_000, 64, torch.bfloat16)],
+                         ids=["long-rows", "packed-rows"])
+def test_more_than_2_to_31_elements_many_rows(rows, T, dtype):
+    """rows * T exceeds 2^31: element offsets are 64-bit everywhere.  Rows at the
+    start, in the middle and at the very end (element offsets beyond 2^31) against
+    the fp64 loops."""
+    from accelerated_scan import _abi
+
+    assert rows * T > 2**31
+    gen = torch.Generator(device=DEVICE).manual_seed(1)
+    g = torch.rand(1, rows, T, device=DEVICE, generator=gen).to(dtype)
+    x = torch.randn(1, rows, T, device=DEVICE, generator=gen).to(dtype)
+    out = torch.empty_like(g)
+    _abi.forward(g, x, out, False)
+    d = torch.randn(1, rows, T, device=DEVICE, generator=gen).to(dtype)
+    dg, dx = torch.empty_like(g), torch.empty_like(g)
+    _abi.backward(g, out, d, dg, dx)
+    torch.cuda.synchronize()
+    picks = [0, 1, rows // 2, (2**31) // T, (2**31) // T + 1, rows - 2, rows - 1]
+    _check_rows_against_truth(g, x, d, out, dg, dx, picks, dtype, "beyond 2^31")
+
+
+def test_more_than_2_to_31_elements_split_rows():
+    """Three rows of 2^30 fp32 elements each (4 GiB per row), split over the
+    GPU.  Zero gates planted near the ends of the last row make its tail (forward) and its
+    head (backward) independent of the rest, so both can be checked against the
+    fp64 loops on short segments."""
+    from accelerated_scan import _abi
+
+    rows, T, seg = 3, 1 << 30, 5000
+    assert _abi.load().ascan_workspace_bytes(rows, T, 0) > 0
+    gen = torch.Generator(device=DEVICE).manual_seed(2)
+    g = torch.rand(1, rows, T, device=DEVICE, generator=gen)
+    x = torch.randn(1, rows, T, device=DEVICE, generator=gen)
+    g[0, :, T - seg] = 0.0  # the state restarts here
+    g[0, :, seg] = 0.0      # the adjoint of elements [0, seg) does not see what follows
+    out = torch.empty_like(g)
+    _abi.forward(g, x, out, False)
+    torch.cuda.synchronize()
+    r = rows - 1
+    tail = seqscan.forward(g[0, r, T - seg:].cpu().numpy()[None], x[0, r, T - seg:].cpu().numpy()[None])
+    np.testing.assert_allclose(out[0, r, T - seg:].cpu().numpy()[None], tail, rtol=2e-5, atol=2e-5 * np.abs(tail).max())
+    d = torch.randn(1, rows, T, device=DEVICE, generator=gen)
+    del x
+    dg, dx = torch.empty_like(g), torch.empty_like(g)
+    _abi.backward(g, out, d, dg, dx)
+    torch.cuda.synchronize()
+    gh, oh, dh = (t[0, r, :seg].cpu().numpy()[None] for t in (g, out, d))
+    t_dg, t_dx = seqscan.backward(gh, oh, dh)
+    np.testing.assert_allclose(dx[0, r, :seg].cpu().numpy()[None], t_dx, rtol=2e-5, atol=2e-5 * np.abs(t_dx).max())
+    np.testing.assert_allclose(dg[0, r, :seg].cpu().numpy()[None], t_dg, rtol=2e-5, atol=2e-5 * np.abs(t_dg).max())
+    # and the very last elements of the backward pass (nothing follows them)
+    gt, ot, dt = (t[0, r, T - seg:].cpu().numpy()[None] for t in (g, out, d))
+    t_dg, t_dx = seqscan.backward(gt, ot, dt)
+    np.testing.assert_allclose(dx[0, r, T - seg:].cpu().numpy()[None], t_dx, rtol=2e-5, atol=2e-5 * np.abs(t_dx).max())
+    np.testing.assert_allclose(dg[0, r, T - seg + 1:].cpu().numpy()[None], t_dg[:, 1:], rtol=2e-5, atol=2e-5 * np.abs(t_dg).max())
+
+
 # ---------------------------------------------------------------------------
 # The five benchmark configurations (shapes and dtypes the reference is quoted on)
 # ---------------------------------------------------------------------------
