@@ -287,6 +287,10 @@ def main():
         return 2
     from accelerated_scan import _abi
 
+    if not _abi.library_path().exists():  # normally built beforehand; build only when nothing is there
+        import __graft_entry__
+
+        __graft_entry__.build()
     _abi.load()  # no fallback: fail here if the HIP library is missing
 
     shape = tuple(args.shape)
