@@ -29,7 +29,7 @@ hipError_t launch_backward_split(const void* gates, const void* states, const vo
                                  int grid, int64_t ntiles, const Workspace& ws, hipStream_t stream) {
     using S = typename Tr::S;
     using TokS = typename Tr::TokS;
-    constexpr int U = REGULAR ? Tuning<Tr>::UB : Tuning<Tr>::UBG;
+    constexpr int U = REGULAR ? SplitTuning<Tr>::UB : SplitTuning<Tr>::UBG;
     auto kernel = scan_backward_kernel<Tr, kSplitWaves, U, true, REGULAR, true, ACT, false>;
     const unsigned resident = resident_workgroups(kernel, 64 * kSplitWaves);
     if (resident == 0) return hipErrorInvalidConfiguration;
@@ -87,8 +87,10 @@ int backward_typed(const void* gates, const void* states, const void* grad_out, 
         return launch_status(err);
     }
     if (same_lead && ws.ptr != nullptr) {
-        const bool regular = lead == 0 && T % (SUB * kSplitWaves) == 0;
-        const int64_t ntiles = host_tiles_per_row<Tr>(T, (regular ? SUB : SUBG) * kSplitWaves, regular, at);
+        constexpr int64_t SUBS = (int64_t)SplitTuning<Tr>::UB * 64 * Tr::EPV;
+        constexpr int64_t SUBSG = (int64_t)SplitTuning<Tr>::UBG * 64 * Tr::EPV;
+        const bool regular = lead == 0 && T % (SUBS * kSplitWaves) == 0;
+        const int64_t ntiles = host_tiles_per_row<Tr>(T, (regular ? SUBS : SUBSG) * kSplitWaves, regular, at);
         if (want_split(rows, ntiles) && workspace_fits(ws, rows, ntiles)) {
 #define ASCAN_BWD_SPLIT(REG, ACT)                                                                              \
     launch_backward_split<Tr, REG, ACT>(gates, states, grad_out, d_gates, d_tokens, initial, d_initial, rows, T, \

@@ -45,6 +45,8 @@ __global__ void __launch_bounds__(64 * kMaxWavesPerBlock)
     // Split rows: the workgroups take tiles by ticket, row by row, until none
     // is left; a workgroup only ever waits for tiles whose owners started before it.
     __shared__ long long split_mailbox[2];
+    __shared__ u32x4_t parked[SPLIT ? 3 * U * 64 : 1];  // wave 0's raw vectors during its walk back
+    __shared__ V parked_values[SPLIT ? 4 * U * 64 : 1];  // and its per-lane scan results
     SplitWalk walk;  // starts at row blockIdx % rows
     walk.row = SPLIT ? (int64_t)(blockIdx.x % rows) : 0;
     walk.has_drawn = false;
@@ -210,8 +212,32 @@ __global__ void __launch_bounds__(64 * kMaxWavesPerBlock)
 
         V c;
         if constexpr (SPLIT) {
-            exchange_carries_split<V, W, U>(totA, totX, c, slots, w, lane, split, split_records(split, rows) + row * ntiles, 1, k,
-                                            vzero<V>());
+            exchange_carries_split<V, W, U>(
+                totA, totX, c, slots, w, lane, split, split_records(split, rows) + row * ntiles, 1, k, vzero<V>(),
+                [&] {
+#pragma unroll
+                    for (int j = 0; j < U; ++j) {
+                        parked[(3 * j) * 64 + lane] = araw[j];
+                        parked[(3 * j + 1) * 64 + lane] = draw[j];
+                        parked[(3 * j + 2) * 64 + lane] = xraw[j];
+                        parked_values[(4 * j) * 64 + lane] = a_next[j];
+                        parked_values[(4 * j + 1) * 64 + lane] = x_prev[j];
+                        parked_values[(4 * j + 2) * 64 + lane] = exA[j];
+                        parked_values[(4 * j + 3) * 64 + lane] = exX[j];
+                    }
+                },
+                [&] {
+#pragma unroll
+                    for (int j = 0; j < U; ++j) {
+                        araw[j] = parked[(3 * j) * 64 + lane];
+                        draw[j] = parked[(3 * j + 1) * 64 + lane];
+                        xraw[j] = parked[(3 * j + 2) * 64 + lane];
+                        a_next[j] = parked_values[(4 * j) * 64 + lane];
+                        x_prev[j] = parked_values[(4 * j + 1) * 64 + lane];
+                        exA[j] = parked_values[(4 * j + 2) * 64 + lane];
+                        exX[j] = parked_values[(4 * j + 3) * 64 + lane];
+                    }
+                });
         } else {
             exchange_carries<V, W, U, PACKED>(totA, totX, carry, c, slots, (int)(k & 1), w, lane);
         }

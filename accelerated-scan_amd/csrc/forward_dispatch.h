@@ -26,7 +26,7 @@ hipError_t launch_forward_split(const void* gates, const void* tokens, void* out
                                 int64_t T, int grid, int64_t ntiles, const Workspace& ws, hipStream_t stream) {
     using S = typename Tr::S;
     using TokS = typename Tr::TokS;
-    constexpr int U = REGULAR ? Tuning<Tr>::U : Tuning<Tr>::UG;
+    constexpr int U = REGULAR ? SplitTuning<Tr>::U : SplitTuning<Tr>::UG;
     auto kernel = scan_forward_kernel<Tr, kSplitWaves, U, REV, true, REGULAR, true, ACT, false>;
     const unsigned resident = resident_workgroups(kernel, 64 * kSplitWaves);
     if (resident == 0) return hipErrorInvalidConfiguration;
@@ -81,8 +81,10 @@ int forward_typed(const void* gates, const void* tokens, void* out, const void* 
         return launch_status(err);
     }
     if (same_lead && ws.ptr != nullptr) {
-        const bool regular = lead == 0 && T % (SUB * kSplitWaves) == 0;
-        const int64_t ntiles = host_tiles_per_row<Tr>(T, (regular ? SUB : SUBG) * kSplitWaves, regular, at);
+        constexpr int64_t SUBS = (int64_t)SplitTuning<Tr>::U * 64 * Tr::EPV;
+        constexpr int64_t SUBSG = (int64_t)SplitTuning<Tr>::UG * 64 * Tr::EPV;
+        const bool regular = lead == 0 && T % (SUBS * kSplitWaves) == 0;
+        const int64_t ntiles = host_tiles_per_row<Tr>(T, (regular ? SUBS : SUBSG) * kSplitWaves, regular, at);
         if (want_split(rows, ntiles) && workspace_fits(ws, rows, ntiles)) {
 #define ASCAN_FWD_SPLIT(REV, REG, ACT) \
     launch_forward_split<Tr, REV, REG, ACT>(gates, tokens, out, initial, rows, T, at.grid, ntiles, ws, stream)

@@ -45,6 +45,7 @@ __global__ void __launch_bounds__(64 * kMaxWavesPerBlock)
     // Split rows: the workgroups take tiles by ticket, row by row, until none
     // is left; a workgroup only ever waits for tiles whose owners started before it.
     __shared__ long long split_mailbox[2];
+    __shared__ u32x4_t parked[SPLIT ? 2 * U * 64 : 1];  // wave 0's raw vectors during its walk back
     SplitWalk walk;  // starts at row blockIdx % rows
     walk.row = SPLIT ? (int64_t)(blockIdx.x % rows) : 0;
     walk.has_drawn = false;
@@ -147,8 +148,22 @@ __global__ void __launch_bounds__(64 * kMaxWavesPerBlock)
 
         V c;
         if constexpr (SPLIT) {
-            exchange_carries_split<V, W, U>(totA, totX, c, slots, w, lane, split, split_records(split, rows) + row * ntiles, 1, k,
-                                            row_start);
+            exchange_carries_split<V, W, U>(
+                totA, totX, c, slots, w, lane, split, split_records(split, rows) + row * ntiles, 1, k, row_start,
+                [&] {
+#pragma unroll
+                    for (int j = 0; j < U; ++j) {
+                        parked[(2 * j) * 64 + lane] = graw[j];
+                        parked[(2 * j + 1) * 64 + lane] = traw[j];
+                    }
+                },
+                [&] {
+#pragma unroll
+                    for (int j = 0; j < U; ++j) {
+                        graw[j] = parked[(2 * j) * 64 + lane];
+                        traw[j] = parked[(2 * j + 1) * 64 + lane];
+                    }
+                });
         } else {
             exchange_carries<V, W, U, PACKED>(totA, totX, carry, c, slots, (int)(k & 1), w, lane);
         }

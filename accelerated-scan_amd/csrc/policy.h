@@ -32,6 +32,15 @@ template <> struct Tuning<TraitsF16> { static constexpr int U = 4, UG = 2, UB = 
 template <> struct Tuning<TraitsC64> { static constexpr int U = 4, UG = 4, UB = 2, UBG = 2; };
 template <> struct Tuning<TraitsC64RealTokens> : Tuning<TraitsC64> {};
 
+// The same four for split rows (forward regular / general, backward regular /
+// general).  The split kernels also hold the ticket walk and the look-back in
+// registers, so some of them take smaller tiles than their plain counterparts.
+template <class Tr> struct SplitTuning {
+    static constexpr int U = Tuning<Tr>::U, UG = Tuning<Tr>::UG, UB = Tuning<Tr>::UB, UBG = Tuning<Tr>::UBG;
+};
+template <> struct SplitTuning<TraitsC64> { static constexpr int U = 2, UG = 2, UB = 2, UBG = 2; };
+template <> struct SplitTuning<TraitsC64RealTokens> : SplitTuning<TraitsC64> {};
+
 // Launch geometry: W waves per row, R rows per workgroup (W*R <= 16).
 struct Plan {
     int waves_per_row;

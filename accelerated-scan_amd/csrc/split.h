@@ -280,10 +280,17 @@ __device__ __forceinline__ V split_look_back(SplitHeader* header, SplitRecord* m
 
 // exchange_carries for a workgroup that owns a single tile of a split row: the
 // tile carry comes from split_look_back instead of the previous loop iteration.
-template <class V, int W, int U>
+//
+// Wave 0 walks back over the row's earlier tiles while it holds its sub-tile in
+// registers like every other wave, and the walk needs registers of its own.
+// `set_aside()` / `take_back()` are called by wave 0 only, around the walk: the
+// kernels park their raw vectors in LDS there, which frees those registers for
+// the walk without a trip through scratch memory.
+template <class V, int W, int U, class SetAside, class TakeBack>
 __device__ __forceinline__ void exchange_carries_split(const V (&totA)[U], const V (&totX)[U], V& c, V* slots,
                                                        int w, int lane, SplitHeader* header, SplitRecord* mine,
-                                                       int64_t stride, int64_t k, V row_start) {
+                                                       int64_t stride, int64_t k, V row_start, SetAside set_aside,
+                                                       TakeBack take_back) {
     V TA = totA[0], TX = totX[0];
 #pragma unroll
     for (int j = 1; j < U; ++j) {
@@ -309,8 +316,10 @@ __device__ __forceinline__ void exchange_carries_split(const V (&totA)[U], const
     }
     V* carry_slot = slots + kSlotsPerBuffer;
     if (w == 0) {  // wave-uniform
+        set_aside();
         const V carry_in = split_look_back(header, mine, stride, k, runA, runX, row_start, lane);
         if (lane == 0) *carry_slot = carry_in;
+        take_back();
     }
     __syncthreads();
     c = vfma(mineA, *carry_slot, mineX);
