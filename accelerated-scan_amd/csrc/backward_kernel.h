@@ -79,6 +79,9 @@ __global__ void __launch_bounds__(64 * kMaxWavesPerBlock)
     typename Tr::TokS* __restrict__ dtrow = d_tokens + row * T - lo;
 
     V carry = vzero<V>();
+    // the row's index as a scalar (rows < 2^31), for the two per-row addresses
+    // below: kept per lane they would sit in vector registers across the tile loop
+    const int64_t row_scalar = (int64_t)__builtin_amdgcn_readfirstlane((int)row);
 
     // Gradient of x[-1], conj(gate[0]) * g[0], from g at position 0 of the row's
     // first tile.  Positions below the row's first element (position lo) carry
@@ -86,7 +89,7 @@ __global__ void __launch_bounds__(64 * kMaxWavesPerBlock)
     // with lo == 0 the last factor is still missing.
     auto store_start_gradient = [&](V g_low) {
         if (lo == 0) g_low = vmul(vconj(activate1<ACT>(Tr::load1(arow))), g_low);
-        if (lane == 0) Tr::store1(d_initial + row, g_low);
+        if (lane == 0) Tr::store1(d_initial + row_scalar, g_low);
     };
 
     // Position of this wave's sub-tile in tile step k (reverse time).
@@ -97,6 +100,11 @@ __global__ void __launch_bounds__(64 * kMaxWavesPerBlock)
     // One tile step of this wave; FULL as in the forward kernel.
     auto tile_step = [&](int64_t k, auto full_tag) {
         constexpr bool FULL = decltype(full_tag)::value;
+        // The ragged copy (at most two tile steps of a row) works out whatever depends
+        // on the lane on the spot: made opaque here, none of it is computed ahead of
+        // the tile loop and kept in registers (or scratch) through the mask-free copy.
+        int lane = threadIdx.x & 63;
+        if constexpr (!FULL) asm volatile("" : "+v"(lane));
         const int64_t sub_base = sub_tile_base(k);
         const int64_t sub_end = sub_base + SUB;
         const Window win = make_window(lo, hi, sub_base);
@@ -110,7 +118,7 @@ __global__ void __launch_bounds__(64 * kMaxWavesPerBlock)
         // x[-1], the state the forward scan started from (absent = zero), is
         // needed by the sub-tile that holds the row's first element
         V x_start = vzero<V>();
-        if (!PACKED && initial != nullptr && sub_base <= lo && lo < sub_end) x_start = Tr::load1(initial + row);  // wave-uniform
+        if (!PACKED && initial != nullptr && sub_base <= lo && lo < sub_end) x_start = Tr::load1(initial + row_scalar);  // wave-uniform
         Cuts<Tr> cuts;  // packed rows take their initial states at the cuts instead
         if constexpr (PACKED) {
             cuts = stage_row_starts<Tr>(initial != nullptr ? initial + first_row : nullptr, (int)T, (int)len,

@@ -92,6 +92,11 @@ __global__ void __launch_bounds__(64 * kMaxWavesPerBlock)
     // row; it exists only in the kernels for arbitrary row starts and lengths.
     auto tile_step = [&](int64_t k, auto full_tag) {
         constexpr bool FULL = decltype(full_tag)::value;
+        // The ragged copy (at most two tile steps of a row) works out whatever depends
+        // on the lane on the spot: made opaque here, none of it is computed ahead of
+        // the tile loop and kept in registers (or scratch) through the mask-free copy.
+        int lane = threadIdx.x & 63;
+        if constexpr (!FULL) asm volatile("" : "+v"(lane));
         const int64_t sub_base = sub_tile_base(k);
         const Window win = make_window(lo, hi, sub_base);
         const bool touches = FULL || (win.hi > 0 && win.lo < SUB);  // wave-uniform
