@@ -57,7 +57,9 @@ __global__ void __launch_bounds__(64 * kMaxWavesPerBlock)
     if constexpr (SPLIT) {
         if (!take_split_tile(split, rows, ntiles, walk, row, k_begin, split_mailbox)) break;
         k_end = k_begin + 1;
-        w = threadIdx.x >> 6;
+        int thread = threadIdx.x;
+        asm volatile("" : "+v"(thread));  // nothing derived from the wave index is carried from visit to visit
+        w = thread >> 6;
         slot_base = 0;
     } else if (!first_visit) {
         break;
@@ -104,7 +106,7 @@ __global__ void __launch_bounds__(64 * kMaxWavesPerBlock)
         // on the lane on the spot: made opaque here, none of it is computed ahead of
         // the tile loop and kept in registers (or scratch) through the mask-free copy.
         int lane = threadIdx.x & 63;
-        if constexpr (!FULL) asm volatile("" : "+v"(lane));
+        if constexpr (!FULL || SPLIT) asm volatile("" : "+v"(lane));  // split rows: one tile step per visit, same reasoning
         const int64_t sub_base = sub_tile_base(k);
         const int64_t sub_end = sub_base + SUB;
         const Window win = make_window(lo, hi, sub_base);
