@@ -32,7 +32,6 @@ __global__ void __launch_bounds__(64 * kMaxWavesPerBlock)
     constexpr int64_t TILE = SUB * W;
     static_assert(!PACKED || (!SPLIT && !REGULAR), "packed rows use the general kernels, one group per workgroup");
 
-    const int lane = threadIdx.x & 63;
     // Packed rows: this workgroup scans rows [first_row, first_row + nrows) as one row of `len` elements.
     const int64_t first_row = PACKED ? (int64_t)blockIdx.x * group : 0;
     const int64_t len = PACKED ? (rows - first_row < group ? rows - first_row : (int64_t)group) * T : T;
