@@ -42,15 +42,15 @@ hipError_t launch_backward_split(const void* gates, const void* states, const vo
                   static_cast<SplitHeader*>(ws.ptr), static_cast<const S*>(initial), static_cast<S*>(d_initial), grid, 0);
 }
 
-template <class Tr, bool ALIGNED, int ACT>
+template <class Tr, int PW, bool ALIGNED, int ACT>
 hipError_t launch_backward_packed(const void* gates, const void* states, const void* grad_out, void* d_gates,
                                   void* d_tokens, const void* initial, void* d_initial, int64_t rows, int64_t T,
                                   int grid, int group, hipStream_t stream) {
     using S = typename Tr::S;
     using TokS = typename Tr::TokS;
     const unsigned blocks = (unsigned)((rows + group - 1) / group);
-    return launch(scan_backward_kernel<Tr, kPackedWaves, Tuning<Tr>::UBG, ALIGNED, false, false, ACT, true>, blocks,
-                  64u * kPackedWaves, stream, static_cast<const S*>(gates), static_cast<const S*>(states),
+    return launch(scan_backward_kernel<Tr, PW, Tuning<Tr>::UBG, ALIGNED, false, false, ACT, true>, blocks,
+                  64u * PW, stream, static_cast<const S*>(gates), static_cast<const S*>(states),
                   static_cast<const S*>(grad_out), static_cast<S*>(d_gates), static_cast<TokS*>(d_tokens), rows, T,
                   static_cast<SplitHeader*>(nullptr), static_cast<const S*>(initial), static_cast<S*>(d_initial), grid,
                   group);
@@ -72,16 +72,32 @@ int backward_typed(const void* gates, const void* states, const void* grad_out, 
     if (access != Access::kRegular) plan = choose_plan(T, SUBG, kElem, kTrimPlan<Tr>);
     const int R = plan.rows_per_block;
     hipError_t err = hipSuccess;
+#define ASCAN_BWD_PACKED(PW, AL, ACT)                                                                                  \
+    launch_backward_packed<Tr, PW, AL, ACT>(gates, states, grad_out, d_gates, d_tokens, initial, d_initial, rows, T, \
+                                            at.grid, group, stream)
+    // 16-bit rows of 512 bytes and more, vectorised flavour, plenty of them: groups of the wider workgroup
+    if constexpr (Tr::kNarrow) {
+        if (same_lead && T * kElem >= kPackedWideRowBytes) {
+            const int group = packed_group(rows, T, kElem, SUBG * kPackedWavesWide, at.grid);
+            if (group != 0 && rows / group >= kPackedWideMinGroups) {
+                if (act == kGateSigmoid) {
+                    err = ASCAN_BWD_PACKED(kPackedWavesWide, true, kGateSigmoid);
+                } else {
+                    err = ASCAN_BWD_PACKED(kPackedWavesWide, true, kGateIdentity);
+                }
+                return launch_status(err);
+            }
+        }
+    }
     if (const int group = packed_group(rows, T, kElem, SUBG * kPackedWaves, same_lead ? at.grid : 1)) {
-#define ASCAN_BWD_PACKED(AL, ACT)                                                                                  \
-    launch_backward_packed<Tr, AL, ACT>(gates, states, grad_out, d_gates, d_tokens, initial, d_initial, rows, T, \
-                                        at.grid, group, stream)
         if (act == kGateSigmoid) {
             if constexpr (kHasSigmoid<Tr>) {
-                err = same_lead ? ASCAN_BWD_PACKED(true, kGateSigmoid) : ASCAN_BWD_PACKED(false, kGateSigmoid);
+                err = same_lead ? ASCAN_BWD_PACKED(kPackedWaves, true, kGateSigmoid)
+                                : ASCAN_BWD_PACKED(kPackedWaves, false, kGateSigmoid);
             }
         } else {
-            err = same_lead ? ASCAN_BWD_PACKED(true, kGateIdentity) : ASCAN_BWD_PACKED(false, kGateIdentity);
+            err = same_lead ? ASCAN_BWD_PACKED(kPackedWaves, true, kGateIdentity)
+                            : ASCAN_BWD_PACKED(kPackedWaves, false, kGateIdentity);
         }
 #undef ASCAN_BWD_PACKED
         return launch_status(err);

@@ -239,6 +239,14 @@ int64_t host_tiles_per_row(int64_t T, int64_t tile, bool regular, const Lead& at
 // grid like the first.  ASCAN_PACKED_MAX_ROW_BYTES overrides the limit (0
 // switches packing off), read once.
 constexpr int kPackedWaves = 4;
+// The 16-bit backward kernels do better with 8-wave workgroups once rows reach
+// 512 bytes (measured, 4 -> 8 waves: bf16 (64,4096,256) 5.1 -> 5.6 TB/s,
+// (16,4096,1000) 5.4 -> 5.7, (64,4096,500) 5.5 -> 5.8; shorter rows and the
+// forward kernels lose 5-15 %, fp32 and complex64 gain or lose a few per cent
+// depending on the row length).
+constexpr int kPackedWavesWide = 8;
+constexpr int64_t kPackedWideRowBytes = 512;
+constexpr int64_t kPackedWideMinGroups = 2048;  // fewer, larger workgroups only when there are plenty (8 per compute unit)
 constexpr int64_t kPackedMaxRowBytesDefault = 2048;
 
 int64_t packed_max_row_bytes() {
@@ -264,8 +272,11 @@ int packed_group(int64_t rows, int64_t T, int64_t element_bytes, int64_t tile, i
     if (rows < 2 || T * element_bytes >= packed_max_row_bytes()) return 0;
     int64_t group = (tile - grid) / T;
     if (group < 2) return 0;
+    // a whole number of grid cells per group, so that every group starts on the grid like
+    // the first, unless that would leave more than 15 % of the tile empty
     const int64_t whole_lines = grid / gcd64(T, grid);  // rows per whole number of grid cells
-    if (group >= whole_lines) group -= group % whole_lines;
+    const int64_t whole = group - group % whole_lines;
+    if (whole > 0 && whole * 100 >= group * 85) group = whole;
     return (int)group;
 }
 
