@@ -43,12 +43,33 @@ __device__ __forceinline__ void split_position(int rel, int T, float inv_T, int&
 
 // Forward / reverse scan: at the element that starts the recurrence of its row
 // (first in time order), token += gate * x_start and gate = 0.
+//
+// Rows at least as long as a vector put at most one such element into a
+// vector; its index is worked out once per vector and the elements only compare
+// their (compile-time) index with it.  Shorter rows take the element-by-element
+// walk.
 template <class Tr, bool REV>
 __device__ __forceinline__ void cut_rows(typename Tr::V (&g)[Tr::EPV], typename Tr::V (&t)[Tr::EPV], int rel0,
                                          const Cuts<Tr>& cuts) {
     using V = typename Tr::V;
     int row, pos;
     split_position(rel0, cuts.T, cuts.inv_T, row, pos);
+    if (cuts.T >= Tr::EPV) {  // wave-uniform
+        // forward: the row's first element (pos 0); reverse: its last (pos T-1)
+        const int at = REV ? cuts.T - 1 - pos : (pos == 0 ? 0 : cuts.T - pos);
+        const int cut_row = REV ? row : row + (pos != 0);
+        const bool valid = at < Tr::EPV && (unsigned)(rel0 + at) < (unsigned)cuts.len;
+        const int cut_at = valid ? at : -1;
+        V start = vzero<V>();
+        if (cuts.stage != nullptr && valid) start = Tr::load1(cuts.stage + (cut_row - cuts.first_row));
+#pragma unroll
+        for (int e = 0; e < Tr::EPV; ++e) {
+            const bool cut = cut_at == e;
+            t[e] = vselect(cut, vfma(g[e], start, t[e]), t[e]);
+            g[e] = vselect(cut, vzero<V>(), g[e]);
+        }
+        return;
+    }
 #pragma unroll
     for (int e = 0; e < Tr::EPV; ++e) {
         const bool valid = (unsigned)(rel0 + e) < (unsigned)cuts.len;
@@ -68,7 +89,8 @@ __device__ __forceinline__ void cut_rows(typename Tr::V (&g)[Tr::EPV], typename 
 // `before[e]` the state that precedes it; at a row's last element nothing
 // follows (0), at its first the state before it is the row's initial state.
 // is_first[e] / row_of[e] tell the caller where to put the gradient of that
-// initial state.
+// initial state.  Rows at least as long as a vector have at most one first and
+// one last element in a vector (as above).
 template <class Tr>
 __device__ __forceinline__ void cut_rows_backward(typename Tr::V (&after)[Tr::EPV], typename Tr::V (&before)[Tr::EPV],
                                                   bool (&is_first)[Tr::EPV], int (&row_of)[Tr::EPV], int rel0,
@@ -76,6 +98,26 @@ __device__ __forceinline__ void cut_rows_backward(typename Tr::V (&after)[Tr::EP
     using V = typename Tr::V;
     int row, pos;
     split_position(rel0, cuts.T, cuts.inv_T, row, pos);
+    if (cuts.T >= Tr::EPV) {  // wave-uniform
+        const int first_e = pos == 0 ? 0 : cuts.T - pos;
+        const int last_e = cuts.T - 1 - pos;
+        const int first_row = row + (pos != 0);
+        const bool first_valid = first_e < Tr::EPV && (unsigned)(rel0 + first_e) < (unsigned)cuts.len;
+        const bool last_valid = last_e < Tr::EPV && (unsigned)(rel0 + last_e) < (unsigned)cuts.len;
+        const int first_at = first_valid ? first_e : -1;
+        const int last_at = last_valid ? last_e : -1;
+        V start = vzero<V>();
+        if (cuts.stage != nullptr && first_valid) start = Tr::load1(cuts.stage + (first_row - cuts.first_row));
+#pragma unroll
+        for (int e = 0; e < Tr::EPV; ++e) {
+            const bool first = first_at == e;
+            before[e] = vselect(first, start, before[e]);
+            after[e] = vselect(last_at == e, vzero<V>(), after[e]);
+            is_first[e] = first;
+            row_of[e] = first_row;
+        }
+        return;
+    }
 #pragma unroll
     for (int e = 0; e < Tr::EPV; ++e) {
         const bool valid = (unsigned)(rel0 + e) < (unsigned)cuts.len;
