@@ -129,13 +129,18 @@ __global__ void __launch_bounds__(64 * kMaxWavesPerBlock)
 
         // Pass 1: fold each vector into one (A, X) pair and scan the pairs.
         V totA[U], totX[U], exA[U], exX[U];
+        CutAt<V> cut_found[PACKED ? U : 1];  // packed rows: where each vector is cut, kept for pass 2
 #pragma unroll
         for (int j = 0; j < U; ++j) {
             V g[EPV], t[EPV];
             Tr::unpack(graw[j], g);
             activate<ACT>(g);
             Tr::unpack(traw[j], t);
-            if constexpr (PACKED) cut_rows<Tr, REV>(g, t, (int)(sub_base - lo) + vec_offset<U, EPV, REV>(j, lane), cuts);
+            if constexpr (PACKED) {
+                const int rel = (int)(sub_base - lo) + vec_offset<U, EPV, REV>(j, lane);
+                cut_found[j] = locate_cut<Tr, REV>(rel, cuts);
+                cut_rows<Tr, REV>(g, t, rel, cuts, cut_found[j]);
+            }
             constexpr int e0 = REV ? EPV - 1 : 0;
             V A = g[e0];
             V X = t[e0];
@@ -185,7 +190,9 @@ __global__ void __launch_bounds__(64 * kMaxWavesPerBlock)
             Tr::unpack(graw[j], g);
             activate<ACT>(g);
             Tr::unpack(traw[j], t);
-            if constexpr (PACKED) cut_rows<Tr, REV>(g, t, (int)(sub_base - lo) + vec_offset<U, EPV, REV>(j, lane), cuts);
+            if constexpr (PACKED) {
+                cut_rows<Tr, REV>(g, t, (int)(sub_base - lo) + vec_offset<U, EPV, REV>(j, lane), cuts, cut_found[j]);
+            }
             V x = carry_in<PACKED>(exA[j], c, exX[j]);  // state entering this lane's vector
             c = carry_in<PACKED>(totA[j], c, totX[j]);  // state entering the next block
             V o[EPV];

@@ -45,31 +45,48 @@ __device__ __forceinline__ void split_position(int rel, int T, float inv_T, int&
 // (first in time order), token += gate * x_start and gate = 0.
 //
 // Rows at least as long as a vector put at most one such element into a
-// vector; its index is worked out once per vector and the elements only compare
-// their (compile-time) index with it.  Shorter rows take the element-by-element
-// walk.
+// vector: it is located once per vector (locate_cut; the kernel keeps the answer
+// for its second pass over the registers) and the elements only compare their
+// compile-time index with it.  Shorter rows take the element-by-element walk
+// every time.
+template <class V>
+struct CutAt {
+    int at;   // index of the element in the vector, or -1
+    V start;  // the state its row starts from
+};
+
 template <class Tr, bool REV>
-__device__ __forceinline__ void cut_rows(typename Tr::V (&g)[Tr::EPV], typename Tr::V (&t)[Tr::EPV], int rel0,
-                                         const Cuts<Tr>& cuts) {
+__device__ __forceinline__ CutAt<typename Tr::V> locate_cut(int rel0, const Cuts<Tr>& cuts) {
     using V = typename Tr::V;
-    int row, pos;
-    split_position(rel0, cuts.T, cuts.inv_T, row, pos);
+    CutAt<V> found{-1, vzero<V>()};
     if (cuts.T >= Tr::EPV) {  // wave-uniform
+        int row, pos;
+        split_position(rel0, cuts.T, cuts.inv_T, row, pos);
         // forward: the row's first element (pos 0); reverse: its last (pos T-1)
         const int at = REV ? cuts.T - 1 - pos : (pos == 0 ? 0 : cuts.T - pos);
         const int cut_row = REV ? row : row + (pos != 0);
         const bool valid = at < Tr::EPV && (unsigned)(rel0 + at) < (unsigned)cuts.len;
-        const int cut_at = valid ? at : -1;
-        V start = vzero<V>();
-        if (cuts.stage != nullptr && valid) start = Tr::load1(cuts.stage + (cut_row - cuts.first_row));
+        if (valid) found.at = at;
+        if (cuts.stage != nullptr && valid) found.start = Tr::load1(cuts.stage + (cut_row - cuts.first_row));
+    }
+    return found;
+}
+
+template <class Tr, bool REV>
+__device__ __forceinline__ void cut_rows(typename Tr::V (&g)[Tr::EPV], typename Tr::V (&t)[Tr::EPV], int rel0,
+                                         const Cuts<Tr>& cuts, const CutAt<typename Tr::V>& found) {
+    using V = typename Tr::V;
+    if (cuts.T >= Tr::EPV) {  // wave-uniform
 #pragma unroll
         for (int e = 0; e < Tr::EPV; ++e) {
-            const bool cut = cut_at == e;
-            t[e] = vselect(cut, vfma(g[e], start, t[e]), t[e]);
+            const bool cut = found.at == e;
+            t[e] = vselect(cut, vfma(g[e], found.start, t[e]), t[e]);
             g[e] = vselect(cut, vzero<V>(), g[e]);
         }
         return;
     }
+    int row, pos;
+    split_position(rel0, cuts.T, cuts.inv_T, row, pos);
 #pragma unroll
     for (int e = 0; e < Tr::EPV; ++e) {
         const bool valid = (unsigned)(rel0 + e) < (unsigned)cuts.len;
