@@ -17,8 +17,9 @@ scan (oracle/ref_scan.py, the restatement of the reference's ref.scan) on the
 host cores on a bounded sample of the same workload.
 
 Other workloads: --dtype {fp32,bf16,fp16,c64} --shape B D T.  --sweep FILE runs
-the reference's benchmark grid and --precision FILE its max-abs-error table,
-one JSON line per point into FILE (the single summary line is still printed).
+the reference's benchmark grid, one JSON line per point into FILE (the single
+summary line is still printed).  The reference's max-abs-error table is
+tests/precision_table.py.
 """
 
 import argparse
@@ -58,8 +59,6 @@ def parse_args():
     ap.add_argument("--sweep", type=str, default=None, metavar="FILE",
                     help="also run the reference's benchmark grid ((8,1536,T), T=128..65536, forward / "
                          "reverse / backward / train, fp32 and bf16; complex (1,512,131072)) into FILE")
-    ap.add_argument("--precision", type=str, default=None, metavar="FILE",
-                    help="also write max-abs error vs the fp64 recurrence, T=32..65536, fp32/fp16/bf16")
     return ap.parse_args()
 
 
@@ -221,35 +220,6 @@ def run_sweep(path, steps, warmup):
         emit(rec)
 
 
-def run_precision(path):
-    """Max-abs error against the fp64 recurrence for U(0,1) inputs, T = 32..65536,
-    shape (1, 512, T) -- the quantity the reference plots in max-abs-error.png
-    (README.md:60-64 of the reference).  Also reports the torch tree scan run in
-    the same storage dtype, which is what the reference's kernels are judged by."""
-    import numpy as np
-    import torch
-
-    from accelerated_scan.warp import scan_forward
-    from oracle import ref_scan, seqscan
-
-    with open(path, "w") as f:
-        for T in [2 ** i for i in range(5, 17)]:
-            gen = torch.Generator().manual_seed(3407)
-            gates32 = torch.rand(1, 512, T, generator=gen)
-            tokens32 = torch.rand(1, 512, T, generator=gen)
-            rec = {"T": T}
-            for name, dt in (("fp32", torch.float32), ("fp16", torch.float16), ("bf16", torch.bfloat16)):
-                g = gates32.to(dt)
-                x = tokens32.to(dt)
-                truth = seqscan.forward(g.float().numpy(), x.float().numpy())
-                hip = scan_forward(g.to("cuda:0"), x.to("cuda:0")).float().cpu().numpy()
-                tree = ref_scan.scan(g.to("cuda:0"), x.to("cuda:0")).float().cpu().numpy()
-                rec[f"{name}_hip_max_abs_err"] = float(np.abs(hip - truth).max())
-                rec[f"{name}_tree_scan_same_dtype_max_abs_err"] = float(np.abs(tree - truth).max())
-            f.write(json.dumps(rec) + "\n")
-            f.flush()
-
-
 def cpu_baseline(shape, dtype_name):
     """Tree scan (the reference's CPU path, restated) forward+backward on the
     host cores, on a slice of the workload's rows sized to take ~10-30 s."""
@@ -321,8 +291,6 @@ def main():
 
     if args.sweep:
         run_sweep(args.sweep, max(5, args.steps), args.warmup)
-    if args.precision:
-        run_precision(args.precision)
 
     dtype_field = {"fp32": "f32", "bf16": "bf16 storage, f32 arithmetic",
                    "fp16": "f16 storage, f32 arithmetic", "c64": "complex64 (f32 pairs)"}[args.dtype]
