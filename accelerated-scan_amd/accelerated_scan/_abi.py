@@ -13,7 +13,7 @@ from pathlib import Path
 
 import torch
 
-ABI_VERSION = 4
+ABI_VERSION = 5
 
 # ascan_gate codes of include/ascan.h
 GATE_IDENTITY, GATE_SIGMOID = 0, 1

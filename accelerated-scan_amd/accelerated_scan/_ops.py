@@ -6,6 +6,13 @@ autograd nodes in ``warp``, ``scalar`` and ``complex`` therefore switch to
 these operators while a graph is being captured and call the C ABI directly
 otherwise (less Python overhead per call).  The reference advertises
 ``torch.compile`` for its torch scan only (README.md:36 of the reference).
+
+The three forward operators carry autograd formulas of their own
+(``torch.library.register_autograd``, at the end of this file), so
+``torch.ops.accelerated_scan.scan_forward(gates, tokens, False)`` is
+differentiable without any ``autograd.Function`` around it, in eager mode and
+under ``torch.compile``.  Every operator validates its arguments itself: they
+are public as ``torch.ops.accelerated_scan.*``.
 """
 
 from typing import Tuple
@@ -15,8 +22,40 @@ import torch
 from . import _abi
 
 
+def _check_dense(first: torch.Tensor, others, token_like=None, states=()) -> None:
+    """All tensors of a call: device tensors on one device, contiguous, of one
+    shape; ``others`` share the dtype of ``first``; ``token_like`` may be
+    float32 beside complex64; ``states`` hold one element per row."""
+    def fail(what):
+        raise RuntimeError(f"accelerated_scan: expected {what}")
+
+    if not first.is_cuda:
+        fail("device tensors")
+    if first.dim() < 1:
+        fail("tensors with a sequence axis")
+    for t in tuple(others) + ((token_like,) if token_like is not None else ()):
+        if not t.is_cuda or t.device != first.device:
+            fail("all tensors on one GPU")
+        if t.shape != first.shape:
+            fail(f"tensors of one shape, got {tuple(first.shape)} and {tuple(t.shape)}")
+        if not t.is_contiguous():
+            fail("contiguous tensors")
+    if not first.is_contiguous():
+        fail("contiguous tensors")
+    for t in others:
+        if t.dtype != first.dtype:
+            fail(f"tensors of one dtype, got {first.dtype} and {t.dtype}")
+    if token_like is not None:
+        _abi.dtype_code(first.dtype, token_like.dtype)  # raises for unsupported combinations
+    for t in states:
+        if (not t.is_cuda or t.device != first.device or t.dtype != first.dtype
+                or t.shape != first.shape[:-1] or not t.is_contiguous()):
+            fail(f"a contiguous {first.dtype} state of shape {tuple(first.shape[:-1])} on {first.device}")
+
+
 @torch.library.custom_op("accelerated_scan::scan_forward", mutates_args=())
 def scan_forward(gates: torch.Tensor, tokens: torch.Tensor, reverse: bool) -> torch.Tensor:
+    _check_dense(gates, (), token_like=tokens)
     out = torch.empty_like(gates)  # complex gates with real tokens give complex states
     _abi.forward(gates, tokens, out, reverse)
     return out
@@ -31,6 +70,7 @@ def _(gates, tokens, reverse):
 def scan_backward(
     gates: torch.Tensor, states: torch.Tensor, grad_out: torch.Tensor, real_tokens: bool
 ) -> Tuple[torch.Tensor, torch.Tensor]:
+    _check_dense(gates, (states, grad_out))
     d_gates = torch.empty_like(gates)
     d_tokens = _empty_token_grad(gates, real_tokens)
     _abi.backward(gates, states, grad_out, d_gates, d_tokens)
@@ -44,6 +84,7 @@ def _(gates, states, grad_out, real_tokens):
 
 @torch.library.custom_op("accelerated_scan::scan_forward_from", mutates_args=())
 def scan_forward_from(gates: torch.Tensor, tokens: torch.Tensor, initial: torch.Tensor, reverse: bool) -> torch.Tensor:
+    _check_dense(gates, (), token_like=tokens, states=(initial,))
     out = torch.empty_like(gates)
     _abi.forward(gates, tokens, out, reverse, initial=initial)
     return out
@@ -58,6 +99,7 @@ def _(gates, tokens, initial, reverse):
 def scan_backward_from(
     gates: torch.Tensor, states: torch.Tensor, initial: torch.Tensor, grad_out: torch.Tensor, real_tokens: bool
 ) -> Tuple[torch.Tensor, torch.Tensor, torch.Tensor]:
+    _check_dense(gates, (states, grad_out), states=(initial,))
     d_gates = torch.empty_like(gates)
     d_tokens = _empty_token_grad(gates, real_tokens)
     d_initial = torch.zeros_like(initial)  # stays zero for an empty sequence
@@ -72,6 +114,7 @@ def _(gates, states, initial, grad_out, real_tokens):
 
 @torch.library.custom_op("accelerated_scan::scan_forward_gated", mutates_args=())
 def scan_forward_gated(gate_inputs: torch.Tensor, tokens: torch.Tensor, initial: torch.Tensor, gate: int) -> torch.Tensor:
+    _check_dense(gate_inputs, (tokens,), states=(initial,))
     out = torch.empty_like(gate_inputs)
     _abi.forward_gated(gate_inputs, tokens, out, gate, initial=initial)
     return out
@@ -86,6 +129,7 @@ def _(gate_inputs, tokens, initial, gate):
 def scan_backward_gated(
     gate_inputs: torch.Tensor, states: torch.Tensor, initial: torch.Tensor, grad_out: torch.Tensor, gate: int
 ) -> Tuple[torch.Tensor, torch.Tensor, torch.Tensor]:
+    _check_dense(gate_inputs, (states, grad_out), states=(initial,))
     d_gate_inputs = torch.empty_like(gate_inputs)
     d_tokens = torch.empty_like(gate_inputs)
     d_initial = torch.zeros_like(initial)  # stays zero for an empty sequence
@@ -109,3 +153,77 @@ def _empty_token_grad(gates: torch.Tensor, real_tokens: bool) -> torch.Tensor:
 def capturing() -> bool:
     """True while torch.compile is tracing the caller."""
     return torch.compiler.is_compiling()
+
+
+# ---------------------------------------------------------------------------
+# Autograd formulas of the forward operators.  The gradient of a scan is the
+# fused backward operator (accelerated_scan/warp.py:50-65 of the reference:
+# g[t] = grad[t] + gates[t+1] * g[t+1], d_tokens = g, d_gates[t] = g[t] * x[t-1]).
+# A reverse scan is the forward scan of the flipped sequences, flipped, so its
+# gradient is the flipped gradient of that scan.
+# ---------------------------------------------------------------------------
+def _flip(t: torch.Tensor) -> torch.Tensor:
+    return t.flip(-1).contiguous()
+
+
+def _real_tokens(gates: torch.Tensor, tokens: torch.Tensor) -> bool:
+    return gates.is_complex() and not tokens.is_complex()
+
+
+def _setup_scan_forward(ctx, inputs, output):
+    gates, tokens, reverse = inputs
+    ctx.save_for_backward(gates, output)
+    ctx.reverse = reverse
+    ctx.real_tokens = _real_tokens(gates, tokens)
+
+
+def _backward_scan_forward(ctx, grad):
+    gates, states = ctx.saved_tensors
+    grad = grad.contiguous()
+    if ctx.reverse:
+        d_gates, d_tokens = scan_backward(_flip(gates), _flip(states), _flip(grad), ctx.real_tokens)
+        return _flip(d_gates), _flip(d_tokens), None
+    d_gates, d_tokens = scan_backward(gates, states, grad, ctx.real_tokens)
+    return d_gates, d_tokens, None
+
+
+torch.library.register_autograd(
+    "accelerated_scan::scan_forward", _backward_scan_forward, setup_context=_setup_scan_forward)
+
+
+def _setup_scan_forward_from(ctx, inputs, output):
+    gates, tokens, initial, reverse = inputs
+    ctx.save_for_backward(gates, output, initial)
+    ctx.reverse = reverse
+    ctx.real_tokens = _real_tokens(gates, tokens)
+
+
+def _backward_scan_forward_from(ctx, grad):
+    gates, states, initial = ctx.saved_tensors
+    grad = grad.contiguous()
+    if ctx.reverse:
+        d_gates, d_tokens, d_initial = scan_backward_from(
+            _flip(gates), _flip(states), initial, _flip(grad), ctx.real_tokens)
+        return _flip(d_gates), _flip(d_tokens), d_initial, None
+    d_gates, d_tokens, d_initial = scan_backward_from(gates, states, initial, grad, ctx.real_tokens)
+    return d_gates, d_tokens, d_initial, None
+
+
+torch.library.register_autograd(
+    "accelerated_scan::scan_forward_from", _backward_scan_forward_from, setup_context=_setup_scan_forward_from)
+
+
+def _setup_scan_forward_gated(ctx, inputs, output):
+    gate_inputs, _, initial, gate = inputs
+    ctx.save_for_backward(gate_inputs, output, initial)
+    ctx.gate = gate
+
+
+def _backward_scan_forward_gated(ctx, grad):
+    gate_inputs, states, initial = ctx.saved_tensors
+    d_gate_inputs, d_tokens, d_initial = scan_backward_gated(gate_inputs, states, initial, grad.contiguous(), ctx.gate)
+    return d_gate_inputs, d_tokens, d_initial, None
+
+
+torch.library.register_autograd(
+    "accelerated_scan::scan_forward_gated", _backward_scan_forward_gated, setup_context=_setup_scan_forward_gated)

@@ -65,6 +65,28 @@ size_t token_size(int dtype) { return dtype == ASCAN_C64_REAL_TOKENS ? 4 : eleme
 
 bool element_aligned(const void* p, size_t es) { return (reinterpret_cast<uintptr_t>(p) % es) == 0; }
 
+// A buffer of a call as a byte range (null buffers are empty ranges).
+struct Span {
+    uintptr_t begin, end;
+};
+Span span_of(const void* p, int64_t elements, size_t element_bytes) {
+    const uintptr_t b = reinterpret_cast<uintptr_t>(p);
+    return Span{b, p ? b + (uintptr_t)elements * element_bytes : b};
+}
+bool overlap(const Span& a, const Span& b) { return a.begin < b.end && b.begin < a.end; }
+
+// True when an output range meets an input range or another output range.
+template <size_t NI, size_t NO>
+bool outputs_overlap(const Span (&inputs)[NI], const Span (&outputs)[NO]) {
+    for (size_t o = 0; o < NO; ++o) {
+        for (size_t i = 0; i < NI; ++i)
+            if (overlap(outputs[o], inputs[i])) return true;
+        for (size_t q = o + 1; q < NO; ++q)
+            if (overlap(outputs[o], outputs[q])) return true;
+    }
+    return false;
+}
+
 // Largest row count one launch can address: gridDim.x is limited to 2^31-1.
 constexpr int64_t kMaxBlocks = 2147483647LL;
 
@@ -84,6 +106,12 @@ int forward_checked(const void* gates, const void* tokens, void* out, const void
     if (!element_aligned(gates, es) || !element_aligned(tokens, token_size(dtype)) || !element_aligned(out, es) ||
         !element_aligned(initial, es))
         return ASCAN_ERR_MISALIGNED;
+    {
+        const int64_t n = rows * seqlen;
+        const Span inputs[] = {span_of(gates, n, es), span_of(tokens, n, token_size(dtype)), span_of(initial, rows, es)};
+        const Span outputs[] = {span_of(out, n, es)};
+        if (outputs_overlap(inputs, outputs)) return ASCAN_ERR_OVERLAP;
+    }
     const ForwardCall call{gates, tokens, out, initial, rows, seqlen, reverse != 0, act, ws,
                            static_cast<hipStream_t>(stream)};
     switch (dtype) {
@@ -108,6 +136,14 @@ int backward_checked(const void* gates, const void* states, const void* grad_out
         !element_aligned(d_gates, es) || !element_aligned(d_tokens, token_size(dtype)) ||
         !element_aligned(initial, es) || !element_aligned(d_initial, es))
         return ASCAN_ERR_MISALIGNED;
+    {
+        const int64_t n = rows * seqlen;
+        const Span inputs[] = {span_of(gates, n, es), span_of(states, n, es), span_of(grad_out, n, es),
+                               span_of(initial, rows, es)};
+        const Span outputs[] = {span_of(d_gates, n, es), span_of(d_tokens, n, token_size(dtype)),
+                                span_of(d_initial, rows, es)};
+        if (outputs_overlap(inputs, outputs)) return ASCAN_ERR_OVERLAP;
+    }
     const BackwardCall call{gates, states, grad_out, d_gates, d_tokens, initial, d_initial, rows, seqlen, act, ws,
                             static_cast<hipStream_t>(stream)};
     switch (dtype) {
@@ -205,6 +241,7 @@ const char* ascan_status_string(int status) {
         case ASCAN_ERR_LAUNCH: return "the HIP runtime reported a launch error";
         case ASCAN_ERR_BAD_ACTIVATION:
             return "unsupported gate activation: expecting identity, or sigmoid with float32, bfloat16 or float16";
+        case ASCAN_ERR_OVERLAP: return "an output buffer overlaps an input or another output buffer of the call";
         default: return "unknown status";
     }
 }

@@ -99,12 +99,8 @@ __device__ __forceinline__ cfloat poison(cfloat) { return cfloat{__builtin_nanf(
 // the call can be captured into a graph).
 __global__ void split_reset_kernel(uint32_t* words, size_t nwords, unsigned long long wait_limit) {
     const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
-    if (i < nwords) words[i] = 0u;
-    if (i == 0) {
-        // the limit occupies words 2 and 3 of the header
-        words[2] = (uint32_t)wait_limit;
-        words[3] = (uint32_t)(wait_limit >> 32);
-    }
+    // the limit occupies words 2 and 3 of the header; every word has exactly one writer
+    if (i < nwords) words[i] = i == 2 ? (uint32_t)wait_limit : (i == 3 ? (uint32_t)(wait_limit >> 32) : 0u);
 }
 
 // Layout of the table: header, one ticket line per row, one record per (row, tile).

@@ -23,11 +23,26 @@
  *     nothing, keeps no reference after the call returns and holds no mutable
  *     global state, so calls are re-entrant from any host thread (the *_split
  *     calls additionally need a caller-provided workspace per concurrent call);
+ *   - kernels are launched on the calling thread's CURRENT HIP device: every
+ *     pointer of a call (buffers, workspace) must be memory of that device and
+ *     `stream` a stream of that device.  The library does not look the pointers
+ *     up; a caller with several GPUs makes the right one current first
+ *     (hipSetDevice), as the Python binding does;
  *   - work is enqueued on `stream` (a hipStream_t passed as void*, NULL = the
  *     default stream) and the call returns without synchronising;
  *   - rows are dense: row r starts at element r*seqlen; 64-bit element offsets
  *     are used throughout, so rows*seqlen may exceed 2^31;
- *   - input and output buffers must not overlap;
+ *   - no output buffer may overlap an input buffer or another output buffer of
+ *     the same call (the kernels read and write rows in tiles, out of order
+ *     across workgroups): such a call is refused with ASCAN_ERR_OVERLAP and
+ *     nothing is launched;
+ *   - rows shorter than 2 KiB are scanned several to a workgroup, as one long
+ *     sequence with a zero gate inserted in front of every row.  In that mode a
+ *     gate of exactly zero discards the state it multiplies even when that state
+ *     is not finite (0 * inf counts as 0, not NaN), for the inserted zeros and
+ *     for zeros stored in `gates` alike; for longer rows, as in the reference,
+ *     a stored zero gate times a non-finite state is NaN.  Finite data is not
+ *     affected;
  *   - arithmetic is done in fp32 for every dtype (bf16/fp16 are storage
  *     formats, rounded to nearest-even on store);
  *   - buffers whose addresses agree modulo 16 (the usual case: allocator
@@ -47,7 +62,7 @@
 extern "C" {
 #endif
 
-#define ASCAN_ABI_VERSION 4
+#define ASCAN_ABI_VERSION 5
 
 /* Marks the exported entry points (the library is built with hidden visibility). */
 #define ASCAN_API __attribute__((visibility("default")))
@@ -76,7 +91,8 @@ enum ascan_status {
     ASCAN_ERR_BAD_DTYPE     = 3, /* dtype is not an ascan_dtype (warp.cuh:390-391) */
     ASCAN_ERR_MISALIGNED    = 4, /* a pointer is not aligned to its element size */
     ASCAN_ERR_LAUNCH        = 5, /* the HIP runtime refused the launch (see ascan_last_hip_error) */
-    ASCAN_ERR_BAD_ACTIVATION = 6 /* gate is not an ascan_gate, or not available for this dtype */
+    ASCAN_ERR_BAD_ACTIVATION = 6, /* gate is not an ascan_gate, or not available for this dtype */
+    ASCAN_ERR_OVERLAP       = 7  /* an output buffer overlaps an input or another output of the call */
 };
 
 /* What the kernels make of the stored gate values (the *_gated entry points). */

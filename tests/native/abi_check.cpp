@@ -145,6 +145,16 @@ void check_status_codes(hipStream_t stream) {
     EXPECT(ascan_forward(a.p, b.p, c.p, -1, 16, ASCAN_F32, 0, stream) == ASCAN_ERR_BAD_SHAPE);
     EXPECT(ascan_forward((char*)a.p + 2, b.p, c.p, 1, 16, ASCAN_F32, 0, stream) == ASCAN_ERR_MISALIGNED);
     EXPECT(ascan_backward(a.p, b.p, c.p, nullptr, a.p, 1, 16, ASCAN_F32, stream) == ASCAN_ERR_NULL_POINTER);
+    // outputs may not overlap inputs or each other; buffers that merely touch are fine
+    EXPECT(ascan_forward(a.p, b.p, a.p, 1, 16, ASCAN_F32, 0, stream) == ASCAN_ERR_OVERLAP);
+    EXPECT(ascan_forward(a.p, b.p, (char*)b.p + 32, 1, 16, ASCAN_F32, 0, stream) == ASCAN_ERR_OVERLAP);
+    EXPECT(ascan_backward(a.p, b.p, c.p, (char*)a.p + 1024, (char*)a.p + 1024 + 60, 1, 16, ASCAN_F32, stream) ==
+           ASCAN_ERR_OVERLAP);
+    EXPECT(ascan_backward(a.p, b.p, c.p, (char*)c.p + 60, (char*)a.p + 1024, 1, 16, ASCAN_F32, stream) ==
+           ASCAN_ERR_OVERLAP);
+    EXPECT(ascan_forward(a.p, (char*)a.p + 64, (char*)a.p + 128, 1, 16, ASCAN_F32, 0, stream) == ASCAN_OK);
+    EXPECT(ascan_backward(a.p, (char*)a.p + 64, (char*)a.p + 128, (char*)a.p + 192, (char*)a.p + 256, 1, 16, ASCAN_F32,
+                          stream) == ASCAN_OK);
     // empty problems are accepted without touching any pointer
     EXPECT(ascan_forward(nullptr, nullptr, nullptr, 0, 16, ASCAN_F32, 0, stream) == ASCAN_OK);
     EXPECT(ascan_backward(nullptr, nullptr, nullptr, nullptr, nullptr, 4, 0, ASCAN_F32, stream) == ASCAN_OK);

@@ -36,8 +36,8 @@ def test_library_exports_every_declared_symbol():
 def test_abi_version_and_status_strings():
     lib = _abi.load()
     assert lib.ascan_abi_version() == _abi.ABI_VERSION
-    texts = {lib.ascan_status_string(i).decode() for i in range(7)}
-    assert len(texts) == 7 and "ok" in texts
+    texts = {lib.ascan_status_string(i).decode() for i in range(8)}
+    assert len(texts) == 8 and "ok" in texts
     assert lib.ascan_status_string(99).decode() == "unknown status"
 
 
@@ -70,6 +70,28 @@ def test_argument_validation_returns_codes():
     assert lib.ascan_forward(p + 1, p, p, 1, 4, 1, 0, None) == 4
     assert lib.ascan_forward(p + 4, p, p, 1, 4, 3, 0, None) == 4
     assert lib.ascan_backward(p, p, p, p + 2, p, 1, 4, 0, None) == 4
+
+
+def test_overlapping_buffers_are_refused():
+    """An output that overlaps an input or another output is refused by a host-side
+    interval check before anything is launched (include/ascan.h: ASCAN_ERR_OVERLAP)."""
+    lib = _abi.load()
+    buf = ctypes.create_string_buffer(4096)
+    p = ctypes.addressof(buf)
+    p += -p % 64
+    n = 16  # one row of 16 fp32 elements = 64 bytes
+    assert lib.ascan_forward(p, p + 64, p, 1, n, 0, 0, None) == 7              # out is gates
+    assert lib.ascan_forward(p, p + 64, p + 64 + 60, 1, n, 0, 0, None) == 7    # out starts inside tokens
+    assert lib.ascan_forward(p + 60, p + 256, p, 1, n, 0, 0, None) == 7        # gates start inside out
+    assert lib.ascan_forward_from(p, p + 64, p + 128 + 32, p + 128, 1, n, 0, 0, None, 0, None) == 7  # initial inside out
+    assert lib.ascan_backward(p, p + 64, p + 128, p + 128, p + 256, 1, n, 0, None) == 7      # d_gates is grad_out
+    assert lib.ascan_backward(p, p + 64, p + 128, p + 256, p + 256 + 32, 1, n, 0, None) == 7  # the two outputs overlap
+    assert lib.ascan_backward_from(p, p + 64, None, p + 128, p + 192, p + 256, p + 192 + 8, 1, n, 0, None, 0, None) == 7
+    # complex gates with real tokens: the token buffers are half as long
+    assert lib.ascan_forward(p, p + 256, p + 256 + 56, 1, n, 4, 0, None) == 7   # 16 c64 = 128 bytes, tokens 64 bytes
+    # bf16: 32 bytes per row; ranges that only touch are fine for the check (the
+    # call then stops at the next one, here the missing d_tokens)
+    assert lib.ascan_backward(p, p + 32, p + 64, p + 96, None, 1, n, 1, None) == 1
 
 
 def test_workspace_sizing_and_split_entry_validation():
