@@ -54,6 +54,11 @@ _SIGNATURES = {
          ctypes.c_void_p, ctypes.c_size_t, ctypes.c_void_p],
     ),
     "ascan_workspace_timeouts": (ctypes.c_uint, [ctypes.c_void_p]),
+    "ascan_forward_split_static": (
+        ctypes.c_int,
+        [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p,
+         ctypes.c_int64, ctypes.c_int64, ctypes.c_int, ctypes.c_int, ctypes.c_void_p],
+    ),
     "ascan_forward_from": (
         ctypes.c_int,
         [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p,

@@ -39,6 +39,8 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
+#include <atomic>
+
 #include "ascan.h"
 #include "dispatch.h"
 #include "policy.h"
@@ -48,6 +50,37 @@ namespace ascan {
 thread_local int g_last_hip_error = 0;
 
 namespace {
+
+// Split-row table of ascan_forward_split_static: device memory that belongs to the
+// library's code object, so the entry point needs no allocation.  Each GPU the
+// library runs on holds its own copy at its own address until the process ends;
+// the name below is only a host-side handle for hipGetSymbolAddress, never a
+// device address.
+static __device__ __align__(256) unsigned char scratch[ASCAN_STATIC_WORKSPACE_BYTES];
+
+// Address of `scratch` on the current device (looked up once per device), or
+// null with g_last_hip_error set.
+void* static_workspace() {
+    constexpr int kMaxDevices = 64;
+    static std::atomic<void*> known[kMaxDevices];
+    int device = 0;
+    hipError_t e = hipGetDevice(&device);
+    if (e == hipSuccess && (device < 0 || device >= kMaxDevices)) e = hipErrorInvalidDevice;
+    if (e != hipSuccess) {
+        g_last_hip_error = (int)e;
+        return nullptr;
+    }
+    void* ptr = known[device].load(std::memory_order_acquire);
+    if (ptr == nullptr) {
+        e = hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch));
+        if (e != hipSuccess || ptr == nullptr) {
+            g_last_hip_error = (int)(e != hipSuccess ? e : hipErrorInvalidSymbol);
+            return nullptr;
+        }
+        known[device].store(ptr, std::memory_order_release);
+    }
+    return ptr;
+}
 
 size_t element_size(int dtype) {
     switch (dtype) {
@@ -193,6 +226,20 @@ int ascan_forward_split(const void* gates, const void* tokens, void* out, int64_
                            Workspace{workspace, workspace_bytes}, stream);
 }
 
+int ascan_forward_split_static(const void* gates, const void* tokens, void* out, int64_t rows, int64_t seqlen,
+                               int dtype, int reverse, void* stream) {
+    const size_t needed = ascan_workspace_bytes(rows, seqlen, dtype);
+    if (needed > (size_t)ASCAN_STATIC_WORKSPACE_BYTES) return ASCAN_ERR_TOO_LARGE;
+    Workspace ws{nullptr, 0};
+    // needed == 0: rows that are not split (or arguments the checks below refuse) use no table
+    if (needed != 0 && gates && tokens && out) {
+        ws.ptr = static_workspace();
+        if (ws.ptr == nullptr) return ASCAN_ERR_LAUNCH;
+        ws.bytes = (size_t)ASCAN_STATIC_WORKSPACE_BYTES;
+    }
+    return forward_checked(gates, tokens, out, nullptr, rows, seqlen, dtype, reverse, ASCAN_GATE_IDENTITY, ws, stream);
+}
+
 int ascan_backward_split(const void* gates, const void* states, const void* grad_out, void* d_gates,
                          void* d_tokens, int64_t rows, int64_t seqlen, int dtype, void* workspace,
                          size_t workspace_bytes, void* stream) {
@@ -242,6 +289,8 @@ const char* ascan_status_string(int status) {
         case ASCAN_ERR_BAD_ACTIVATION:
             return "unsupported gate activation: expecting identity, or sigmoid with float32, bfloat16 or float16";
         case ASCAN_ERR_OVERLAP: return "an output buffer overlaps an input or another output buffer of the call";
+        case ASCAN_ERR_TOO_LARGE:
+            return "the split-row table of this problem exceeds the library's static workspace (ASCAN_STATIC_WORKSPACE_BYTES)";
         default: return "unknown status";
     }
 }

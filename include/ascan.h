@@ -92,7 +92,8 @@ enum ascan_status {
     ASCAN_ERR_MISALIGNED    = 4, /* a pointer is not aligned to its element size */
     ASCAN_ERR_LAUNCH        = 5, /* the HIP runtime refused the launch (see ascan_last_hip_error) */
     ASCAN_ERR_BAD_ACTIVATION = 6, /* gate is not an ascan_gate, or not available for this dtype */
-    ASCAN_ERR_OVERLAP       = 7  /* an output buffer overlaps an input or another output of the call */
+    ASCAN_ERR_OVERLAP       = 7, /* an output buffer overlaps an input or another output of the call */
+    ASCAN_ERR_TOO_LARGE     = 8  /* ascan_forward_split_static: the table would not fit the static workspace */
 };
 
 /* What the kernels make of the stored gate values (the *_gated entry points). */
@@ -166,6 +167,30 @@ ASCAN_API int ascan_backward_split(const void* gates, const void* states, const 
                          void* workspace, size_t workspace_bytes, void* stream);
 
 ASCAN_API unsigned int ascan_workspace_timeouts(const void* workspace_header_copy);
+
+/*
+ * ascan_forward_split for callers that cannot allocate device memory at all
+ * (code running under HIP graph capture, tight serving loops, harnesses that
+ * forbid hipMalloc): the split-row table lives in a static device-side array
+ * inside the library instead of a caller-provided workspace, and the call
+ * allocates nothing, on the host side or the device side.  It has no
+ * counterpart in the reference.  Results are those of ascan_forward_split.
+ *
+ *   - the array holds ASCAN_STATIC_WORKSPACE_BYTES on every GPU the library is
+ *     used on, from the first call on that GPU until the process ends;
+ *   - a problem whose table (ascan_workspace_bytes) is larger is refused with
+ *     ASCAN_ERR_TOO_LARGE and nothing is launched; problems that are not split
+ *     (ascan_workspace_bytes == 0) run the plain kernels and use no table;
+ *   - all calls on one GPU share that GPU's array (it is cleared by a small
+ *     kernel on `stream` at the start of each call): two calls that may run at
+ *     the same time on one GPU -- different streams, or graph branches -- race
+ *     on it.  Use ascan_forward_split with separate workspaces for those.
+ */
+#define ASCAN_STATIC_WORKSPACE_BYTES (4 * 1024 * 1024)
+
+ASCAN_API int ascan_forward_split_static(const void* gates, const void* tokens, void* out,
+                               int64_t rows, int64_t seqlen, int dtype, int reverse,
+                               void* stream);
 
 /*
  * Scans that start from a given state, for callers that process a long

@@ -36,8 +36,8 @@ def test_library_exports_every_declared_symbol():
 def test_abi_version_and_status_strings():
     lib = _abi.load()
     assert lib.ascan_abi_version() == _abi.ABI_VERSION
-    texts = {lib.ascan_status_string(i).decode() for i in range(8)}
-    assert len(texts) == 8 and "ok" in texts
+    texts = {lib.ascan_status_string(i).decode() for i in range(9)}
+    assert len(texts) == 9 and "ok" in texts
     assert lib.ascan_status_string(99).decode() == "unknown status"
 
 
@@ -119,6 +119,23 @@ def test_workspace_sizing_and_split_entry_validation():
     header = (ctypes.c_uint32 * 16)()
     header[4] = 3
     assert lib.ascan_workspace_timeouts(ctypes.addressof(header)) == 3
+
+
+def test_static_workspace_entry_point_validates_before_touching_the_gpu():
+    """ascan_forward_split_static refuses problems whose table exceeds the static
+    array, and validates like the other entry points, without a GPU."""
+    lib = _abi.load()
+    buf = ctypes.create_string_buffer(4096)
+    p = ctypes.addressof(buf)
+    limit = 4 * 1024 * 1024  # ASCAN_STATIC_WORKSPACE_BYTES
+    assert lib.ascan_workspace_bytes(128, 1 << 24, 0) > limit
+    assert lib.ascan_forward_split_static(p, p + 1024, p + 2048, 128, 1 << 24, 0, 0, None) == 8
+    assert 0 < lib.ascan_workspace_bytes(64, 1 << 22, 0) <= limit
+    assert lib.ascan_forward_split_static(None, p + 1024, p + 2048, 64, 1 << 22, 0, 0, None) == 1
+    assert lib.ascan_forward_split_static(p, p + 1024, p + 2048, 3, 1 << 20, 9, 0, None) == 3
+    assert lib.ascan_forward_split_static(p, p + 1024, p + 2048, -3, 1 << 20, 0, 0, None) == 2
+    assert lib.ascan_forward_split_static(None, None, None, 0, 1 << 20, 0, 0, None) == 0
+    assert "static workspace" in lib.ascan_status_string(8).decode()
 
 
 def test_status_becomes_runtime_error():

@@ -1,0 +1,105 @@
+"""ascan_forward_split_static: the split-row forward scan with its table in the
+library's static device array, for callers that cannot allocate.  Called through
+the raw C ABI and compared with ascan_forward_split (caller-provided workspace)
+and with the fp64 recurrence, on two calls in a row, the second one smaller, so
+that the second call meets the first call's leftovers in the shared array.
+
+The look-back of a split row folds its earlier tiles in an order that depends on
+which of them have published their states yet, so two split runs agree to fp32
+rounding, not bit for bit: the bar is the fp32 one of the other GPU tests,
+2e-5 relative to the largest magnitude.
+"""
+
+import ctypes
+
+import numpy as np
+import pytest
+import torch
+
+from oracle import seqscan
+
+pytestmark = pytest.mark.gpu
+
+DEVICE = "cuda"
+TOO_LARGE = 8
+
+
+def _inputs(rows, T, dtype, seed):
+    gen = torch.Generator().manual_seed(seed)
+    gates = (0.9 + 0.1 * torch.rand(rows, T, generator=gen)).to(dtype)
+    tokens = torch.randn(rows, T, generator=gen).to(dtype)
+    return gates, tokens
+
+
+def _run_both(lib, gates, tokens, code, reverse):
+    from accelerated_scan import _abi
+
+    rows, T = gates.shape
+    g, x = gates.to(DEVICE), tokens.to(DEVICE)
+    nbytes = lib.ascan_workspace_bytes(rows, T, code)
+    assert 0 < nbytes <= 4 * 1024 * 1024, "the case must be a split one that fits the static array"
+    workspace = torch.empty(nbytes, dtype=torch.uint8, device=DEVICE)
+    want = torch.empty_like(g)
+    got = torch.full_like(g, float("nan"))
+    stream = torch.cuda.current_stream().cuda_stream
+    _abi.check(lib.ascan_forward_split(g.data_ptr(), x.data_ptr(), want.data_ptr(), rows, T, code, int(reverse),
+                                       workspace.data_ptr(), nbytes, stream))
+    torch.cuda.synchronize()
+    free_before = torch.cuda.mem_get_info()[0]
+    _abi.check(lib.ascan_forward_split_static(g.data_ptr(), x.data_ptr(), got.data_ptr(), rows, T, code,
+                                              int(reverse), stream))
+    torch.cuda.synchronize()
+    free_after = torch.cuda.mem_get_info()[0]
+    assert _abi.workspace_timeouts(workspace) == 0
+    return got, want, free_before - free_after
+
+
+def _check(got, want, gates, tokens, reverse, tol):
+    truth = seqscan.forward(gates.float().numpy(), tokens.float().numpy(), reverse=reverse)
+    scale = max(1.0, float(np.abs(truth).max()))
+    np.testing.assert_allclose(got.float().cpu().numpy(), want.float().cpu().numpy(), rtol=tol, atol=tol * scale,
+                               err_msg="static table against caller-provided workspace")
+    np.testing.assert_allclose(got.float().cpu().numpy(), truth, rtol=tol, atol=tol * scale,
+                               err_msg="static table against the fp64 recurrence")
+
+
+@pytest.mark.parametrize("dtype,code,tol", [(torch.float32, 0, 2e-5), (torch.bfloat16, 1, 2.0 ** -7)],
+                         ids=["fp32", "bf16"])
+def test_static_table_twice_in_a_row_second_call_smaller(dtype, code, tol):
+    assert torch.cuda.is_available(), "this test needs the MI355X"
+    from accelerated_scan import _abi
+
+    lib = _abi.load()
+    first = _inputs(5, 400000, dtype, seed=101)    # 5 rows x 25 or 49 tiles
+    second = _inputs(2, 70001, dtype, seed=102)    # fewer rows, fewer tiles, odd length
+    grown = []
+    for (gates, tokens), reverse in ((first, False), (second, False), (first, True), (second, True)):
+        got, want, grew = _run_both(lib, gates, tokens, code, reverse)
+        _check(got, want, gates, tokens, reverse, tol)
+        grown.append(grew)
+    # the array exists once per GPU from the first use of the library on; later calls take no device memory
+    assert all(g <= 0 for g in grown[1:]), grown
+
+
+def test_static_table_limit_and_unsplit_shapes():
+    from accelerated_scan import _abi
+
+    lib = _abi.load()
+    g = torch.rand(4, 256, device=DEVICE)
+    x = torch.rand(4, 256, device=DEVICE)
+    out = torch.empty_like(g)
+    stream = torch.cuda.current_stream().cuda_stream
+    # 128 rows of 2^24 elements: 128 x 2049 records of 64 bytes, more than the 4 MiB array -- refused before any access
+    assert lib.ascan_workspace_bytes(128, 1 << 24, 0) > 4 * 1024 * 1024
+    assert lib.ascan_forward_split_static(g.data_ptr(), x.data_ptr(), out.data_ptr(), 128, 1 << 24, 0, 0, stream) == TOO_LARGE
+    assert "static workspace" in lib.ascan_status_string(TOO_LARGE).decode()
+    # a shape that is not split runs the plain kernels: same bits as ascan_forward
+    want = torch.empty_like(g)
+    _abi.check(lib.ascan_forward(g.data_ptr(), x.data_ptr(), want.data_ptr(), 4, 256, 0, 0, stream))
+    _abi.check(lib.ascan_forward_split_static(g.data_ptr(), x.data_ptr(), out.data_ptr(), 4, 256, 0, 0, stream))
+    torch.cuda.synchronize()
+    assert torch.equal(out, want)
+    # validation is that of the other entry points
+    assert lib.ascan_forward_split_static(None, x.data_ptr(), out.data_ptr(), 4, 256, 0, 0, stream) == 1
+    assert lib.ascan_forward_split_static(g.data_ptr(), x.data_ptr(), out.data_ptr(), 4, 256, 9, 0, stream) == 3
+    assert lib.ascan_forward_split_static(g.data_ptr(), x.data_ptr(), g.data_ptr(), 4, 256, 0, 0, stream) == 7
