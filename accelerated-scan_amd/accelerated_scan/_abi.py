@@ -163,22 +163,23 @@ def _stream_handle(index: int) -> int:
     return torch.cuda.current_stream(index).cuda_stream
 
 
-# torch keeps a direct accessor for the same handle (what its own compiled
-# kernels launch on); it skips building a Stream object, several microseconds
-# per call that matter for short sequences.
+# torch keeps direct accessors for the current stream's handle (what its own
+# compiled kernels launch on) and for the current device; they skip building
+# Stream / device objects, several microseconds per call that matter for short
+# sequences.
 _stream_handle = getattr(torch._C, "_cuda_getCurrentRawStream", _stream_handle)
+_current_device = getattr(torch._C, "_cuda_getDevice", torch.cuda.current_device)
 
 
-def _launch(device: torch.device, call) -> None:
-    """Run ``call(stream_handle)`` with ``device`` current (kernels launch on the
-    current device) and map the status."""
-    current = torch.cuda.current_device()
-    index = current if device.index is None else device.index
-    if index == current:
-        status = call(_stream_handle(index))
+def _launch(device: torch.device, fn, *args) -> None:
+    """Call ``fn(*args, stream_handle)`` with ``device`` current (kernels launch on
+    the current device, on torch's current stream there) and map the status."""
+    index = device.index
+    if index is None or index == _current_device():
+        status = fn(*args, _stream_handle(_current_device() if index is None else index))
     else:
         with torch.cuda.device(index):
-            status = call(_stream_handle(index))
+            status = fn(*args, _stream_handle(index))
     if status:
         check(status)
 
@@ -188,7 +189,7 @@ def _workspace_bytes(rows: int, seqlen: int, code: int) -> int:
     return (_lib or load()).ascan_workspace_bytes(rows, seqlen, code)
 
 
-def _workspace(lib, rows: int, seqlen: int, code: int, device: torch.device):
+def _workspace(rows: int, seqlen: int, code: int, device: torch.device):
     """Table for split rows (few rows, long sequences), or None.  Freed by the
     caching allocator in stream order after the kernels that use it."""
     nbytes = _workspace_bytes(rows, seqlen, code)
@@ -209,28 +210,39 @@ def _check_state(state, like, name: str) -> None:
         )
 
 
+def _problem(like, token_like):
+    """(rows, seqlen, ascan_dtype) of a call from a state-like and a token-like tensor."""
+    seqlen = like.shape[-1]
+    rows = like.numel() // seqlen if seqlen else 0
+    dtype, token_dtype = like.dtype, token_like.dtype
+    code = DTYPE_CODES.get(dtype) if dtype == token_dtype else None
+    if code is None:
+        code = dtype_code(dtype, token_dtype)
+    return rows, seqlen, code
+
+
+def _ptr(t):
+    return t.data_ptr() if t is not None else None
+
+
 def forward(gates, tokens, out, reverse: bool, workspace=None, initial=None) -> None:
     """Enqueue the forward scan on the current stream of the tensors' device.
     ``initial`` (one state per row) starts the scan from that state."""
     lib = _lib or load()
-    seqlen = tokens.shape[-1]
-    rows = tokens.numel() // seqlen if seqlen else 0
-    code = dtype_code(gates.dtype, tokens.dtype)
-    if workspace is None:
-        workspace = _workspace(lib, rows, seqlen, code, tokens.device)
+    rows, seqlen, code = _problem(gates, tokens)
+    if workspace is None and _workspace_bytes(rows, seqlen, code):
+        workspace = _workspace(rows, seqlen, code, tokens.device)
     if initial is not None:
         _check_state(initial, out, "initial")
-        _launch(tokens.device, lambda stream: lib.ascan_forward_from(
-            gates.data_ptr(), tokens.data_ptr(), initial.data_ptr(), out.data_ptr(), rows, seqlen, code,
-            1 if reverse else 0, workspace.data_ptr() if workspace is not None else None,
-            workspace.numel() if workspace is not None else 0, stream))
+        _launch(tokens.device, lib.ascan_forward_from, gates.data_ptr(), tokens.data_ptr(), initial.data_ptr(),
+                out.data_ptr(), rows, seqlen, code, 1 if reverse else 0, _ptr(workspace),
+                workspace.numel() if workspace is not None else 0)
     elif workspace is None:
-        _launch(tokens.device, lambda stream: lib.ascan_forward(
-            gates.data_ptr(), tokens.data_ptr(), out.data_ptr(), rows, seqlen, code, 1 if reverse else 0, stream))
+        _launch(tokens.device, lib.ascan_forward, gates.data_ptr(), tokens.data_ptr(), out.data_ptr(), rows,
+                seqlen, code, 1 if reverse else 0)
     else:
-        _launch(tokens.device, lambda stream: lib.ascan_forward_split(
-            gates.data_ptr(), tokens.data_ptr(), out.data_ptr(), rows, seqlen, code, 1 if reverse else 0,
-            workspace.data_ptr(), workspace.numel(), stream))
+        _launch(tokens.device, lib.ascan_forward_split, gates.data_ptr(), tokens.data_ptr(), out.data_ptr(), rows,
+                seqlen, code, 1 if reverse else 0, workspace.data_ptr(), workspace.numel())
 
 
 def backward(gates, states, grad_out, d_gates, d_tokens, workspace=None, initial=None, d_initial=None) -> None:
@@ -238,63 +250,47 @@ def backward(gates, states, grad_out, d_gates, d_tokens, workspace=None, initial
     ``initial`` is the state the forward scan started from; ``d_initial``
     receives its gradient (left untouched for an empty sequence)."""
     lib = _lib or load()
-    seqlen = gates.shape[-1]
-    rows = gates.numel() // seqlen if seqlen else 0
-    code = dtype_code(gates.dtype, d_tokens.dtype)
-    if workspace is None:
-        workspace = _workspace(lib, rows, seqlen, code, gates.device)
+    rows, seqlen, code = _problem(gates, d_tokens)
+    if workspace is None and _workspace_bytes(rows, seqlen, code):
+        workspace = _workspace(rows, seqlen, code, gates.device)
     if initial is not None or d_initial is not None:
         _check_state(initial, states, "initial")
         _check_state(d_initial, states, "d_initial")
-        _launch(gates.device, lambda stream: lib.ascan_backward_from(
-            gates.data_ptr(), states.data_ptr(), initial.data_ptr() if initial is not None else None,
-            grad_out.data_ptr(), d_gates.data_ptr(), d_tokens.data_ptr(),
-            d_initial.data_ptr() if d_initial is not None else None, rows, seqlen, code,
-            workspace.data_ptr() if workspace is not None else None,
-            workspace.numel() if workspace is not None else 0, stream))
+        _launch(gates.device, lib.ascan_backward_from, gates.data_ptr(), states.data_ptr(), _ptr(initial),
+                grad_out.data_ptr(), d_gates.data_ptr(), d_tokens.data_ptr(), _ptr(d_initial), rows, seqlen, code,
+                _ptr(workspace), workspace.numel() if workspace is not None else 0)
     elif workspace is None:
-        _launch(gates.device, lambda stream: lib.ascan_backward(
-            gates.data_ptr(), states.data_ptr(), grad_out.data_ptr(), d_gates.data_ptr(), d_tokens.data_ptr(),
-            rows, seqlen, code, stream))
+        _launch(gates.device, lib.ascan_backward, gates.data_ptr(), states.data_ptr(), grad_out.data_ptr(),
+                d_gates.data_ptr(), d_tokens.data_ptr(), rows, seqlen, code)
     else:
-        _launch(gates.device, lambda stream: lib.ascan_backward_split(
-            gates.data_ptr(), states.data_ptr(), grad_out.data_ptr(), d_gates.data_ptr(), d_tokens.data_ptr(),
-            rows, seqlen, code, workspace.data_ptr(), workspace.numel(), stream))
-
-
-def _ptr(t):
-    return t.data_ptr() if t is not None else None
+        _launch(gates.device, lib.ascan_backward_split, gates.data_ptr(), states.data_ptr(), grad_out.data_ptr(),
+                d_gates.data_ptr(), d_tokens.data_ptr(), rows, seqlen, code, workspace.data_ptr(), workspace.numel())
 
 
 def forward_gated(gate_inputs, tokens, out, gate: int, workspace=None, initial=None) -> None:
     """Forward scan whose gates are ``gate`` (an ascan_gate code) of ``gate_inputs``."""
     lib = _lib or load()
-    seqlen = tokens.shape[-1]
-    rows = tokens.numel() // seqlen if seqlen else 0
-    code = dtype_code(gate_inputs.dtype, tokens.dtype)
+    rows, seqlen, code = _problem(gate_inputs, tokens)
     if workspace is None:
-        workspace = _workspace(lib, rows, seqlen, code, tokens.device)
+        workspace = _workspace(rows, seqlen, code, tokens.device)
     _check_state(initial, out, "initial")
-    _launch(tokens.device, lambda stream: lib.ascan_forward_gated(
-        gate_inputs.data_ptr(), tokens.data_ptr(), _ptr(initial), out.data_ptr(), rows, seqlen, code, gate,
-        _ptr(workspace), workspace.numel() if workspace is not None else 0, stream))
+    _launch(tokens.device, lib.ascan_forward_gated, gate_inputs.data_ptr(), tokens.data_ptr(), _ptr(initial),
+            out.data_ptr(), rows, seqlen, code, gate, _ptr(workspace),
+            workspace.numel() if workspace is not None else 0)
 
 
 def backward_gated(gate_inputs, states, grad_out, d_gate_inputs, d_tokens, gate: int, workspace=None,
                    initial=None, d_initial=None) -> None:
     """Backward of ``forward_gated``: gradients of the gate inputs, the tokens and the initial state."""
     lib = _lib or load()
-    seqlen = gate_inputs.shape[-1]
-    rows = gate_inputs.numel() // seqlen if seqlen else 0
-    code = dtype_code(gate_inputs.dtype, d_tokens.dtype)
+    rows, seqlen, code = _problem(gate_inputs, d_tokens)
     if workspace is None:
-        workspace = _workspace(lib, rows, seqlen, code, gate_inputs.device)
+        workspace = _workspace(rows, seqlen, code, gate_inputs.device)
     _check_state(initial, states, "initial")
     _check_state(d_initial, states, "d_initial")
-    _launch(gate_inputs.device, lambda stream: lib.ascan_backward_gated(
-        gate_inputs.data_ptr(), states.data_ptr(), _ptr(initial), grad_out.data_ptr(), d_gate_inputs.data_ptr(),
-        d_tokens.data_ptr(), _ptr(d_initial), rows, seqlen, code, gate,
-        _ptr(workspace), workspace.numel() if workspace is not None else 0, stream))
+    _launch(gate_inputs.device, lib.ascan_backward_gated, gate_inputs.data_ptr(), states.data_ptr(), _ptr(initial),
+            grad_out.data_ptr(), d_gate_inputs.data_ptr(), d_tokens.data_ptr(), _ptr(d_initial), rows, seqlen, code,
+            gate, _ptr(workspace), workspace.numel() if workspace is not None else 0)
 
 
 def workspace_timeouts(workspace) -> int:

@@ -16,10 +16,15 @@ timings taken inside the timed region; `cpu_baseline` times the torch tree
 scan (oracle/ref_scan.py, the restatement of the reference's ref.scan) on the
 host cores on a bounded sample of the same workload.
 
+`roofline.device_ceiling` is what a kernel without arithmetic reaches on the
+same buffers with the same read/write mix (tests/native/stream_probe.hip),
+timed after the scan's timed region.
+
 Other workloads: --dtype {fp32,bf16,fp16,c64} --shape B D T.  --sweep FILE runs
-the reference's benchmark grid, one JSON line per point into FILE (the single
-summary line is still printed).  The reference's max-abs-error table is
-tests/precision_table.py.
+the reference's benchmark grid, one JSON line per point into FILE and the same
+points as a Markdown table into FILE.md (the single summary line is still
+printed).  The reference's max-abs-error table is asserted by
+tests/test_precision_gpu.py.
 """
 
 import argparse
@@ -38,10 +43,18 @@ HBM_PEAK_GBPS = 8000.0  # MI355X HBM3E, published peak
 
 # HBM bytes per launch of the backward kernel, from two rocprofv3 --pmc runs
 # (FETCH_SIZE x 2.000 + WRITE_SIZE x 1.000 KiB, factors from a plain copy of
-# known size; summaries in profiles/).
+# known size; summaries in profiles/).  Counters cannot be read from inside
+# this script, so the figure is carried over from those runs, not measured in
+# the run that prints it; `traffic_source` in the output says so.
 MEASURED_TRAFFIC_BYTES = {
-    ((8, 1536, 65536), "fp32"): (4721940 * 2 + 6292153) * 1024,
-    ((8, 1536, 65536), "bf16"): (2366704 * 2 + 3146428) * 1024,
+    ((8, 1536, 65536), "fp32"): (4722009 * 2 + 6292387) * 1024,
+    ((8, 1536, 65536), "bf16"): (2367125 * 2 + 3146775) * 1024,
+}
+TRAFFIC_SOURCE = {
+    ((8, 1536, 65536), "fp32"): "profiles/scan_f32_8x1536x65536_fwd_bwd.md (rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE); "
+                                "not measured in this run",
+    ((8, 1536, 65536), "bf16"): "profiles/scan_bf16_8x1536x65536_fwd_bwd.md (rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE); "
+                                "not measured in this run",
 }
 
 
@@ -118,7 +131,13 @@ def run_workload(shape, dtype_name, steps, warmup):
 
     for i in range(warmup):
         step(i)
-    evs = [[torch.cuda.Event(enable_timing=True) for _ in range(3)] for _ in range(steps)]
+    # HIP events around each kernel, on the stream the kernels are launched on
+    # (torch's current stream).  An event record costs about 5 us of stream time,
+    # which is nothing beside the headline's 4.4 ms step but 3-4 % of a 0.4 ms
+    # one: workloads below 1 GiB per tensor carry them on every fourth step.
+    stride = 1 if nsets == 1 else 4
+    evs = [[torch.cuda.Event(enable_timing=True) for _ in range(3)] if i % stride == 0 else None
+           for i in range(steps)]
     torch.cuda.synchronize()
     t0 = time.perf_counter()
     for i in range(steps):
@@ -126,13 +145,16 @@ def run_workload(shape, dtype_name, steps, warmup):
     torch.cuda.synchronize()
     t1 = time.perf_counter()
 
-    fwd_ms = sum(e[0].elapsed_time(e[1]) for e in evs) / steps
-    bwd_ms = sum(e[1].elapsed_time(e[2]) for e in evs) / steps
+    sampled = [e for e in evs if e is not None]
+    fwd_ms = sum(e[0].elapsed_time(e[1]) for e in sampled) / len(sampled)
+    bwd_ms = sum(e[1].elapsed_time(e[2]) for e in sampled) / len(sampled)
     ms_per_step = (t1 - t0) * 1e3 / steps
     return {
+        "buffers": sets,
         "elems": elems,
         "esize": esize,
         "input_sets": nsets,
+        "event_steps": len(sampled),
         "ms_per_step": ms_per_step,
         "fwd_ms": fwd_ms,
         "bwd_ms": bwd_ms,
@@ -140,6 +162,58 @@ def run_workload(shape, dtype_name, steps, warmup):
         "fwd_gbps": 3 * elems * esize / (fwd_ms * 1e-3) / 1e9,
         "bwd_gbps": 5 * elems * esize / (bwd_ms * 1e-3) / 1e9,
     }
+
+
+def load_stream_probe():
+    """The no-arithmetic streaming kernels (tests/native/stream_probe.hip), or None
+    when the probe library has not been built."""
+    import ctypes
+
+    path = ROOT / "tests" / "native" / "libstream_probe.so"
+    if not path.exists():
+        return None
+    lib = ctypes.CDLL(str(path))
+    lib.stream_probe_launch.restype = ctypes.c_int
+    lib.stream_probe_launch.argtypes = ([ctypes.c_void_p] * 5 + [ctypes.c_int64] * 2 + [ctypes.c_int] * 5
+                                        + [ctypes.c_uint, ctypes.c_void_p])
+    return lib
+
+
+def device_ceiling(shape, dtype_name, bufs, steps=12, warmup=4):
+    """Streams the workload's own buffers (`bufs`: the buffer sets of run_workload) with kernels that do no arithmetic:
+    the backward scan's mix (3 tensors read, 2 written) and the forward scan's
+    (2 read, 1 written), as a linear sweep and as one workgroup walking each
+    row.  Returns GB/s per variant; run outside the scan's timed region."""
+    import torch
+
+    probe = load_stream_probe()
+    if probe is None:
+        return None
+    rows = shape[0] * shape[1]
+    row_bytes = shape[2] * bufs[0][0].element_size()
+    turn = [0]  # like the scan's own steps, successive launches rotate over the buffer sets
+    nbytes = rows * row_bytes
+    stream = torch.cuda.current_stream().cuda_stream
+    out = {"unit": "GB/s",
+           "what": "kernels without arithmetic on the same buffers, 16-byte nontemporal accesses "
+                   "(tests/native/stream_probe.hip): linear = consecutive workgroups move consecutive 16 KiB; "
+                   "row_walk = one 1024-thread workgroup per row in 64 KiB tiles with one barrier per tile, "
+                   "the scan kernels' own order"}
+    for name, reads, writes, pattern in (("3R2W_linear", 3, 2, 0), ("3R2W_row_walk", 3, 2, 2),
+                                         ("2R1W_linear", 2, 1, 0), ("2R1W_row_walk", 2, 1, 2)):
+        def fn():
+            g, x, d, states, d_gates, d_tokens = bufs[turn[0] % len(bufs)]
+            turn[0] += 1
+            rc = probe.stream_probe_launch(g.data_ptr(), states.data_ptr(), d.data_ptr(), d_gates.data_ptr(),
+                                           d_tokens.data_ptr(), rows, row_bytes, reads, writes, pattern, 4, 1, 0, stream)
+            if rc != 0:
+                raise RuntimeError(f"stream probe: status {rc}")
+        if (pattern == 0 and nbytes % (16 * 1024)) or (pattern != 0 and row_bytes % (64 * 1024)):
+            out[name] = None  # the probe covers whole chunks / tiles only
+            continue
+        ms = time_call(fn, steps, warmup)
+        out[name] = (reads + writes) * nbytes / ms / 1e6
+    return out
 
 
 def time_call(fn, steps, warmup):
@@ -174,8 +248,10 @@ def run_sweep(path, steps, warmup):
     from accelerated_scan.warp import scan as warp_scan
 
     device = torch.device("cuda:0")
+    records = []
     with open(path, "w") as f:
         def emit(rec):
+            records.append(rec)
             f.write(json.dumps(rec) + "\n")
             f.flush()
 
@@ -218,6 +294,43 @@ def run_sweep(path, steps, warmup):
         ms = time_call(lambda: torch.autograd.grad(complex_scan(g, x), (g, x), grad_out), steps, warmup)
         rec["train_real_inputs_ms"] = ms
         emit(rec)
+    write_sweep_markdown(records, str(path) + ".md", steps, warmup)
+
+
+def write_sweep_markdown(records, path, steps, warmup):
+    """The sweep as a table: ms per call and algorithmic TB/s (3 tensors forward /
+    reverse, 5 backward, 8 train)."""
+    import subprocess
+
+    try:
+        head = subprocess.run(["git", "-C", str(ROOT), "rev-parse", "--short", "HEAD"], capture_output=True,
+                              text=True, check=True).stdout.strip()
+    except Exception:  # no git on the box, or not a checkout
+        head = "unknown"
+    def cell(rec, key):
+        if f"{key}_ms" not in rec:
+            return "—"
+        return f"{rec[f'{key}_ms']:.4f} ({rec[f'{key}_GBps'] / 1e3:.2f})"
+
+    with open(path, "w") as f:
+        f.write("# Scan sweep on MI355X: the reference's benchmark grid (tests/bench.py:14-31 of the reference)\n\n")
+        f.write(f"Generated by `python bench.py --sweep FILE` (source revision {head}; mean of {steps} calls after "
+                f"{warmup} warm-up calls, HIP events; one set of buffers per point, so tensors up to a few hundred MB "
+                "see some Infinity Cache hits). Cells: ms per call (algorithmic TB/s). forward / reverse / backward "
+                "are kernel calls through the C ABI; train = autograd forward + backward of `warp.scan`, "
+                "allocation included.\n")
+        for dt in ("fp32", "bf16"):
+            f.write(f"\n## {dt}, shape (8, 1536, T)\n\n| T | forward | reverse | backward | train |\n|---|---|---|---|---|\n")
+            for rec in records:
+                if rec["dtype"] == dt:
+                    f.write(f"| {rec['shape'][2]} | {cell(rec, 'forward')} | {cell(rec, 'reverse')} | "
+                            f"{cell(rec, 'backward')} | {cell(rec, 'train')} |\n")
+        for rec in records:
+            if rec["dtype"] == "c64":
+                f.write(f"\n## complex64, shape {tuple(rec['shape'])} (tests/bench_complex.py:79-90 of the reference)\n\n"
+                        f"forward + backward through the C ABI: {rec['forward_backward_ms']:.4f} ms "
+                        f"({rec['forward_backward_GBps'] / 1e3:.2f} TB/s); autograd forward + backward with real "
+                        f"inputs: {rec['train_real_inputs_ms']:.4f} ms\n")
 
 
 def cpu_baseline(shape, dtype_name):
@@ -283,11 +396,13 @@ def main():
         for _ in range(3):
             dst.copy_(src)
         torch.cuda.synchronize()
-        run_workload(shape, args.dtype, 3, 0)
+        m = run_workload(shape, args.dtype, 3, 0)
+        device_ceiling(shape, args.dtype, m["buffers"], steps=3, warmup=0)  # the probe kernels, for the same counters
         print(json.dumps({"calibration_copy_bytes_read": src.numel() * 4, "calibration_copy_bytes_written":
                           src.numel() * 4, "workload_shape": list(shape), "dtype": args.dtype}))
         return 0
     m = run_workload(shape, args.dtype, args.steps, args.warmup)
+    ceiling = device_ceiling(shape, args.dtype, m.pop("buffers"))
 
     if args.sweep:
         run_sweep(args.sweep, max(5, args.steps), args.warmup)
@@ -314,6 +429,7 @@ def main():
                 "gates r*exp(i*theta) with r ~ 0.9+0.1*U(0,1), tokens and grad_out complex N(0,1)"
                 if args.dtype == "c64" else "gates 0.999+0.001*U(0,1), tokens U(0,1), grad_out N(0,1)"),
             "input_sets": m["input_sets"],
+            "steps_with_kernel_events": m["event_steps"],
             "fwd_ms": m["fwd_ms"],
             "bwd_ms": m["bwd_ms"],
             "fwd_GBps": m["fwd_gbps"],
@@ -330,6 +446,8 @@ def main():
             "algorithmic_bytes_per_launch": bwd_bytes,
             "avg_launch_ms": m["bwd_ms"],
             "traffic": MEASURED_TRAFFIC_BYTES.get((shape, args.dtype)),
+            "traffic_source": TRAFFIC_SOURCE.get((shape, args.dtype)),
+            "device_ceiling": ceiling,
         },
     }
     if not args.no_cpu_baseline:

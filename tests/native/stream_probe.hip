@@ -1,0 +1,162 @@
+// Streaming probe for MI355X (gfx950): kernels that move the same bytes as the
+// scan kernels, with the same 16-byte nontemporal accesses, and do no
+// arithmetic worth the name.  What they reach is what the memory system
+// delivers for a given mix of reads and writes and a given order of access;
+// bench.py reports it beside the scan's own figure as the device ceiling.
+// Measurement infrastructure: nothing in the library depends on it.
+//
+//   pattern 0  linear sweep: workgroup i moves the i-th 16 KiB of every tensor
+//              (consecutive workgroups touch consecutive memory);
+//   pattern 1  row walk: one 1024-thread workgroup per row, walking the row in
+//              tiles of 64 KiB (16 waves x 4 KiB), as the scan kernels do for
+//              long rows, without their barrier;
+//   pattern 2  row walk with one workgroup barrier per tile;
+//   pattern 3  linear sweep in the row walk's units: workgroup i moves the i-th
+//              tile of every tensor (barrier) and ends.
+// `blocks_per_wave` in {1, 2, 4, 8} sets the tile of patterns 1-3: that many KiB
+// per wave, 16 times as much per workgroup (the scan kernels: 4, 64 KiB tiles).
+// `row_step` > 1 (patterns 1, 2) hands consecutive workgroups rows that far apart.
+// `lds_bytes` of dynamic LDS are requested per workgroup (nothing uses them):
+// more than half a compute unit's LDS keeps workgroups from sharing one.
+//
+// `reads` of the three inputs are read and `writes` of the two outputs are
+// written; every tensor is rows x row_bytes bytes, dense.
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace {
+
+typedef unsigned int u32x4_t __attribute__((ext_vector_type(4)));
+
+constexpr int kThreads = 1024;
+constexpr int64_t kChunk = (int64_t)kThreads * 16;  // bytes one workgroup moves per tensor in one go
+// row walk: a wave moves BPW KiB of every tensor per tile (the scan kernels: 4)
+constexpr int64_t tile_bytes(int bpw) { return (int64_t)kThreads * 16 * bpw; }
+
+struct Tensors {
+    const u32x4_t* in[3];
+    u32x4_t* out[2];
+};
+
+// Read-only probes: a store that the data never triggers keeps the loads alive.
+__device__ __forceinline__ void keep(u32x4_t s, u32x4_t* where) {
+    if ((s.x ^ s.y ^ s.z ^ s.w) == 0x9e3779b9u && s.x == 0x7f4a7c15u) *where = s;
+}
+
+template <int NR, int NW>
+__global__ void __launch_bounds__(kThreads) stream_probe_linear(Tensors t) {
+    const int64_t v = (int64_t)blockIdx.x * kThreads + threadIdx.x;  // vector index
+    u32x4_t s = {1u, 2u, 3u, 4u};
+#pragma unroll
+    for (int r = 0; r < NR; ++r) s += __builtin_nontemporal_load(t.in[r] + v);
+#pragma unroll
+    for (int w = 0; w < NW; ++w) __builtin_nontemporal_store(s + (unsigned)w, t.out[w] + v);
+    if constexpr (NW == 0) keep(s, t.out[0] + v);
+}
+
+template <int NR, int NW, bool BARRIER, int BPW>
+__global__ void __launch_bounds__(kThreads) stream_probe_rows(Tensors t, int64_t row_vectors, int row_step) {
+    constexpr int kBlocksPerWave = BPW;
+    constexpr int64_t kTile = tile_bytes(BPW);
+    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    // one row per workgroup; with row_vectors == one tile, the launch is a linear sweep in tiles.
+    // row_step > 1: consecutive workgroups take rows row_step apart (all rows are still covered)
+    const int64_t per_pass = gridDim.x / row_step;
+    const int64_t row_index = row_step > 1 ? (blockIdx.x % per_pass) * row_step + blockIdx.x / per_pass : blockIdx.x;
+    const int64_t row = row_index * row_vectors;
+    for (int64_t tile = 0; tile < row_vectors; tile += kTile / 16) {
+        const int64_t base = row + tile + (int64_t)wave * (64 * kBlocksPerWave) + lane;
+        u32x4_t s[kBlocksPerWave];
+#pragma unroll
+        for (int j = 0; j < kBlocksPerWave; ++j) {
+            s[j] = u32x4_t{1u, 2u, 3u, 4u};
+#pragma unroll
+            for (int r = 0; r < NR; ++r) s[j] += __builtin_nontemporal_load(t.in[r] + base + j * 64);
+        }
+        if constexpr (BARRIER) __syncthreads();
+#pragma unroll
+        for (int j = 0; j < kBlocksPerWave; ++j) {
+#pragma unroll
+            for (int w = 0; w < NW; ++w) __builtin_nontemporal_store(s[j] + (unsigned)w, t.out[w] + base + j * 64);
+            if constexpr (NW == 0) keep(s[j], t.out[0] + base + j * 64);
+        }
+    }
+}
+
+template <class K>
+hipError_t allow_lds(K kernel, unsigned lds_bytes) {
+    if (lds_bytes <= 64u * 1024u) return hipSuccess;
+    return hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
+                               (int)lds_bytes);
+}
+
+template <int NR, int NW, int BPW>
+hipError_t launch_rows(const Tensors& t, int64_t rows, int64_t row_bytes, int pattern, int row_step,
+                       unsigned lds_bytes, hipStream_t stream) {
+    hipError_t e = pattern == 1 ? allow_lds(stream_probe_rows<NR, NW, false, BPW>, lds_bytes)
+                                : allow_lds(stream_probe_rows<NR, NW, true, BPW>, lds_bytes);
+    if (e != hipSuccess) return e;
+    if (pattern == 1) {
+        hipLaunchKernelGGL((stream_probe_rows<NR, NW, false, BPW>), dim3((unsigned)rows), dim3(kThreads), lds_bytes,
+                           stream, t, row_bytes / 16, row_step);
+    } else if (pattern == 2) {
+        hipLaunchKernelGGL((stream_probe_rows<NR, NW, true, BPW>), dim3((unsigned)rows), dim3(kThreads), lds_bytes,
+                           stream, t, row_bytes / 16, row_step);
+    } else {
+        const int64_t tiles = rows * row_bytes / tile_bytes(BPW);
+        hipLaunchKernelGGL((stream_probe_rows<NR, NW, true, BPW>), dim3((unsigned)tiles), dim3(kThreads), lds_bytes,
+                           stream, t, tile_bytes(BPW) / 16, 1);
+    }
+    return hipGetLastError();
+}
+
+template <int NR, int NW>
+hipError_t launch(const Tensors& t, int64_t rows, int64_t row_bytes, int pattern, int bpw, int row_step,
+                  unsigned lds_bytes, hipStream_t stream) {
+    if (pattern == 0) {
+        const hipError_t e = allow_lds(stream_probe_linear<NR, NW>, lds_bytes);
+        if (e != hipSuccess) return e;
+        const int64_t blocks = rows * row_bytes / kChunk;
+        hipLaunchKernelGGL((stream_probe_linear<NR, NW>), dim3((unsigned)blocks), dim3(kThreads), lds_bytes, stream, t);
+        return hipGetLastError();
+    }
+    switch (bpw) {
+        case 1: return launch_rows<NR, NW, 1>(t, rows, row_bytes, pattern, row_step, lds_bytes, stream);
+        case 2: return launch_rows<NR, NW, 2>(t, rows, row_bytes, pattern, row_step, lds_bytes, stream);
+        case 8: return launch_rows<NR, NW, 8>(t, rows, row_bytes, pattern, row_step, lds_bytes, stream);
+        default: return launch_rows<NR, NW, 4>(t, rows, row_bytes, pattern, row_step, lds_bytes, stream);
+    }
+}
+
+}  // namespace
+
+// Returns 0, -1 for arguments the kernels do not cover, or a hipError_t.
+extern "C" __attribute__((visibility("default"))) int stream_probe_launch(
+    const void* in0, const void* in1, const void* in2, void* out0, void* out1, int64_t rows, int64_t row_bytes,
+    int reads, int writes, int pattern, int blocks_per_wave, int row_step, unsigned lds_bytes, void* stream) {
+    if (row_step < 1 || rows % row_step != 0) return -1;
+    if (rows <= 0 || row_bytes <= 0 || pattern < 0 || pattern > 3 || lds_bytes > 160u * 1024u) return -1;
+    if (blocks_per_wave != 1 && blocks_per_wave != 2 && blocks_per_wave != 4 && blocks_per_wave != 8) return -1;
+    if (pattern == 0 ? (rows * row_bytes) % kChunk != 0 : row_bytes % tile_bytes(blocks_per_wave) != 0) return -1;
+    if (rows * row_bytes / kChunk > 2147483647LL || rows > 2147483647LL) return -1;
+    const void* ins[3] = {in0, in1, in2};
+    void* outs[2] = {out0, out1};
+    for (int r = 0; r < reads; ++r)
+        if (r >= 3 || !ins[r] || reinterpret_cast<uintptr_t>(ins[r]) % 16) return -1;
+    for (int w = 0; w < (writes > 0 ? writes : 1); ++w)  // read-only probes still name out0 (never written)
+        if (w >= 2 || !outs[w] || reinterpret_cast<uintptr_t>(outs[w]) % 16) return -1;
+    Tensors t;
+    for (int r = 0; r < 3; ++r) t.in[r] = static_cast<const u32x4_t*>(ins[r]);
+    for (int w = 0; w < 2; ++w) t.out[w] = static_cast<u32x4_t*>(outs[w]);
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    const int mix = reads * 10 + writes;
+    switch (mix) {
+        case 32: return (int)launch<3, 2>(t, rows, row_bytes, pattern, blocks_per_wave, row_step, lds_bytes, s);
+        case 21: return (int)launch<2, 1>(t, rows, row_bytes, pattern, blocks_per_wave, row_step, lds_bytes, s);
+        case 11: return (int)launch<1, 1>(t, rows, row_bytes, pattern, blocks_per_wave, row_step, lds_bytes, s);
+        case 30: return (int)launch<3, 0>(t, rows, row_bytes, pattern, blocks_per_wave, row_step, lds_bytes, s);
+        case 2: return (int)launch<0, 2>(t, rows, row_bytes, pattern, blocks_per_wave, row_step, lds_bytes, s);
+        default: return -1;
+    }
+}
