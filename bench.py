@@ -300,13 +300,14 @@ def run_sweep(path, steps, warmup):
 def write_sweep_markdown(records, path, steps, warmup):
     """The sweep as a table: ms per call and algorithmic TB/s (3 tensors forward /
     reverse, 5 backward, 8 train)."""
-    import subprocess
+    import hashlib
 
-    try:
-        head = subprocess.run(["git", "-C", str(ROOT), "rev-parse", "--short", "HEAD"], capture_output=True,
-                              text=True, check=True).stdout.strip()
-    except Exception:  # no git on the box, or not a checkout
-        head = "unknown"
+    # identifies the kernels measured wherever the file is written (the GPU box has no git checkout):
+    # sha1 over the library's sources in name order
+    digest = hashlib.sha1()
+    for src in sorted(list((ROOT / "accelerated-scan_amd" / "csrc").glob("*.h*")) + [ROOT / "include" / "ascan.h"]):
+        digest.update(src.name.encode() + b"\0" + src.read_bytes())
+    head = digest.hexdigest()[:12]
     def cell(rec, key):
         if f"{key}_ms" not in rec:
             return "—"
@@ -314,7 +315,7 @@ def write_sweep_markdown(records, path, steps, warmup):
 
     with open(path, "w") as f:
         f.write("# Scan sweep on MI355X: the reference's benchmark grid (tests/bench.py:14-31 of the reference)\n\n")
-        f.write(f"Generated by `python bench.py --sweep FILE` (source revision {head}; mean of {steps} calls after "
+        f.write(f"Generated by `python bench.py --sweep FILE` (sha1 of csrc/* and include/ascan.h in name order: {head}; mean of {steps} calls after "
                 f"{warmup} warm-up calls, HIP events; one set of buffers per point, so tensors up to a few hundred MB "
                 "see some Infinity Cache hits). Cells: ms per call (algorithmic TB/s). forward / reverse / backward "
                 "are kernel calls through the C ABI; train = autograd forward + backward of `warp.scan`, "
