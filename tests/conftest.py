@@ -18,8 +18,18 @@ def pytest_sessionstart(session):
     none is there at all are they built here, so that a fresh checkout can run."""
     import subprocess
 
-    if not (ROOT / "accelerated-scan_amd" / "accelerated_scan" / "libascan.so").exists():
+    library = ROOT / "accelerated-scan_amd" / "accelerated_scan" / "libascan.so"
+    if not library.exists():
         subprocess.run(["make", "-j8", "-C", str(ROOT / "accelerated-scan_amd")], check=True, capture_output=True)
+    else:
+        # a library older than its sources is tested as it is, but not silently
+        sources = list((ROOT / "accelerated-scan_amd" / "csrc").glob("*")) + [ROOT / "include" / "ascan.h"]
+        newer = [p.name for p in sources if p.stat().st_mtime > library.stat().st_mtime]
+        if newer:
+            import warnings
+
+            warnings.warn(f"libascan.so is older than {', '.join(sorted(newer))}: run `make -C accelerated-scan_amd` "
+                          "(or __graft_entry__.build()) to test the current sources")
     if not (ROOT / "oracle" / "_build" / "libseqscan.so").exists():
         subprocess.run(["make", "-C", str(ROOT / "oracle")], check=True, capture_output=True)
 
