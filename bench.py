@@ -61,8 +61,10 @@ TRAFFIC_SOURCE = {
 def parse_args():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=20)
-    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--steps", type=int, default=None,
+                    help="timed steps (default 20; 200 for workloads below 1 GiB per tensor)")
+    ap.add_argument("--warmup", type=int, default=None,
+                    help="untimed warm-up steps (default 5; 100 for workloads below 1 GiB per tensor)")
     ap.add_argument("--dtype", choices=["fp32", "bf16", "fp16", "c64"], default="fp32")
     ap.add_argument("--shape", type=int, nargs=3, default=[8, 1536, 65536], metavar=("B", "D", "T"))
     ap.add_argument("--no-cpu-baseline", action="store_true")
@@ -211,26 +213,37 @@ def device_ceiling(shape, dtype_name, bufs, steps=12, warmup=4):
         if (pattern == 0 and nbytes % (16 * 1024)) or (pattern != 0 and row_bytes % (64 * 1024)):
             out[name] = None  # the probe covers whole chunks / tiles only
             continue
-        ms = time_call(fn, steps, warmup)
+        ms = time_call(fn, steps, warmup, min_ms=30.0)
         out[name] = (reads + writes) * nbytes / ms / 1e6
     return out
 
 
-def time_call(fn, steps, warmup):
-    """Mean milliseconds per call of fn() from HIP events on the current stream."""
+def time_call(fn, steps, warmup, min_ms=0.0):
+    """Mean milliseconds per call of fn() from HIP events on the current stream.
+    With min_ms, short calls are repeated until the timed region lasts about that
+    long (and the warm-up half as long): a handful of microsecond-sized launches
+    is over before the clocks have settled."""
     import torch
+
+    def timed(n):
+        start = torch.cuda.Event(enable_timing=True)
+        stop = torch.cuda.Event(enable_timing=True)
+        torch.cuda.synchronize()
+        start.record()
+        for _ in range(n):
+            fn()
+        stop.record()
+        torch.cuda.synchronize()
+        return start.elapsed_time(stop) / n
 
     for _ in range(warmup):
         fn()
-    start = torch.cuda.Event(enable_timing=True)
-    stop = torch.cuda.Event(enable_timing=True)
-    torch.cuda.synchronize()
-    start.record()
-    for _ in range(steps):
-        fn()
-    stop.record()
-    torch.cuda.synchronize()
-    return start.elapsed_time(stop) / steps
+    per_call = timed(steps)
+    if min_ms > 0.0 and per_call * steps < min_ms:
+        n = min(20000, int(min_ms / max(per_call, 1e-4)) + 1)
+        timed(n // 2)
+        per_call = timed(n)
+    return per_call
 
 
 def run_sweep(path, steps, warmup):
@@ -248,6 +261,7 @@ def run_sweep(path, steps, warmup):
     from accelerated_scan.warp import scan as warp_scan
 
     device = torch.device("cuda:0")
+    min_ms = 40.0  # each point: at least 20 ms of warm-up and 40 ms timed (the reference warms up for seconds per point)
     records = []
     with open(path, "w") as f:
         def emit(rec):
@@ -262,17 +276,17 @@ def run_sweep(path, steps, warmup):
                 out, d_gates, d_tokens = (torch.empty_like(tokens) for _ in range(3))
                 nbytes = tokens.numel() * tokens.element_size()
                 rec = {"dtype": dt, "shape": list(shape)}
-                ms = time_call(lambda: _abi.forward(gates, tokens, out, False), steps, warmup)
+                ms = time_call(lambda: _abi.forward(gates, tokens, out, False), steps, warmup, min_ms)
                 rec["forward_ms"], rec["forward_GBps"] = ms, 3 * nbytes / ms / 1e6
-                ms = time_call(lambda: _abi.forward(gates, tokens, out, True), steps, warmup)
+                ms = time_call(lambda: _abi.forward(gates, tokens, out, True), steps, warmup, min_ms)
                 rec["reverse_ms"], rec["reverse_GBps"] = ms, 3 * nbytes / ms / 1e6
                 _abi.forward(gates, tokens, out, False)
-                ms = time_call(lambda: _abi.backward(gates, out, grad_out, d_gates, d_tokens), steps, warmup)
+                ms = time_call(lambda: _abi.backward(gates, out, grad_out, d_gates, d_tokens), steps, warmup, min_ms)
                 rec["backward_ms"], rec["backward_GBps"] = ms, 5 * nbytes / ms / 1e6
                 if T <= 16384:
                     g = gates.clone().requires_grad_(True)
                     x = tokens.clone().requires_grad_(True)
-                    ms = time_call(lambda: torch.autograd.grad(warp_scan(g, x), (g, x), grad_out), steps, warmup)
+                    ms = time_call(lambda: torch.autograd.grad(warp_scan(g, x), (g, x), grad_out), steps, warmup, min_ms)
                     rec["train_ms"], rec["train_GBps"] = ms, 8 * nbytes / ms / 1e6
                 emit(rec)
                 del gates, tokens, grad_out, out, d_gates, d_tokens
@@ -286,12 +300,12 @@ def run_sweep(path, steps, warmup):
             _abi.forward(gates, tokens, out, False)
             _abi.backward(gates, out, grad_out, d_gates, d_tokens)
 
-        ms = time_call(both, steps, warmup)
+        ms = time_call(both, steps, warmup, min_ms)
         rec = {"dtype": "c64", "shape": list(shape), "forward_backward_ms": ms,
                "forward_backward_GBps": 8 * nbytes / ms / 1e6}
         g = gates.clone().requires_grad_(True)
         x = tokens.real.contiguous().requires_grad_(True)  # real inputs, as the reference's complex bench
-        ms = time_call(lambda: torch.autograd.grad(complex_scan(g, x), (g, x), grad_out), steps, warmup)
+        ms = time_call(lambda: torch.autograd.grad(complex_scan(g, x), (g, x), grad_out), steps, warmup, min_ms)
         rec["train_real_inputs_ms"] = ms
         emit(rec)
     write_sweep_markdown(records, str(path) + ".md", steps, warmup)
@@ -315,8 +329,8 @@ def write_sweep_markdown(records, path, steps, warmup):
 
     with open(path, "w") as f:
         f.write("# Scan sweep on MI355X: the reference's benchmark grid (tests/bench.py:14-31 of the reference)\n\n")
-        f.write(f"Generated by `python bench.py --sweep FILE` (sha1 of csrc/* and include/ascan.h in name order: {head}; mean of {steps} calls after "
-                f"{warmup} warm-up calls, HIP events; one set of buffers per point, so tensors up to a few hundred MB "
+        f.write(f"Generated by `python bench.py --sweep FILE` (sha1 of csrc/* and include/ascan.h in name order: {head}; mean over at "
+                f"least {steps} calls and 40 ms after at least {warmup} calls and 20 ms of warm-up, HIP events; one set of buffers per point, so tensors up to a few hundred MB "
                 "see some Infinity Cache hits). Cells: ms per call (algorithmic TB/s). forward / reverse / backward "
                 "are kernel calls through the C ABI; train = autograd forward + backward of `warp.scan`, "
                 "allocation included.\n")
@@ -391,6 +405,15 @@ def main():
     _abi.load()  # no fallback: fail here if the HIP library is missing
 
     shape = tuple(args.shape)
+    # Sub-millisecond steps need a longer run: with 5 + 20 steps of 0.4 ms the whole measurement is over in 10 ms,
+    # before clocks and caches have settled (measured at (4,1024,8192) complex64: 68.4 % of peak with 5 + 20 steps,
+    # 72.2 % with 100 + 200).  The headline's defaults are the driver's: 5 + 20 steps of 4.4 ms.
+    tensor_bytes = shape[0] * shape[1] * shape[2] * {"fp32": 4, "bf16": 2, "fp16": 2, "c64": 8}[args.dtype]
+    small = tensor_bytes < (1 << 30)
+    if args.steps is None:
+        args.steps = 200 if small else 20
+    if args.warmup is None:
+        args.warmup = 100 if small else 5
     if args.pmc_calibration:
         src = torch.rand(1 << 28, device="cuda:0")  # 1 GiB of fp32
         dst = torch.empty_like(src)
@@ -406,7 +429,7 @@ def main():
     ceiling = device_ceiling(shape, args.dtype, m.pop("buffers"))
 
     if args.sweep:
-        run_sweep(args.sweep, max(5, args.steps), args.warmup)
+        run_sweep(args.sweep, 20, 5)
 
     dtype_field = {"fp32": "f32", "bf16": "bf16 storage, f32 arithmetic",
                    "fp16": "f16 storage, f32 arithmetic", "c64": "complex64 (f32 pairs)"}[args.dtype]
