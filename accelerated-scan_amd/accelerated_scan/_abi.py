@@ -13,10 +13,10 @@ from pathlib import Path
 
 import torch
 
-ABI_VERSION = 5
+ABI_VERSION = 6
 
 # ascan_gate codes of include/ascan.h
-GATE_IDENTITY, GATE_SIGMOID = 0, 1
+GATE_IDENTITY, GATE_SIGMOID, GATE_SIGMOID_LERP = 0, 1, 2
 
 # ascan_dtype codes of include/ascan.h
 F32, BF16, F16, C64, C64_REAL_TOKENS = 0, 1, 2, 3, 4
@@ -83,6 +83,13 @@ _SIGNATURES = {
         [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p,
          ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p,
          ctypes.c_int64, ctypes.c_int64, ctypes.c_int, ctypes.c_int,
+         ctypes.c_void_p, ctypes.c_size_t, ctypes.c_void_p],
+    ),
+    "ascan_backward_lerp": (
+        ctypes.c_int,
+        [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p,
+         ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p,
+         ctypes.c_int64, ctypes.c_int64, ctypes.c_int,
          ctypes.c_void_p, ctypes.c_size_t, ctypes.c_void_p],
     ),
     "ascan_status_string": (ctypes.c_char_p, [ctypes.c_int]),
@@ -291,6 +298,21 @@ def backward_gated(gate_inputs, states, grad_out, d_gate_inputs, d_tokens, gate:
     _launch(gate_inputs.device, lib.ascan_backward_gated, gate_inputs.data_ptr(), states.data_ptr(), _ptr(initial),
             grad_out.data_ptr(), d_gate_inputs.data_ptr(), d_tokens.data_ptr(), _ptr(d_initial), rows, seqlen, code,
             gate, _ptr(workspace), workspace.numel() if workspace is not None else 0)
+
+
+def backward_lerp(gate_inputs, values, states, grad_out, d_gate_inputs, d_values, workspace=None,
+                  initial=None, d_initial=None) -> None:
+    """Backward of ``forward_gated(..., GATE_SIGMOID_LERP)``: gradients of the gate inputs, the values and
+    the initial state of x[t] = a x[t-1] + (1 - a) values[t], a = sigmoid(gate_inputs)."""
+    lib = _lib or load()
+    rows, seqlen, code = _problem(gate_inputs, d_values)
+    if workspace is None:
+        workspace = _workspace(rows, seqlen, code, gate_inputs.device)
+    _check_state(initial, states, "initial")
+    _check_state(d_initial, states, "d_initial")
+    _launch(gate_inputs.device, lib.ascan_backward_lerp, gate_inputs.data_ptr(), values.data_ptr(), states.data_ptr(),
+            _ptr(initial), grad_out.data_ptr(), d_gate_inputs.data_ptr(), d_values.data_ptr(), _ptr(d_initial), rows,
+            seqlen, code, _ptr(workspace), workspace.numel() if workspace is not None else 0)
 
 
 def workspace_timeouts(workspace) -> int:

@@ -9,6 +9,14 @@ Against the unfused pair of calls that saves the sigmoid's forward pass (one
 read, one write), its backward pass (two reads, one write) and the saved gates
 tensor.
 
+``sigmoid_lerp_scan(gate_logits, values)`` solves the gated interpolation
+``x[t] = a[t] * x[t-1] + (1 - a[t]) * values[t]`` with ``a = sigmoid(gate_logits)``
+-- ``x[t] = torch.lerp(values[t], x[t-1], a[t])`` -- in which the tokens
+``(1 - a) * values`` never exist in memory either: the forward kernel reads
+logits and values (2 tensors in, 1 out, where the unfused sequence of sigmoid,
+multiply and scan moves 9), the backward kernel reads logits, values, states
+and the incoming gradient and writes both gradients (4 in, 2 out, against 21).
+
 The reference's ``scan`` takes finished gates (accelerated_scan/warp.py:68-83);
 the linear-RNN layers that call it (README.md:8,42 of the reference) typically
 compute them with a sigmoid just before the scan.
@@ -83,3 +91,48 @@ def sigmoid_scan(gate_logits, tokens, initial=None):
     if initial is None:
         initial = torch.zeros(gate_logits.shape[:-1], dtype=gate_logits.dtype, device=gate_logits.device)
     return SigmoidScan.apply(gate_logits, tokens, initial)
+
+
+class SigmoidLerpScan(torch.autograd.Function):
+    """Autograd node of the gated interpolation: saves (gate_logits, values, states, initial)."""
+
+    @staticmethod
+    def forward(ctx, gate_logits, values, initial):
+        _check(gate_logits, values, initial)
+        initial = initial.contiguous()
+        if _ops.capturing():
+            states = _ops.scan_forward_gated(gate_logits, values, initial, _abi.GATE_SIGMOID_LERP)
+        else:
+            states = torch.empty_like(gate_logits)
+            _abi.forward_gated(gate_logits, values, states, _abi.GATE_SIGMOID_LERP, initial=initial)
+        ctx.save_for_backward(gate_logits, values, states, initial)
+        return states
+
+    @staticmethod
+    def backward(ctx, grad_output):
+        gate_logits, values, states, initial = ctx.saved_tensors
+        grad_output = grad_output.contiguous()
+        if _ops.capturing():
+            return _ops.scan_backward_lerp(gate_logits, values, states, initial, grad_output)
+        d_logits = torch.empty_like(gate_logits)
+        d_values = torch.empty_like(gate_logits)
+        d_initial = torch.zeros_like(initial)  # stays zero for an empty sequence
+        _abi.backward_lerp(gate_logits, values, states, grad_output, d_logits, d_values, initial=initial,
+                           d_initial=d_initial)
+        return d_logits, d_values, d_initial
+
+
+def sigmoid_lerp_scan(gate_logits, values, initial=None):
+    """Solve ``x[t] = a[t] * x[t-1] + (1 - a[t]) * values[t]`` with ``a = sigmoid(gate_logits)``.
+
+    Arguments:
+        gate_logits (torch.Tensor): shape (B, C, T), contiguous; fp32, bf16 or fp16.
+        values (torch.Tensor): shape (B, C, T), contiguous, same dtype.
+        initial (torch.Tensor, optional): shape (B, C), the state ``x[-1]`` (zero if absent).
+
+    Returns:
+        (torch.Tensor): the states, shape (B, C, T); differentiable in all arguments.
+    """
+    if initial is None:
+        initial = torch.zeros(gate_logits.shape[:-1], dtype=gate_logits.dtype, device=gate_logits.device)
+    return SigmoidLerpScan.apply(gate_logits, values, initial)

@@ -125,8 +125,12 @@ constexpr int64_t kMaxBlocks = 2147483647LL;
 
 bool activation_supported(int act, int dtype, bool reverse) {
     if (act == ASCAN_GATE_IDENTITY) return true;
-    return act == ASCAN_GATE_SIGMOID && !reverse && (dtype == ASCAN_F32 || dtype == ASCAN_BF16 || dtype == ASCAN_F16);
+    return (act == ASCAN_GATE_SIGMOID || act == ASCAN_GATE_SIGMOID_LERP) && !reverse &&
+           (dtype == ASCAN_F32 || dtype == ASCAN_BF16 || dtype == ASCAN_F16);
 }
+static_assert(ASCAN_GATE_IDENTITY == kGateIdentity && ASCAN_GATE_SIGMOID == kGateSigmoid &&
+                  ASCAN_GATE_SIGMOID_LERP == kGateSigmoidLerp,
+              "the kernels' gate codes are the ABI's");
 
 int forward_checked(const void* gates, const void* tokens, void* out, const void* initial, int64_t rows,
                     int64_t seqlen, int dtype, int reverse, int act, const Workspace& ws, void* stream) {
@@ -156,29 +160,31 @@ int forward_checked(const void* gates, const void* tokens, void* out, const void
     }
 }
 
+// `values` is the fourth input of the interpolating gate and null for every other gate.
 int backward_checked(const void* gates, const void* states, const void* grad_out, void* d_gates, void* d_tokens,
-                     const void* initial, void* d_initial, int64_t rows, int64_t seqlen, int dtype, int act,
-                     const Workspace& ws, void* stream) {
+                     const void* initial, void* d_initial, const void* values, int64_t rows, int64_t seqlen,
+                     int dtype, int act, const Workspace& ws, void* stream) {
     const size_t es = element_size(dtype);
     if (es == 0) return ASCAN_ERR_BAD_DTYPE;
     if (!activation_supported(act, dtype, false)) return ASCAN_ERR_BAD_ACTIVATION;
     if (rows < 0 || seqlen < 0 || rows > kMaxBlocks) return ASCAN_ERR_BAD_SHAPE;
     if (rows == 0 || seqlen == 0) return ASCAN_OK;
     if (!gates || !states || !grad_out || !d_gates || !d_tokens) return ASCAN_ERR_NULL_POINTER;
+    if (act == ASCAN_GATE_SIGMOID_LERP && !values) return ASCAN_ERR_NULL_POINTER;
     if (!element_aligned(gates, es) || !element_aligned(states, es) || !element_aligned(grad_out, es) ||
         !element_aligned(d_gates, es) || !element_aligned(d_tokens, token_size(dtype)) ||
-        !element_aligned(initial, es) || !element_aligned(d_initial, es))
+        !element_aligned(initial, es) || !element_aligned(d_initial, es) || !element_aligned(values, es))
         return ASCAN_ERR_MISALIGNED;
     {
         const int64_t n = rows * seqlen;
         const Span inputs[] = {span_of(gates, n, es), span_of(states, n, es), span_of(grad_out, n, es),
-                               span_of(initial, rows, es)};
+                               span_of(initial, rows, es), span_of(values, n, es)};
         const Span outputs[] = {span_of(d_gates, n, es), span_of(d_tokens, n, token_size(dtype)),
                                 span_of(d_initial, rows, es)};
         if (outputs_overlap(inputs, outputs)) return ASCAN_ERR_OVERLAP;
     }
-    const BackwardCall call{gates, states, grad_out, d_gates, d_tokens, initial, d_initial, rows, seqlen, act, ws,
-                            static_cast<hipStream_t>(stream)};
+    const BackwardCall call{gates, states, grad_out, d_gates, d_tokens, initial, d_initial, values, rows, seqlen, act,
+                            ws, static_cast<hipStream_t>(stream)};
     switch (dtype) {
         case ASCAN_F32: return backward_f32(call);
         case ASCAN_BF16: return backward_bf16(call);
@@ -203,7 +209,7 @@ int ascan_forward(const void* gates, const void* tokens, void* out, int64_t rows
 
 int ascan_backward(const void* gates, const void* states, const void* grad_out, void* d_gates, void* d_tokens,
                    int64_t rows, int64_t seqlen, int dtype, void* stream) {
-    return backward_checked(gates, states, grad_out, d_gates, d_tokens, nullptr, nullptr, rows, seqlen, dtype,
+    return backward_checked(gates, states, grad_out, d_gates, d_tokens, nullptr, nullptr, nullptr, rows, seqlen, dtype,
                             ASCAN_GATE_IDENTITY, Workspace{nullptr, 0}, stream);
 }
 
@@ -243,7 +249,7 @@ int ascan_forward_split_static(const void* gates, const void* tokens, void* out,
 int ascan_backward_split(const void* gates, const void* states, const void* grad_out, void* d_gates,
                          void* d_tokens, int64_t rows, int64_t seqlen, int dtype, void* workspace,
                          size_t workspace_bytes, void* stream) {
-    return backward_checked(gates, states, grad_out, d_gates, d_tokens, nullptr, nullptr, rows, seqlen, dtype,
+    return backward_checked(gates, states, grad_out, d_gates, d_tokens, nullptr, nullptr, nullptr, rows, seqlen, dtype,
                             ASCAN_GATE_IDENTITY, Workspace{workspace, workspace_bytes}, stream);
 }
 
@@ -257,7 +263,7 @@ int ascan_forward_from(const void* gates, const void* tokens, const void* initia
 int ascan_backward_from(const void* gates, const void* states, const void* initial, const void* grad_out,
                         void* d_gates, void* d_tokens, void* d_initial, int64_t rows, int64_t seqlen, int dtype,
                         void* workspace, size_t workspace_bytes, void* stream) {
-    return backward_checked(gates, states, grad_out, d_gates, d_tokens, initial, d_initial, rows, seqlen, dtype,
+    return backward_checked(gates, states, grad_out, d_gates, d_tokens, initial, d_initial, nullptr, rows, seqlen, dtype,
                             ASCAN_GATE_IDENTITY, Workspace{workspace, workspace_bytes}, stream);
 }
 
@@ -270,8 +276,16 @@ int ascan_forward_gated(const void* gate_inputs, const void* tokens, const void*
 int ascan_backward_gated(const void* gate_inputs, const void* states, const void* initial, const void* grad_out,
                          void* d_gate_inputs, void* d_tokens, void* d_initial, int64_t rows, int64_t seqlen,
                          int dtype, int gate, void* workspace, size_t workspace_bytes, void* stream) {
-    return backward_checked(gate_inputs, states, grad_out, d_gate_inputs, d_tokens, initial, d_initial, rows, seqlen,
-                            dtype, gate, Workspace{workspace, workspace_bytes}, stream);
+    if (gate == ASCAN_GATE_SIGMOID_LERP) return ASCAN_ERR_BAD_ACTIVATION;  // needs the values: ascan_backward_lerp
+    return backward_checked(gate_inputs, states, grad_out, d_gate_inputs, d_tokens, initial, d_initial, nullptr, rows,
+                            seqlen, dtype, gate, Workspace{workspace, workspace_bytes}, stream);
+}
+
+int ascan_backward_lerp(const void* gate_inputs, const void* values, const void* states, const void* initial,
+                        const void* grad_out, void* d_gate_inputs, void* d_values, void* d_initial, int64_t rows,
+                        int64_t seqlen, int dtype, void* workspace, size_t workspace_bytes, void* stream) {
+    return backward_checked(gate_inputs, states, grad_out, d_gate_inputs, d_values, initial, d_initial, values, rows,
+                            seqlen, dtype, ASCAN_GATE_SIGMOID_LERP, Workspace{workspace, workspace_bytes}, stream);
 }
 
 unsigned int ascan_workspace_timeouts(const void* workspace_header_copy) {
@@ -287,7 +301,7 @@ const char* ascan_status_string(int status) {
         case ASCAN_ERR_MISALIGNED: return "a buffer is not aligned to its element size";
         case ASCAN_ERR_LAUNCH: return "the HIP runtime reported a launch error";
         case ASCAN_ERR_BAD_ACTIVATION:
-            return "unsupported gate activation: expecting identity, or sigmoid with float32, bfloat16 or float16";
+            return "unsupported gate activation: expecting identity, or a sigmoid gate with float32, bfloat16 or float16";
         case ASCAN_ERR_OVERLAP: return "an output buffer overlaps an input or another output buffer of the call";
         case ASCAN_ERR_TOO_LARGE:
             return "the split-row table of this problem exceeds the library's static workspace (ASCAN_STATIC_WORKSPACE_BYTES)";

@@ -8,28 +8,39 @@
 namespace ascan {
 namespace {
 
+// The arguments every backward launch passes on unchanged.
+struct BackwardBuffers {
+    const void* gates;
+    const void* states;
+    const void* grad_out;
+    void* d_gates;
+    void* d_tokens;
+    const void* initial;
+    void* d_initial;
+    const void* values;  // the interpolating gate's fourth input, else null
+};
+
 template <class Tr, int W, bool ALIGNED, bool REGULAR, int ACT>
-hipError_t launch_backward(const void* gates, const void* states, const void* grad_out, void* d_gates,
-                           void* d_tokens, const void* initial, void* d_initial, int64_t rows, int64_t T, int grid,
-                           int rows_per_block, hipStream_t stream) {
+hipError_t launch_backward(const BackwardBuffers& b, int64_t rows, int64_t T, int grid, int rows_per_block,
+                           hipStream_t stream) {
     using S = typename Tr::S;
     using TokS = typename Tr::TokS;
-    constexpr int U = REGULAR ? Tuning<Tr>::UB : Tuning<Tr>::UBG;
+    constexpr int U = backward_blocks<ACT>(REGULAR ? Tuning<Tr>::UB : Tuning<Tr>::UBG);
     const unsigned blocks = (unsigned)((rows + rows_per_block - 1) / rows_per_block);
     const unsigned threads = 64u * W * rows_per_block;
     return launch(scan_backward_kernel<Tr, W, U, ALIGNED, REGULAR, false, ACT, false>, blocks, threads, stream,
-                  static_cast<const S*>(gates), static_cast<const S*>(states), static_cast<const S*>(grad_out),
-                  static_cast<S*>(d_gates), static_cast<TokS*>(d_tokens), rows, T,
-                  static_cast<SplitHeader*>(nullptr), static_cast<const S*>(initial), static_cast<S*>(d_initial), grid, 0);
+                  static_cast<const S*>(b.gates), static_cast<const S*>(b.states), static_cast<const S*>(b.grad_out),
+                  static_cast<S*>(b.d_gates), static_cast<TokS*>(b.d_tokens), rows, T,
+                  static_cast<SplitHeader*>(nullptr), static_cast<const S*>(b.initial), static_cast<S*>(b.d_initial),
+                  grid, 0, static_cast<const S*>(b.values));
 }
 
 template <class Tr, bool REGULAR, int ACT>
-hipError_t launch_backward_split(const void* gates, const void* states, const void* grad_out, void* d_gates,
-                                 void* d_tokens, const void* initial, void* d_initial, int64_t rows, int64_t T,
-                                 int grid, int64_t ntiles, const Workspace& ws, hipStream_t stream) {
+hipError_t launch_backward_split(const BackwardBuffers& b, int64_t rows, int64_t T, int grid, int64_t ntiles,
+                                 const Workspace& ws, hipStream_t stream) {
     using S = typename Tr::S;
     using TokS = typename Tr::TokS;
-    constexpr int U = REGULAR ? SplitTuning<Tr>::UB : SplitTuning<Tr>::UBG;
+    constexpr int U = backward_blocks<ACT>(REGULAR ? SplitTuning<Tr>::UB : SplitTuning<Tr>::UBG);
     auto kernel = scan_backward_kernel<Tr, kSplitWaves, U, true, REGULAR, true, ACT, false>;
     const unsigned resident = resident_workgroups(kernel, 64 * kSplitWaves);
     if (resident == 0) return hipErrorInvalidConfiguration;
@@ -37,34 +48,34 @@ hipError_t launch_backward_split(const void* gates, const void* states, const vo
     if (e != hipSuccess) return e;
     const int64_t tiles = rows * ntiles;
     return launch(kernel, (unsigned)(tiles < resident ? tiles : resident), 64u * kSplitWaves, stream,
-                  static_cast<const S*>(gates), static_cast<const S*>(states), static_cast<const S*>(grad_out),
-                  static_cast<S*>(d_gates), static_cast<TokS*>(d_tokens), rows, T,
-                  static_cast<SplitHeader*>(ws.ptr), static_cast<const S*>(initial), static_cast<S*>(d_initial), grid, 0);
+                  static_cast<const S*>(b.gates), static_cast<const S*>(b.states), static_cast<const S*>(b.grad_out),
+                  static_cast<S*>(b.d_gates), static_cast<TokS*>(b.d_tokens), rows, T,
+                  static_cast<SplitHeader*>(ws.ptr), static_cast<const S*>(b.initial), static_cast<S*>(b.d_initial),
+                  grid, 0, static_cast<const S*>(b.values));
 }
 
 template <class Tr, int PW, bool ALIGNED, int ACT>
-hipError_t launch_backward_packed(const void* gates, const void* states, const void* grad_out, void* d_gates,
-                                  void* d_tokens, const void* initial, void* d_initial, int64_t rows, int64_t T,
-                                  int grid, int group, hipStream_t stream) {
+hipError_t launch_backward_packed(const BackwardBuffers& b, int64_t rows, int64_t T, int grid, int group,
+                                  hipStream_t stream) {
     using S = typename Tr::S;
     using TokS = typename Tr::TokS;
     const unsigned blocks = (unsigned)((rows + group - 1) / group);
     return launch(scan_backward_kernel<Tr, PW, Tuning<Tr>::UBG, ALIGNED, false, false, ACT, true>, blocks,
-                  64u * PW, stream, static_cast<const S*>(gates), static_cast<const S*>(states),
-                  static_cast<const S*>(grad_out), static_cast<S*>(d_gates), static_cast<TokS*>(d_tokens), rows, T,
-                  static_cast<SplitHeader*>(nullptr), static_cast<const S*>(initial), static_cast<S*>(d_initial), grid,
-                  group);
+                  64u * PW, stream, static_cast<const S*>(b.gates), static_cast<const S*>(b.states),
+                  static_cast<const S*>(b.grad_out), static_cast<S*>(b.d_gates), static_cast<TokS*>(b.d_tokens), rows,
+                  T, static_cast<SplitHeader*>(nullptr), static_cast<const S*>(b.initial),
+                  static_cast<S*>(b.d_initial), grid, group, static_cast<const S*>(b.values));
 }
 
 template <class Tr>
-int backward_typed(const void* gates, const void* states, const void* grad_out, void* d_gates, void* d_tokens,
-                   const void* initial, void* d_initial, int64_t rows, int64_t T, int act, const Workspace& ws,
+int backward_typed(const BackwardBuffers& b, int64_t rows, int64_t T, int act, const Workspace& ws,
                    hipStream_t stream) {
     constexpr int64_t kElem = (int64_t)sizeof(typename Tr::S);
-    constexpr int64_t SUB = (int64_t)Tuning<Tr>::UB * 64 * Tr::EPV;    // regular kernels
-    constexpr int64_t SUBG = (int64_t)Tuning<Tr>::UBG * 64 * Tr::EPV;  // kernels with masking code
-    const void* const state_like[] = {gates, states, grad_out, d_gates};
-    const Lead at = find_lead<Tr>(state_like, d_tokens);
+    const int64_t SUB = (int64_t)backward_blocks_of(act, Tuning<Tr>::UB) * 64 * Tr::EPV;  // regular kernels
+    constexpr int64_t SUBG = (int64_t)Tuning<Tr>::UBG * 64 * Tr::EPV;                     // kernels with masking code
+    static_assert(Tuning<Tr>::UBG <= 2 && SplitTuning<Tr>::UBG <= 2, "the interpolating gate assumes 2 KiB per wave here");
+    const void* const state_like[] = {b.gates, b.states, b.grad_out, b.d_gates, b.values ? b.values : b.gates};
+    const Lead at = find_lead<Tr>(state_like, b.d_tokens);
     const bool same_lead = at.same;
     const int lead = at.lead;
     Plan plan = choose_plan(T, SUB, kElem, kTrimPlan<Tr>);
@@ -72,84 +83,61 @@ int backward_typed(const void* gates, const void* states, const void* grad_out, 
     if (access != Access::kRegular) plan = choose_plan(T, SUBG, kElem, kTrimPlan<Tr>);
     const int R = plan.rows_per_block;
     hipError_t err = hipSuccess;
-#define ASCAN_BWD_PACKED(PW, AL, ACT)                                                                                  \
-    launch_backward_packed<Tr, PW, AL, ACT>(gates, states, grad_out, d_gates, d_tokens, initial, d_initial, rows, T, \
-                                            at.grid, group, stream)
     // 16-bit rows of 512 bytes and more, vectorised flavour, plenty of them: groups of the wider workgroup
     if constexpr (Tr::kNarrow) {
         if (same_lead && T * kElem >= kPackedWideRowBytes) {
             const int group = packed_group(rows, T, kElem, SUBG * kPackedWavesWide, at.grid);
             if (group != 0 && rows / group >= kPackedWideMinGroups) {
-                if (act == kGateSigmoid) {
-                    err = ASCAN_BWD_PACKED(kPackedWavesWide, true, kGateSigmoid);
-                } else {
-                    err = ASCAN_BWD_PACKED(kPackedWavesWide, true, kGateIdentity);
-                }
+                err = with_gate<Tr>(act, [&](auto gate) {
+                    return launch_backward_packed<Tr, kPackedWavesWide, true, decltype(gate)::value>(b, rows, T, at.grid,
+                                                                                                     group, stream);
+                });
                 return launch_status(err);
             }
         }
     }
     if (const int group = packed_group(rows, T, kElem, SUBG * kPackedWaves, same_lead ? at.grid : 1)) {
-        if (act == kGateSigmoid) {
-            if constexpr (kHasSigmoid<Tr>) {
-                err = same_lead ? ASCAN_BWD_PACKED(kPackedWaves, true, kGateSigmoid)
-                                : ASCAN_BWD_PACKED(kPackedWaves, false, kGateSigmoid);
-            }
-        } else {
-            err = same_lead ? ASCAN_BWD_PACKED(kPackedWaves, true, kGateIdentity)
-                            : ASCAN_BWD_PACKED(kPackedWaves, false, kGateIdentity);
-        }
-#undef ASCAN_BWD_PACKED
+        err = with_gate<Tr>(act, [&](auto gate) {
+            constexpr int ACT = decltype(gate)::value;
+            return same_lead ? launch_backward_packed<Tr, kPackedWaves, true, ACT>(b, rows, T, at.grid, group, stream)
+                             : launch_backward_packed<Tr, kPackedWaves, false, ACT>(b, rows, T, at.grid, group, stream);
+        });
         return launch_status(err);
     }
     if (same_lead && ws.ptr != nullptr) {
-        constexpr int64_t SUBS = (int64_t)SplitTuning<Tr>::UB * 64 * Tr::EPV;
+        const int64_t SUBS = (int64_t)backward_blocks_of(act, SplitTuning<Tr>::UB) * 64 * Tr::EPV;
         constexpr int64_t SUBSG = (int64_t)SplitTuning<Tr>::UBG * 64 * Tr::EPV;
         const bool regular = lead == 0 && T % (SUBS * kSplitWaves) == 0;
         const int64_t ntiles = host_tiles_per_row<Tr>(T, (regular ? SUBS : SUBSG) * kSplitWaves, regular, at);
         if (want_split(rows, ntiles) && workspace_fits(ws, rows, ntiles)) {
-#define ASCAN_BWD_SPLIT(REG, ACT)                                                                              \
-    launch_backward_split<Tr, REG, ACT>(gates, states, grad_out, d_gates, d_tokens, initial, d_initial, rows, T, \
-                                        at.grid, ntiles, ws, stream)
-            if (act == kGateSigmoid) {
-                if constexpr (kHasSigmoid<Tr>) {
-                    err = regular ? ASCAN_BWD_SPLIT(true, kGateSigmoid) : ASCAN_BWD_SPLIT(false, kGateSigmoid);
-                }
-            } else {
-                err = regular ? ASCAN_BWD_SPLIT(true, kGateIdentity) : ASCAN_BWD_SPLIT(false, kGateIdentity);
-            }
-#undef ASCAN_BWD_SPLIT
+            err = with_gate<Tr>(act, [&](auto gate) {
+                constexpr int ACT = decltype(gate)::value;
+                return regular ? launch_backward_split<Tr, true, ACT>(b, rows, T, at.grid, ntiles, ws, stream)
+                               : launch_backward_split<Tr, false, ACT>(b, rows, T, at.grid, ntiles, ws, stream);
+            });
             return launch_status(err);
         }
     }
-#define ASCAN_BWD_ARGS gates, states, grad_out, d_gates, d_tokens, initial, d_initial, rows, T, at.grid, R, stream
-#define ASCAN_BWD(WV, AL, REG)                                                              \
-    do {                                                                                    \
-        if (act == kGateSigmoid) {                                                          \
-            if constexpr (kHasSigmoid<Tr>)                                                  \
-                err = launch_backward<Tr, WV, AL, REG, kGateSigmoid>(ASCAN_BWD_ARGS);       \
-        } else {                                                                            \
-            err = launch_backward<Tr, WV, AL, REG, kGateIdentity>(ASCAN_BWD_ARGS);          \
-        }                                                                                   \
-    } while (0)
-#define ASCAN_BWD_W(AL, REG)                            \
-    switch (plan.waves_per_row) {                       \
-        case 1: ASCAN_BWD(1, AL, REG); break;           \
-        case 2: ASCAN_BWD(2, AL, REG); break;           \
-        case 4: ASCAN_BWD(4, AL, REG); break;           \
-        case 8: ASCAN_BWD(8, AL, REG); break;           \
-        default: ASCAN_BWD(16, AL, REG); break;         \
-    }
+    auto with_waves = [&](auto aligned, auto reg) {
+        return with_gate<Tr>(act, [&](auto gate) {
+            constexpr int ACT = decltype(gate)::value;
+            constexpr bool AL = decltype(aligned)::value, REG = decltype(reg)::value;
+            switch (plan.waves_per_row) {
+                case 1: return launch_backward<Tr, 1, AL, REG, ACT>(b, rows, T, at.grid, R, stream);
+                case 2: return launch_backward<Tr, 2, AL, REG, ACT>(b, rows, T, at.grid, R, stream);
+                case 4: return launch_backward<Tr, 4, AL, REG, ACT>(b, rows, T, at.grid, R, stream);
+                case 8: return launch_backward<Tr, 8, AL, REG, ACT>(b, rows, T, at.grid, R, stream);
+                default: return launch_backward<Tr, 16, AL, REG, ACT>(b, rows, T, at.grid, R, stream);
+            }
+        });
+    };
     if (access == Access::kRegular) {
-        ASCAN_BWD_W(true, true);
+        err = with_waves(std::true_type{}, std::true_type{});
     } else if (access == Access::kVector) {
-        ASCAN_BWD_W(true, false);
+        err = with_waves(std::true_type{}, std::false_type{});
     } else {
-        ASCAN_BWD_W(false, false);
+        err = with_waves(std::false_type{}, std::false_type{});
     }
-#undef ASCAN_BWD_W
-#undef ASCAN_BWD
-#undef ASCAN_BWD_ARGS
     return launch_status(err);
 }
 
@@ -157,11 +145,11 @@ int backward_typed(const void* gates, const void* states, const void* grad_out, 
 }  // namespace ascan
 
 // Defines ascan::NAME, the backward entry of one dtype, in the including file.
-#define ASCAN_DEFINE_BACKWARD(NAME, TRAITS)                                                                  \
-    int ascan::NAME(const ascan::BackwardCall& c) {                                                          \
-        return ascan::backward_typed<ascan::TRAITS>(c.gates, c.states, c.grad_out, c.d_gates, c.d_tokens,   \
-                                                    c.initial, c.d_initial, c.rows, c.seqlen, c.gate,       \
-                                                    c.workspace, c.stream);                                 \
+#define ASCAN_DEFINE_BACKWARD(NAME, TRAITS)                                                                     \
+    int ascan::NAME(const ascan::BackwardCall& c) {                                                             \
+        const ascan::BackwardBuffers b{c.gates, c.states, c.grad_out, c.d_gates, c.d_tokens, c.initial, c.d_initial, \
+                                       c.values};                                                               \
+        return ascan::backward_typed<ascan::TRAITS>(b, c.rows, c.seqlen, c.gate, c.workspace, c.stream);        \
     }
 
 #endif  // ASCAN_BACKWARD_DISPATCH_H_

@@ -17,6 +17,9 @@ namespace {
 // ---------------------------------------------------------------------------
 // Fused backward kernel: reverse-time scan over gate[t+1] producing d_tokens,
 // and d_gates[t] = d_tokens[t] * conj(x[t-1]) in the same pass.
+// With the interpolating gate (x[t] = a x[t-1] + (1 - a) v[t], a = sigmoid(z))
+// the kernel also reads the values v and writes, for the same g,
+// d_v[t] = g[t] (1 - a[t]) and d_z[t] = g[t] (x[t-1] - v[t]) a[t] (1 - a[t]).
 // ---------------------------------------------------------------------------
 template <class Tr, int W, int U, bool ALIGNED, bool REGULAR, bool SPLIT, int ACT, bool PACKED>
 __global__ void __launch_bounds__(64 * kMaxWavesPerBlock)
@@ -24,13 +27,15 @@ __global__ void __launch_bounds__(64 * kMaxWavesPerBlock)
                          const typename Tr::S* __restrict__ grad_out, typename Tr::S* __restrict__ d_gates,
                          typename Tr::TokS* __restrict__ d_tokens, int64_t rows, int64_t T, SplitHeader* split,
                          const typename Tr::S* __restrict__ initial, typename Tr::S* __restrict__ d_initial, int G,
-                         int group) {
+                         int group, const typename Tr::S* __restrict__ values) {
     using S = typename Tr::S;
     using V = typename Tr::V;
     constexpr int EPV = Tr::EPV;
     constexpr int64_t SUB = (int64_t)U * 64 * EPV;
     constexpr int64_t TILE = SUB * W;
     static_assert(!PACKED || (!SPLIT && !REGULAR), "packed rows use the general kernels, one group per workgroup");
+    constexpr bool LERP = ACT == kGateSigmoidLerp;  // `values` is a fourth input
+    constexpr int NIN = LERP ? 4 : 3;
 
     const int lane = threadIdx.x & 63;
     // Packed rows: this workgroup scans rows [first_row, first_row + nrows) as one row of `len` elements.
@@ -45,7 +50,7 @@ __global__ void __launch_bounds__(64 * kMaxWavesPerBlock)
     // Split rows: the workgroups take tiles by ticket, row by row, until none
     // is left; a workgroup only ever waits for tiles whose owners started before it.
     __shared__ long long split_mailbox[2];
-    __shared__ u32x4_t parked[SPLIT ? 3 * U * 64 : 1];  // wave 0's raw vectors during its walk back
+    __shared__ u32x4_t parked[SPLIT ? NIN * U * 64 : 1];  // wave 0's raw vectors during its walk back
     __shared__ V parked_values[SPLIT ? 4 * U * 64 : 1];  // and its per-lane scan results
     SplitWalk walk;  // starts at row blockIdx % rows
     walk.row = SPLIT ? (int64_t)(blockIdx.x % rows) : 0;
@@ -77,6 +82,7 @@ __global__ void __launch_bounds__(64 * kMaxWavesPerBlock)
     const S* __restrict__ arow = gates + row * T - lo;
     const S* __restrict__ xrow = states + row * T - lo;
     const S* __restrict__ drow = grad_out + row * T - lo;
+    const S* __restrict__ vrow = LERP ? values + row * T - lo : nullptr;
     S* __restrict__ dgrow = d_gates + row * T - lo;
     typename Tr::TokS* __restrict__ dtrow = d_tokens + row * T - lo;
 
@@ -114,6 +120,7 @@ __global__ void __launch_bounds__(64 * kMaxWavesPerBlock)
         const S* __restrict__ asub = arow + sub_base;
         const S* __restrict__ dsub = drow + sub_base;
         const S* __restrict__ xsub = xrow + sub_base;
+        const S* __restrict__ vsub = LERP ? vrow + sub_base : nullptr;
         S* __restrict__ dgsub = dgrow + sub_base;
         typename Tr::TokS* __restrict__ dtsub = dtrow + sub_base;
 
@@ -127,7 +134,7 @@ __global__ void __launch_bounds__(64 * kMaxWavesPerBlock)
                                         (int)(sub_base - lo), (int)SUB, stage_all + w * SUB, lane);
         }
 
-        u32x4_t araw[U], draw[U], xraw[U];
+        u32x4_t araw[U], draw[U], xraw[U], vraw[LERP ? U : 1];
         if (touches) {
 #pragma unroll
             for (int j = 0; j < U; ++j) {
@@ -135,6 +142,7 @@ __global__ void __launch_bounds__(64 * kMaxWavesPerBlock)
                 araw[j] = load_raw<Tr, ALIGNED, FULL>(asub, off, win, identity_gate<ACT, V>());
                 draw[j] = load_raw<Tr, ALIGNED, FULL>(dsub, off, win, vzero<V>());
                 xraw[j] = load_raw<Tr, ALIGNED, FULL>(xsub, off, win, x_start);
+                if constexpr (LERP) vraw[j] = load_raw<Tr, ALIGNED, FULL>(vsub, off, win, vzero<V>());
             }
         } else {
 #pragma unroll
@@ -142,6 +150,7 @@ __global__ void __launch_bounds__(64 * kMaxWavesPerBlock)
                 araw[j] = fill_raw<Tr>(identity_gate<ACT, V>());
                 draw[j] = fill_raw<Tr>(vzero<V>());
                 xraw[j] = fill_raw<Tr>(x_start);
+                if constexpr (LERP) vraw[j] = fill_raw<Tr>(vzero<V>());
             }
         }
 
@@ -169,9 +178,9 @@ __global__ void __launch_bounds__(64 * kMaxWavesPerBlock)
         V totA[U], totX[U], exA[U], exX[U];
 #pragma unroll
         for (int j = 0; j < U; ++j) {
-            V a[EPV], d[EPV], x[EPV];
+            V a[EPV], d[EPV], x[EPV], a_rest[EPV];  // a_rest = 1 - a, interpolating gate only
             Tr::unpack(araw[j], a);
-            activate<ACT>(a);
+            activate_with_complement<ACT>(a, a_rest);
             Tr::unpack(draw[j], d);
             Tr::unpack(xraw[j], x);
             V hi_edge, lo_edge;
@@ -227,9 +236,10 @@ __global__ void __launch_bounds__(64 * kMaxWavesPerBlock)
                 [&] {
 #pragma unroll
                     for (int j = 0; j < U; ++j) {
-                        parked[(3 * j) * 64 + lane] = araw[j];
-                        parked[(3 * j + 1) * 64 + lane] = draw[j];
-                        parked[(3 * j + 2) * 64 + lane] = xraw[j];
+                        parked[(NIN * j) * 64 + lane] = araw[j];
+                        parked[(NIN * j + 1) * 64 + lane] = draw[j];
+                        parked[(NIN * j + 2) * 64 + lane] = xraw[j];
+                        if constexpr (LERP) parked[(NIN * j + 3) * 64 + lane] = vraw[j];
                         parked_values[(4 * j) * 64 + lane] = a_next[j];
                         parked_values[(4 * j + 1) * 64 + lane] = x_prev[j];
                         parked_values[(4 * j + 2) * 64 + lane] = exA[j];
@@ -239,9 +249,10 @@ __global__ void __launch_bounds__(64 * kMaxWavesPerBlock)
                 [&] {
 #pragma unroll
                     for (int j = 0; j < U; ++j) {
-                        araw[j] = parked[(3 * j) * 64 + lane];
-                        draw[j] = parked[(3 * j + 1) * 64 + lane];
-                        xraw[j] = parked[(3 * j + 2) * 64 + lane];
+                        araw[j] = parked[(NIN * j) * 64 + lane];
+                        draw[j] = parked[(NIN * j + 1) * 64 + lane];
+                        xraw[j] = parked[(NIN * j + 2) * 64 + lane];
+                        if constexpr (LERP) vraw[j] = parked[(NIN * j + 3) * 64 + lane];
                         a_next[j] = parked_values[(4 * j) * 64 + lane];
                         x_prev[j] = parked_values[(4 * j + 1) * 64 + lane];
                         exA[j] = parked_values[(4 * j + 2) * 64 + lane];
@@ -258,12 +269,14 @@ __global__ void __launch_bounds__(64 * kMaxWavesPerBlock)
                 forget_unpacked(araw[j]);
                 forget_unpacked(draw[j]);
                 forget_unpacked(xraw[j]);
+                if constexpr (LERP) forget_unpacked(vraw[j]);
             }
-            V a[EPV], d[EPV], x[EPV];
+            V a[EPV], d[EPV], x[EPV], a_rest[EPV], v[LERP ? EPV : 1];
             Tr::unpack(araw[j], a);
-            activate<ACT>(a);
+            activate_with_complement<ACT>(a, a_rest);
             Tr::unpack(draw[j], d);
             Tr::unpack(xraw[j], x);
+            if constexpr (LERP) Tr::unpack(vraw[j], v);
             V gr = carry_in<PACKED>(exA[j], c, exX[j]);  // g entering this lane's vector from above
             c = carry_in<PACKED>(totA[j], c, totX[j]);
             const int off = vec_offset<U, EPV, true>(j, lane);
@@ -278,13 +291,20 @@ __global__ void __launch_bounds__(64 * kMaxWavesPerBlock)
             if constexpr (PACKED) {
                 cut_rows_backward<Tr>(after, before, is_first, row_of, (int)(sub_base - lo) + off, cuts);
             }
-            V dt[EPV], dg[EPV];
+            V dt[EPV], dg[EPV], gs[PACKED ? EPV : 1];  // gs: g itself, for the rows' initial states
 #pragma unroll
             for (int e = EPV - 1; e >= 0; --e) {
                 gr = carry_in<PACKED>(vconj(after[e]), gr, d[e]);
-                dt[e] = gr;
-                dg[e] = vmul(gr, vconj(before[e]));
-                if constexpr (ACT != kGateIdentity) dg[e] = vmul(dg[e], gate_slope<ACT>(a[e]));
+                if constexpr (PACKED) gs[e] = gr;
+                if constexpr (LERP) {
+                    // token = (1 - a) v:  d_v = g (1 - a);  d_a = g (x[t-1] - v);  d_z = d_a a (1 - a)
+                    dt[e] = gr * a_rest[e];
+                    dg[e] = (gr * (before[e] - v[e])) * (a[e] * a_rest[e]);
+                } else {
+                    dt[e] = gr;
+                    dg[e] = vmul(gr, vconj(before[e]));
+                    if constexpr (ACT != kGateIdentity) dg[e] = vmul(dg[e], gate_slope<ACT>(a[e]));
+                }
             }
             if (touches) {
                 store_tok_vec<Tr, ALIGNED, FULL>(dtsub, off, win, dt);
@@ -295,7 +315,7 @@ __global__ void __launch_bounds__(64 * kMaxWavesPerBlock)
                 if (d_initial != nullptr) {
 #pragma unroll
                     for (int e = 0; e < EPV; ++e) {
-                        if (is_first[e]) Tr::store1(d_initial + first_row + row_of[e], vmul(vconj(a[e]), dt[e]));
+                        if (is_first[e]) Tr::store1(d_initial + first_row + row_of[e], vmul(vconj(a[e]), gs[e]));
                     }
                 }
             }

@@ -50,6 +50,23 @@ hipError_t launch_forward_packed(const void* gates, const void* tokens, void* ou
                   grid, group);
 }
 
+// Turns (gate, reverse, flag) into compile-time tags and calls go(rev, flag, gate).
+// A gate other than the identity implies forward time.
+template <class Tr, class Go>
+hipError_t dispatch_forward(int act, bool reverse, bool flag, Go&& go) {
+    return with_gate<Tr>(act, [&](auto gate) {
+        constexpr int ACT = decltype(gate)::value;
+        if constexpr (ACT != kGateIdentity) {
+            return flag ? go(std::false_type{}, std::true_type{}, gate) : go(std::false_type{}, std::false_type{}, gate);
+        } else {
+            if (reverse) {
+                return flag ? go(std::true_type{}, std::true_type{}, gate) : go(std::true_type{}, std::false_type{}, gate);
+            }
+            return flag ? go(std::false_type{}, std::true_type{}, gate) : go(std::false_type{}, std::false_type{}, gate);
+        }
+    });
+}
+
 template <class Tr>
 int forward_typed(const void* gates, const void* tokens, void* out, const void* initial, int64_t rows, int64_t T,
                   bool reverse, int act, const Workspace& ws, hipStream_t stream) {
@@ -65,19 +82,14 @@ int forward_typed(const void* gates, const void* tokens, void* out, const void* 
     if (access != Access::kRegular) plan = choose_plan(T, SUBG, kElem, kTrimPlan<Tr>);
     const int R = plan.rows_per_block;
     hipError_t err = hipSuccess;
+    // Gated kernels run forward in time only (validated by the entry points); REV below is a
+    // compile-time false for them.
     if (const int group = packed_group(rows, T, kElem, SUBG * kPackedWaves, same_lead ? at.grid : 1)) {
-#define ASCAN_FWD_PACKED(REV, AL, ACT) \
-    launch_forward_packed<Tr, REV, AL, ACT>(gates, tokens, out, initial, rows, T, at.grid, group, stream)
-        if (act == kGateSigmoid) {
-            if constexpr (kHasSigmoid<Tr>) {
-                err = same_lead ? ASCAN_FWD_PACKED(false, true, kGateSigmoid) : ASCAN_FWD_PACKED(false, false, kGateSigmoid);
-            }
-        } else if (same_lead) {
-            err = reverse ? ASCAN_FWD_PACKED(true, true, kGateIdentity) : ASCAN_FWD_PACKED(false, true, kGateIdentity);
-        } else {
-            err = reverse ? ASCAN_FWD_PACKED(true, false, kGateIdentity) : ASCAN_FWD_PACKED(false, false, kGateIdentity);
-        }
-#undef ASCAN_FWD_PACKED
+        auto go = [&](auto rev, auto aligned, auto gate) {
+            return launch_forward_packed<Tr, decltype(rev)::value, decltype(aligned)::value, decltype(gate)::value>(
+                gates, tokens, out, initial, rows, T, at.grid, group, stream);
+        };
+        err = dispatch_forward<Tr>(act, reverse, same_lead, go);
         return launch_status(err);
     }
     if (same_lead && ws.ptr != nullptr) {
@@ -86,51 +98,38 @@ int forward_typed(const void* gates, const void* tokens, void* out, const void* 
         const bool regular = lead == 0 && T % (SUBS * kSplitWaves) == 0;
         const int64_t ntiles = host_tiles_per_row<Tr>(T, (regular ? SUBS : SUBSG) * kSplitWaves, regular, at);
         if (want_split(rows, ntiles) && workspace_fits(ws, rows, ntiles)) {
-#define ASCAN_FWD_SPLIT(REV, REG, ACT) \
-    launch_forward_split<Tr, REV, REG, ACT>(gates, tokens, out, initial, rows, T, at.grid, ntiles, ws, stream)
-            if (act == kGateSigmoid) {
-                if constexpr (kHasSigmoid<Tr>) {
-                    err = regular ? ASCAN_FWD_SPLIT(false, true, kGateSigmoid) : ASCAN_FWD_SPLIT(false, false, kGateSigmoid);
-                }
-            } else if (regular) {
-                err = reverse ? ASCAN_FWD_SPLIT(true, true, kGateIdentity) : ASCAN_FWD_SPLIT(false, true, kGateIdentity);
-            } else {
-                err = reverse ? ASCAN_FWD_SPLIT(true, false, kGateIdentity) : ASCAN_FWD_SPLIT(false, false, kGateIdentity);
-            }
-#undef ASCAN_FWD_SPLIT
+            auto go = [&](auto rev, auto reg, auto gate) {
+                return launch_forward_split<Tr, decltype(rev)::value, decltype(reg)::value, decltype(gate)::value>(
+                    gates, tokens, out, initial, rows, T, at.grid, ntiles, ws, stream);
+            };
+            err = dispatch_forward<Tr>(act, reverse, regular, go);
             return launch_status(err);
         }
     }
-#define ASCAN_FWD_ARGS gates, tokens, out, initial, rows, T, at.grid, R, stream
-#define ASCAN_FWD(WV, AL, REG)                                                                  \
-    do {                                                                                        \
-        if (act == kGateSigmoid) {                                                              \
-            if constexpr (kHasSigmoid<Tr>)                                                      \
-                err = launch_forward<Tr, WV, false, AL, REG, kGateSigmoid>(ASCAN_FWD_ARGS);     \
-        } else if (reverse) {                                                                   \
-            err = launch_forward<Tr, WV, true, AL, REG, kGateIdentity>(ASCAN_FWD_ARGS);         \
-        } else {                                                                                \
-            err = launch_forward<Tr, WV, false, AL, REG, kGateIdentity>(ASCAN_FWD_ARGS);        \
-        }                                                                                       \
-    } while (0)
-#define ASCAN_FWD_W(AL, REG)                            \
-    switch (plan.waves_per_row) {                       \
-        case 1: ASCAN_FWD(1, AL, REG); break;           \
-        case 2: ASCAN_FWD(2, AL, REG); break;           \
-        case 4: ASCAN_FWD(4, AL, REG); break;           \
-        case 8: ASCAN_FWD(8, AL, REG); break;           \
-        default: ASCAN_FWD(16, AL, REG); break;         \
-    }
+    auto with_waves = [&](auto aligned, auto reg) {
+        auto go = [&](auto rev, auto waves, auto gate) {
+            return launch_forward<Tr, decltype(waves)::value, decltype(rev)::value, decltype(aligned)::value,
+                                  decltype(reg)::value, decltype(gate)::value>(gates, tokens, out, initial, rows, T,
+                                                                               at.grid, R, stream);
+        };
+        auto by_waves = [&](auto rev, auto, auto gate) {
+            switch (plan.waves_per_row) {
+                case 1: return go(rev, std::integral_constant<int, 1>{}, gate);
+                case 2: return go(rev, std::integral_constant<int, 2>{}, gate);
+                case 4: return go(rev, std::integral_constant<int, 4>{}, gate);
+                case 8: return go(rev, std::integral_constant<int, 8>{}, gate);
+                default: return go(rev, std::integral_constant<int, 16>{}, gate);
+            }
+        };
+        return dispatch_forward<Tr>(act, reverse, true, by_waves);
+    };
     if (access == Access::kRegular) {
-        ASCAN_FWD_W(true, true);
+        err = with_waves(std::true_type{}, std::true_type{});
     } else if (access == Access::kVector) {
-        ASCAN_FWD_W(true, false);
+        err = with_waves(std::true_type{}, std::false_type{});
     } else {
-        ASCAN_FWD_W(false, false);
+        err = with_waves(std::false_type{}, std::false_type{});
     }
-#undef ASCAN_FWD_W
-#undef ASCAN_FWD
-#undef ASCAN_FWD_ARGS
     return launch_status(err);
 }
 

@@ -134,8 +134,8 @@ __global__ void __launch_bounds__(64 * kMaxWavesPerBlock)
         for (int j = 0; j < U; ++j) {
             V g[EPV], t[EPV];
             Tr::unpack(graw[j], g);
-            activate<ACT>(g);
             Tr::unpack(traw[j], t);
+            activate_pair<ACT>(g, t);
             if constexpr (PACKED) {
                 const int rel = (int)(sub_base - lo) + vec_offset<U, EPV, REV>(j, lane);
                 cut_found[j] = locate_cut<Tr, REV>(rel, cuts);
@@ -188,8 +188,8 @@ __global__ void __launch_bounds__(64 * kMaxWavesPerBlock)
             }
             V g[EPV], t[EPV];
             Tr::unpack(graw[j], g);
-            activate<ACT>(g);
             Tr::unpack(traw[j], t);
+            activate_pair<ACT>(g, t);
             if constexpr (PACKED) {
                 cut_rows<Tr, REV>(g, t, (int)(sub_base - lo) + vec_offset<U, EPV, REV>(j, lane), cuts, cut_found[j]);
             }

@@ -13,27 +13,84 @@ namespace {
 // apply the non-linearity in registers as the values are unpacked, which spares
 // the caller a pass that materialises the gates and, in the backward pass, one
 // that turns d_gates into the gradient of the logits.
-//   kGateIdentity: the stored values are the gates (the reference's operator);
-//   kGateSigmoid : gate = 1 / (1 + exp(-stored)), real dtypes only.
+//   kGateIdentity   : the stored values are the gates (the reference's operator);
+//   kGateSigmoid    : gate = 1 / (1 + exp(-stored)), real dtypes only;
+//   kGateSigmoidLerp: the same gate, and the token is (1 - gate) * stored value:
+//                     x[t] = gate * x[t-1] + (1 - gate) * v[t], the gated
+//                     interpolation of linear-RNN layers.  The tokens never
+//                     exist in memory either.
 // ---------------------------------------------------------------------------
-constexpr int kGateIdentity = 0, kGateSigmoid = 1;
+constexpr int kGateIdentity = 0, kGateSigmoid = 1, kGateSigmoidLerp = 2;
+
+template <int ACT>
+constexpr bool kGateIsSigmoid = ACT == kGateSigmoid || ACT == kGateSigmoidLerp;
 
 __device__ __forceinline__ float sigmoid(float v) {
     // v_exp_f32 computes 2^x; v_rcp_f32 is accurate to 1 ulp
     return __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(v * -1.4426950408889634f));
 }
 
+// sigmoid(v) and 1 - sigmoid(v) = sigmoid(-v), each to about 2 ulp of its own
+// magnitude: with t = exp(-|v|) the larger of the two is 1 / (1 + t) and the
+// smaller t / (1 + t), so neither is formed as a difference from 1 and nothing
+// overflows (v = +inf gives exactly (1, 0): the identity gate and a zero token).
+__device__ __forceinline__ void sigmoid_pair(float v, float& gate, float& complement) {
+    const float t = __builtin_amdgcn_exp2f(__builtin_fabsf(v) * -1.4426950408889634f);
+    const float large = __builtin_amdgcn_rcpf(1.0f + t);
+    const float small = t * large;
+    const bool positive = v >= 0.0f;
+    gate = positive ? large : small;
+    complement = positive ? small : large;
+}
+
 template <int ACT, class V, int N>
 __device__ __forceinline__ void activate(V (&g)[N]) {
+    static_assert(ACT != kGateSigmoidLerp, "the interpolating gate goes through activate_pair / activate_with_complement");
     if constexpr (ACT == kGateSigmoid) {
 #pragma unroll
         for (int e = 0; e < N; ++e) g[e] = sigmoid(g[e]);
+    }
+}
+// Gates and tokens of a vector from the stored values: g holds gate
+// pre-activations on entry and gates on exit; t holds the tokens, or for the
+// interpolating gate the values v on entry and (1 - gate) * v on exit.
+template <int ACT, class V, int N>
+__device__ __forceinline__ void activate_pair(V (&g)[N], V (&t)[N]) {
+    if constexpr (ACT == kGateSigmoidLerp) {
+#pragma unroll
+        for (int e = 0; e < N; ++e) {
+            float gate, complement;
+            sigmoid_pair(g[e], gate, complement);
+            g[e] = gate;
+            t[e] = complement * t[e];
+        }
+    } else {
+        activate<ACT>(g);
+    }
+}
+// Gates and their complements 1 - gate (the interpolating gate's backward pass).
+template <int ACT, class V, int N>
+__device__ __forceinline__ void activate_with_complement(V (&g)[N], V (&c)[N]) {
+    if constexpr (ACT == kGateSigmoidLerp) {
+#pragma unroll
+        for (int e = 0; e < N; ++e) {
+            float gate, complement;
+            sigmoid_pair(g[e], gate, complement);
+            g[e] = gate;
+            c[e] = complement;
+        }
+    } else {
+        activate<ACT>(g);
     }
 }
 template <int ACT, class V>
 __device__ __forceinline__ V activate1(V g) {
     if constexpr (ACT == kGateSigmoid) {
         return sigmoid(g);
+    } else if constexpr (ACT == kGateSigmoidLerp) {
+        float gate, complement;
+        sigmoid_pair(g, gate, complement);
+        return gate;
     } else {
         return g;
     }
@@ -41,13 +98,13 @@ __device__ __forceinline__ V activate1(V g) {
 // Stored value whose activation is the identity gate 1 (for out-of-row positions).
 template <int ACT, class V>
 __device__ __forceinline__ V identity_gate() {
-    if constexpr (ACT == kGateSigmoid) {
+    if constexpr (kGateIsSigmoid<ACT>) {
         return __builtin_inff();
     } else {
         return vone<V>();
     }
 }
-// d gate / d stored, from the gate's value.
+// d gate / d stored, from the gate's value (and, where known, its complement).
 template <int ACT, class V>
 __device__ __forceinline__ V gate_slope(V gate) {
     if constexpr (ACT == kGateSigmoid) {

@@ -13,6 +13,7 @@
 
 #include "ascan.h"
 #include "dispatch.h"
+#include "gate.h"
 #include "split.h"
 #include "traits.h"
 
@@ -296,9 +297,28 @@ Access choose_access(bool same_lead, int lead, int64_t T, int64_t tile) {
     return Access::kVector;
 }
 
-// Kernels with the sigmoid gate exist for the real dtypes, forward in time.
+// Kernels with the sigmoid gates exist for the real dtypes, forward in time.
 template <class Tr>
 constexpr bool kHasSigmoid = std::is_same<typename Tr::V, float>::value;
+
+// Calls f(std::integral_constant<int, ACT>) for the gate code `act`, which the
+// entry points have validated against the dtype.
+template <class Tr, class F>
+hipError_t with_gate(int act, F&& f) {
+    if constexpr (kHasSigmoid<Tr>) {
+        if (act == kGateSigmoid) return f(std::integral_constant<int, kGateSigmoid>{});
+        if (act == kGateSigmoidLerp) return f(std::integral_constant<int, kGateSigmoidLerp>{});
+    }
+    return f(std::integral_constant<int, kGateIdentity>{});
+}
+
+// The backward kernel of the interpolating gate holds a fourth input tensor in
+// registers and takes 2 KiB per wave and tile at most.
+template <int ACT>
+constexpr int backward_blocks(int blocks) {
+    return ACT == kGateSigmoidLerp && blocks > 2 ? 2 : blocks;
+}
+inline int backward_blocks_of(int act, int blocks) { return act == kGateSigmoidLerp && blocks > 2 ? 2 : blocks; }
 
 }  // namespace
 }  // namespace ascan

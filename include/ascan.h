@@ -62,7 +62,7 @@
 extern "C" {
 #endif
 
-#define ASCAN_ABI_VERSION 5
+#define ASCAN_ABI_VERSION 6
 
 /* Marks the exported entry points (the library is built with hidden visibility). */
 #define ASCAN_API __attribute__((visibility("default")))
@@ -99,7 +99,14 @@ enum ascan_status {
 /* What the kernels make of the stored gate values (the *_gated entry points). */
 enum ascan_gate {
     ASCAN_GATE_IDENTITY = 0, /* stored values are the gates: the reference's operator */
-    ASCAN_GATE_SIGMOID  = 1  /* gate = 1 / (1 + exp(-stored)); float32, bfloat16, float16 */
+    ASCAN_GATE_SIGMOID  = 1, /* gate = 1 / (1 + exp(-stored)); float32, bfloat16, float16 */
+    /*
+     * The same gate, and the second input holds values v rather than tokens:
+     * token = (1 - gate) * v, i.e. x[t] = gate * x[t-1] + (1 - gate) * v[t], the
+     * gated interpolation of linear-RNN layers.  Forward: ascan_forward_gated;
+     * backward: ascan_backward_lerp (it needs v).  float32, bfloat16, float16.
+     */
+    ASCAN_GATE_SIGMOID_LERP = 2
 };
 
 /*
@@ -235,8 +242,9 @@ ASCAN_API int ascan_backward_from(const void* gates, const void* states, const v
  *
  * with g, d_tokens and d_initial as in ascan_backward_from.  No counterpart in
  * the reference.  gate = ASCAN_GATE_IDENTITY makes these calls the *_from ones
- * (forward in time only); ASCAN_GATE_SIGMOID needs a real dtype, else
- * ASCAN_ERR_BAD_ACTIVATION.  The sigmoid is evaluated in fp32 with the
+ * (forward in time only); the sigmoid gates need a real dtype, else
+ * ASCAN_ERR_BAD_ACTIVATION (as does ASCAN_GATE_SIGMOID_LERP in
+ * ascan_backward_gated, which lacks the values: see ascan_backward_lerp).  The sigmoid is evaluated in fp32 with the
  * hardware's exp2 and reciprocal (about 2 ulp).
  */
 ASCAN_API int ascan_forward_gated(const void* gate_inputs, const void* tokens, const void* initial, void* out,
@@ -247,6 +255,26 @@ ASCAN_API int ascan_backward_gated(const void* gate_inputs, const void* states, 
                          const void* grad_out, void* d_gate_inputs, void* d_tokens, void* d_initial,
                          int64_t rows, int64_t seqlen, int dtype, int gate,
                          void* workspace, size_t workspace_bytes, void* stream);
+
+/*
+ * Backward pass of ascan_forward_gated(gate_inputs, values, ..., ASCAN_GATE_SIGMOID_LERP):
+ *
+ *     a[t]             = sigmoid(gate_inputs[t])
+ *     forward          : x[t] = a[t] * x[t-1] + (1 - a[t]) * values[t],   x[-1] = initial (NULL: 0)
+ *     g[t]             = grad_out[t] + a[t+1] * g[t+1]
+ *     d_values[t]      = g[t] * (1 - a[t])
+ *     d_gate_inputs[t] = g[t] * (x[t-1] - values[t]) * a[t] * (1 - a[t])
+ *     d_initial        = a[0] * g[0]
+ *
+ * One fused reverse-time pass: 4 tensors read, 2 written (against 3 + 2 for the
+ * scan alone plus three elementwise passes over 11 tensors for the token
+ * product and its gradient when they are done outside).  1 - a is evaluated as
+ * sigmoid(-gate_inputs), not as a difference.  No counterpart in the reference.
+ */
+ASCAN_API int ascan_backward_lerp(const void* gate_inputs, const void* values, const void* states, const void* initial,
+                        const void* grad_out, void* d_gate_inputs, void* d_values, void* d_initial,
+                        int64_t rows, int64_t seqlen, int dtype,
+                        void* workspace, size_t workspace_bytes, void* stream);
 
 /* Static, human-readable text for an ascan_status code. */
 ASCAN_API const char* ascan_status_string(int status);

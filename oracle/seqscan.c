@@ -272,3 +272,49 @@ void seq_backward_sigmoid_f32(const float* z, const float* state, const float* i
         if (dinit) dinit[r] = (T > 0) ? sigmoid64((double)zr[0]) * a : 0.0;
     }
 }
+
+/*
+ * Gated interpolation (no counterpart in the reference): the gate is the
+ * sigmoid of a stored pre-activation and the token its complement times a
+ * stored value,
+ *   a[t] = 1 / (1 + exp(-z[t])),  out[t] = a[t] * out[t-1] + (1 - a[t]) * v[t],  out[-1] = init
+ *   g[t] = dout[t] + a[t+1] * g[t+1]
+ *   dv[t] = g[t] * (1 - a[t]),  dz[t] = g[t] * (state[t-1] - v[t]) * a[t] * (1 - a[t]),  dinit = a[0] * g[0]
+ * 1 - a is taken as 1 / (1 + exp(z)), which keeps its relative accuracy for
+ * large z.  Pinned by tests/test_oracle.py: torch autograd through the plain
+ * float64 loop with torch.sigmoid and torch.lerp, the sigmoid functions above
+ * on tokens (1 - sigmoid(z)) * v formed in float64, and closed forms (constant
+ * v gives out = v for init = v; z = 0 gives the running average with weights
+ * 2^-(k+1)).
+ */
+void seq_forward_lerp_f32(const float* z, const float* v, const float* init, double* out, int64_t rows, int64_t T) {
+#pragma omp parallel for schedule(static)
+    for (int64_t r = 0; r < rows; ++r) {
+        double s = init ? (double)init[r] : 0.0;
+        for (int64_t t = 0; t < T; ++t) {
+            const double zt = (double)z[r * T + t];
+            s = sigmoid64(zt) * s + sigmoid64(-zt) * (double)v[r * T + t];
+            out[r * T + t] = s;
+        }
+    }
+}
+
+void seq_backward_lerp_f32(const float* z, const float* v, const float* state, const float* init, const float* dout,
+                           double* dz, double* dv, double* dinit, int64_t rows, int64_t T) {
+#pragma omp parallel for schedule(static)
+    for (int64_t r = 0; r < rows; ++r) {
+        const float* zr = z + r * T;
+        const float* vr = v + r * T;
+        const float* sr = state + r * T;
+        const double x0 = init ? (double)init[r] : 0.0;
+        double g = 0.0;
+        for (int64_t t = T - 1; t >= 0; --t) {
+            const double gnext = (t + 1 < T) ? sigmoid64((double)zr[t + 1]) : 1.0;
+            g = (double)dout[r * T + t] + gnext * g;
+            const double a = sigmoid64((double)zr[t]), rest = sigmoid64(-(double)zr[t]);
+            dv[r * T + t] = g * rest;
+            dz[r * T + t] = g * (((t > 0) ? (double)sr[t - 1] : x0) - (double)vr[t]) * a * rest;
+        }
+        if (dinit) dinit[r] = (T > 0) ? sigmoid64((double)zr[0]) * g : 0.0;
+    }
+}

@@ -39,9 +39,12 @@ def _load():
         lib.seq_backward_from_c64.argtypes = [p, p, p, p, p, p, p, i64, i64]
         lib.seq_forward_sigmoid_f32.argtypes = [p, p, p, p, i64, i64]
         lib.seq_backward_sigmoid_f32.argtypes = [p, p, p, p, p, p, p, i64, i64]
+        lib.seq_forward_lerp_f32.argtypes = [p, p, p, p, i64, i64]
+        lib.seq_backward_lerp_f32.argtypes = [p, p, p, p, p, p, p, p, i64, i64]
         for f in (lib.seq_forward_f32, lib.seq_forward_c64, lib.seq_backward_f32, lib.seq_backward_c64,
                   lib.seq_forward_from_f32, lib.seq_forward_from_c64, lib.seq_backward_from_f32,
-                  lib.seq_backward_from_c64, lib.seq_forward_sigmoid_f32, lib.seq_backward_sigmoid_f32):
+                  lib.seq_backward_from_c64, lib.seq_forward_sigmoid_f32, lib.seq_backward_sigmoid_f32,
+                  lib.seq_forward_lerp_f32, lib.seq_backward_lerp_f32):
             f.restype = None
         _lib = lib
     return _lib
@@ -164,3 +167,44 @@ def backward_sigmoid(gate_logits, states, grad_out, initial=None):
         lib.seq_backward_sigmoid_f32(zp, sp, ip, dp, dz.ctypes.data_as(ctypes.c_void_p),
                                      dx.ctypes.data_as(ctypes.c_void_p), di.ctypes.data_as(ctypes.c_void_p), rows, T)
     return dz, dx, di
+
+
+def forward_lerp(gate_logits, values, initial=None):
+    """Sequential gated interpolation in fp64:
+    x[t] = a[t] * x[t-1] + (1 - a[t]) * values[t], a = sigmoid(gate_logits) (real inputs)."""
+    lib = _load()
+    z, zp = _prep(gate_logits, np.float32)
+    v, vp = _prep(values, np.float32)
+    assert z.shape == v.shape
+    ip = None
+    if initial is not None:
+        i, ip = _prep(initial, np.float32)
+        assert i.shape == z.shape[:-1]
+    T = z.shape[-1]
+    rows = z.size // T if T else 0
+    out = np.empty(z.shape, dtype=np.float64)
+    lib.seq_forward_lerp_f32(zp, vp, ip, out.ctypes.data_as(ctypes.c_void_p), rows, T)
+    return out
+
+
+def backward_lerp(gate_logits, values, states, grad_out, initial=None):
+    """(d_gate_logits, d_values, d_initial) of the gated interpolation, in fp64."""
+    lib = _load()
+    z, zp = _prep(gate_logits, np.float32)
+    v, vp = _prep(values, np.float32)
+    s, sp = _prep(states, np.float32)
+    d, dp = _prep(grad_out, np.float32)
+    assert z.shape == v.shape == s.shape == d.shape
+    ip = None
+    if initial is not None:
+        i, ip = _prep(initial, np.float32)
+        assert i.shape == z.shape[:-1]
+    T = z.shape[-1]
+    rows = z.size // T if T else 0
+    dz = np.empty(z.shape, dtype=np.float64)
+    dv = np.empty(z.shape, dtype=np.float64)
+    di = np.zeros(z.shape[:-1], dtype=np.float64)
+    if rows:
+        lib.seq_backward_lerp_f32(zp, vp, sp, ip, dp, dz.ctypes.data_as(ctypes.c_void_p),
+                                  dv.ctypes.data_as(ctypes.c_void_p), di.ctypes.data_as(ctypes.c_void_p), rows, T)
+    return dz, dv, di

@@ -1,5 +1,5 @@
 // C ABI check without Python or torch: a plain HIP host program that links
-// libascan.so through include/ascan.h, drives every entry point with buffers
+// libascan.so through include/ascan.h, drives every compute entry point with buffers
 // from hipMalloc on a stream of its own, and compares the results with the
 // sequential fp64 loops of the test oracle (oracle/seqscan.c).  Also checks the
 // status codes of invalid calls.  Exit status 0 and a final "ok" line on success.
@@ -18,6 +18,12 @@ void seq_forward_from_f32(const float* g, const float* x, const float* init, dou
                           int reverse);
 void seq_backward_from_f32(const float* g, const float* state, const float* init, const float* dout, double* dg,
                            double* dx, double* dinit, int64_t rows, int64_t T);
+void seq_forward_sigmoid_f32(const float* z, const float* x, const float* init, double* out, int64_t rows, int64_t T);
+void seq_backward_sigmoid_f32(const float* z, const float* state, const float* init, const float* dout, double* dz,
+                              double* dx, double* dinit, int64_t rows, int64_t T);
+void seq_forward_lerp_f32(const float* z, const float* v, const float* init, double* out, int64_t rows, int64_t T);
+void seq_backward_lerp_f32(const float* z, const float* v, const float* state, const float* init, const float* dout,
+                           double* dz, double* dv, double* dinit, int64_t rows, int64_t T);
 }
 
 #define HIP_OK(call)                                                                          \
@@ -137,6 +143,66 @@ void check_problem(int64_t rows, int64_t T, bool with_initial, hipStream_t strea
     }
 }
 
+// The gated entry points (sigmoid gate; sigmoid gate with interpolated values) and the
+// split-row forward scan whose table is the library's static array.
+void check_gated_and_static(int64_t rows, int64_t T, hipStream_t stream) {
+    std::printf("gated rows=%lld T=%lld\n", (long long)rows, (long long)T);
+    std::fflush(stdout);
+    const size_t n = (size_t)rows * (size_t)T;
+    Lcg rng{(uint64_t)(rows * 7919 + T)};
+    std::vector<float> z(n), x(n), d(n), init(rows);
+    for (size_t i = 0; i < n; ++i) {
+        z[i] = 8.0f * rng.uniform() - 3.0f;
+        x[i] = 2.0f * rng.uniform() - 1.0f;
+        d[i] = 2.0f * rng.uniform() - 1.0f;
+    }
+    for (auto& v : init) v = 4.0f * rng.uniform() - 2.0f;
+    DeviceBuffer dz_in(n * 4), dx_in(n * 4), dd_in(n * 4), dinit_in(rows * 4);
+    DeviceBuffer out(n * 4), d_z(n * 4), d_x(n * 4), d_init(rows * 4);
+    upload(dz_in, z, stream);
+    upload(dx_in, x, stream);
+    upload(dd_in, d, stream);
+    upload(dinit_in, init, stream);
+    const size_t ws_bytes = ascan_workspace_bytes(rows, T, ASCAN_F32);
+    DeviceBuffer ws(ws_bytes);
+    void* ws_ptr = ws_bytes ? ws.p : nullptr;
+    std::vector<double> t_out(n), t_dz(n), t_dx(n), t_di(rows);
+    const double tol = 4e-5;  // the in-kernel sigmoid (about 2 ulp) enters every gate
+
+    EXPECT(ascan_forward_gated(dz_in.p, dx_in.p, dinit_in.p, out.p, rows, T, ASCAN_F32, ASCAN_GATE_SIGMOID, ws_ptr,
+                               ws_bytes, stream) == ASCAN_OK);
+    EXPECT(ascan_backward_gated(dz_in.p, out.p, dinit_in.p, dd_in.p, d_z.p, d_x.p, d_init.p, rows, T, ASCAN_F32,
+                                ASCAN_GATE_SIGMOID, ws_ptr, ws_bytes, stream) == ASCAN_OK);
+    std::vector<float> h_out = download(out, n, stream);
+    seq_forward_sigmoid_f32(z.data(), x.data(), init.data(), t_out.data(), rows, T);
+    seq_backward_sigmoid_f32(z.data(), h_out.data(), init.data(), d.data(), t_dz.data(), t_dx.data(), t_di.data(), rows, T);
+    EXPECT(worst(h_out, t_out) <= tol);
+    EXPECT(worst(download(d_z, n, stream), t_dz) <= tol);
+    EXPECT(worst(download(d_x, n, stream), t_dx) <= tol);
+    EXPECT(worst(download(d_init, rows, stream), t_di) <= tol);
+
+    EXPECT(ascan_forward_gated(dz_in.p, dx_in.p, dinit_in.p, out.p, rows, T, ASCAN_F32, ASCAN_GATE_SIGMOID_LERP, ws_ptr,
+                               ws_bytes, stream) == ASCAN_OK);
+    EXPECT(ascan_backward_lerp(dz_in.p, dx_in.p, out.p, dinit_in.p, dd_in.p, d_z.p, d_x.p, d_init.p, rows, T, ASCAN_F32,
+                               ws_ptr, ws_bytes, stream) == ASCAN_OK);
+    h_out = download(out, n, stream);
+    seq_forward_lerp_f32(z.data(), x.data(), init.data(), t_out.data(), rows, T);
+    seq_backward_lerp_f32(z.data(), x.data(), h_out.data(), init.data(), d.data(), t_dz.data(), t_dx.data(), t_di.data(),
+                          rows, T);
+    EXPECT(worst(h_out, t_out) <= tol);
+    EXPECT(worst(download(d_z, n, stream), t_dz) <= tol);
+    EXPECT(worst(download(d_x, n, stream), t_dx) <= tol);
+    EXPECT(worst(download(d_init, rows, stream), t_di) <= tol);
+
+    // static-table forward scan: stored values in [0, 1) as gates (x from a zero state)
+    std::vector<float> g(n);
+    for (size_t i = 0; i < n; ++i) g[i] = rng.uniform();
+    upload(dz_in, g, stream);
+    EXPECT(ascan_forward_split_static(dz_in.p, dx_in.p, out.p, rows, T, ASCAN_F32, 0, stream) == ASCAN_OK);
+    seq_forward_from_f32(g.data(), x.data(), nullptr, t_out.data(), rows, T, 0);
+    EXPECT(worst(download(out, n, stream), t_out) <= 2e-5);
+}
+
 void check_status_codes(hipStream_t stream) {
     DeviceBuffer a(4096), b(4096), c(4096);
     EXPECT(ascan_abi_version() == ASCAN_ABI_VERSION);
@@ -161,6 +227,16 @@ void check_status_codes(hipStream_t stream) {
     EXPECT(ascan_workspace_bytes(100000, 65536, ASCAN_F32) == 0);
     EXPECT(ascan_workspace_bytes(2, 1 << 20, ASCAN_F32) > 0);
     EXPECT(ascan_status_string(ASCAN_ERR_MISALIGNED) != nullptr);
+    // gates: unknown code; a sigmoid gate with a complex dtype; the interpolating gate without its values
+    EXPECT(ascan_forward_gated(a.p, b.p, nullptr, c.p, 1, 16, ASCAN_F32, 9, nullptr, 0, stream) == ASCAN_ERR_BAD_ACTIVATION);
+    EXPECT(ascan_forward_gated(a.p, b.p, nullptr, c.p, 1, 16, ASCAN_C64, ASCAN_GATE_SIGMOID_LERP, nullptr, 0, stream) ==
+           ASCAN_ERR_BAD_ACTIVATION);
+    EXPECT(ascan_backward_gated(a.p, b.p, nullptr, c.p, (char*)a.p + 1024, (char*)a.p + 2048, nullptr, 1, 16, ASCAN_F32,
+                                ASCAN_GATE_SIGMOID_LERP, nullptr, 0, stream) == ASCAN_ERR_BAD_ACTIVATION);
+    EXPECT(ascan_backward_lerp(a.p, nullptr, b.p, nullptr, c.p, (char*)a.p + 1024, (char*)a.p + 2048, nullptr, 1, 16,
+                               ASCAN_F32, nullptr, 0, stream) == ASCAN_ERR_NULL_POINTER);
+    // the static-table entry point refuses what does not fit its array
+    EXPECT(ascan_forward_split_static(a.p, b.p, c.p, 128, 1 << 24, ASCAN_F32, 0, stream) == ASCAN_ERR_TOO_LARGE);
 }
 
 }  // namespace
@@ -178,6 +254,8 @@ int main() {
         check_problem(p[0], p[1], false, stream);
         check_problem(p[0], p[1], true, stream);
     }
+    const int64_t gated[][2] = {{9, 40}, {300, 1024}, {64, 4099}, {12, 65536}, {3, 300000}};
+    for (const auto& p : gated) check_gated_and_static(p[0], p[1], stream);
     HIP_OK(hipStreamSynchronize(stream));
     HIP_OK(hipStreamDestroy(stream));
     std::printf("ok\n");

@@ -355,3 +355,62 @@ def test_sigmoid_vs_plain_scan_of_rounded_gates_and_closed_form():
     x = tokens[:1, :1, :50].numpy()
     np.testing.assert_allclose(seqscan.forward_sigmoid(np.full_like(x, 40.0), x), np.cumsum(x.astype(np.float64), -1), rtol=1e-12, atol=1e-12)
     np.testing.assert_allclose(seqscan.forward_sigmoid(np.full_like(x, -40.0), x), x, rtol=1e-12, atol=1e-12)
+
+
+# ---------------------------------------------------------------------------
+# Gated interpolation x[t] = a x[t-1] + (1 - a) v[t], a = sigmoid(z) (oracle functions *_lerp)
+# ---------------------------------------------------------------------------
+@pytest.mark.parametrize("T", [1, 2, 9, 64])
+@pytest.mark.parametrize("with_initial", [False, True])
+def test_lerp_vs_autograd_of_loop(T, with_initial):
+    """Values and all three gradients against torch autograd through the explicit
+    float64 loop written with torch.lerp (x = lerp(v, x_prev, a))."""
+    gen = torch.Generator().manual_seed(900 + T)
+    logits = 3.0 * torch.randn(2, 2, T, generator=gen)
+    values, grad_out = (torch.randn(2, 2, T, generator=gen) for _ in range(2))
+    initial = torch.randn(2, 2, generator=gen) if with_initial else torch.zeros(2, 2)
+    zw, vw, iw = (t.double().requires_grad_(True) for t in (logits, values, initial))
+    a = torch.sigmoid(zw)
+    state, outs = iw, []
+    for t in range(T):
+        state = torch.lerp(vw[..., t], state, a[..., t])
+        outs.append(state)
+    out = torch.stack(outs, dim=-1)
+    dz_ref, dv_ref, di_ref = torch.autograd.grad(out, (zw, vw, iw), grad_out.double())
+    init_arg = initial.numpy() if with_initial else None
+    fwd = seqscan.forward_lerp(logits.numpy(), values.numpy(), init_arg)
+    np.testing.assert_allclose(fwd, out.detach().numpy(), rtol=1e-12, atol=1e-12)
+    dz, dv, di = seqscan.backward_lerp(logits.numpy(), values.numpy(), fwd.astype(np.float32), grad_out.numpy(), init_arg)
+    np.testing.assert_allclose(dv, dv_ref.numpy(), rtol=1e-12, atol=1e-12)
+    np.testing.assert_allclose(di, di_ref.numpy(), rtol=1e-12, atol=1e-12)
+    np.testing.assert_allclose(dz, dz_ref.numpy(), rtol=1e-5, atol=1e-5)  # states rounded to fp32 before the subtraction
+
+
+def test_lerp_vs_sigmoid_scan_of_formed_tokens_and_closed_forms():
+    gen = torch.Generator().manual_seed(23)
+    logits = 2.0 * torch.randn(3, 4, 200, generator=gen)
+    values, grad_out = (torch.randn(3, 4, 200, generator=gen) for _ in range(2))
+    a = torch.sigmoid(logits.double())
+    tokens = ((1 - a) * values.double())
+    fwd = seqscan.forward_lerp(logits.numpy(), values.numpy())
+    # the sigmoid-gated scan of the tokens (1 - a) v formed outside (rounded to fp32 on that side)
+    np.testing.assert_allclose(fwd, seqscan.forward_sigmoid(logits.numpy(), tokens.float().numpy()), rtol=1e-5, atol=1e-5)
+    states = fwd.astype(np.float32)
+    dz, dv, _ = seqscan.backward_lerp(logits.numpy(), values.numpy(), states, grad_out.numpy())
+    dz_scan, dt, _ = seqscan.backward_sigmoid(logits.numpy(), states, grad_out.numpy())
+    # chain rule through tokens = (1 - a) v:  d_v = d_tokens (1 - a);  d_z = d_z(scan) - d_tokens v a (1 - a)
+    np.testing.assert_allclose(dv, dt * (1 - a).numpy(), rtol=1e-10, atol=1e-12)
+    np.testing.assert_allclose(dz, dz_scan - dt * (values.double() * a * (1 - a)).numpy(), rtol=1e-8, atol=1e-10)
+    # a constant value is a fixed point: started from it, the state never moves, whatever the gates
+    v = np.full((2, 3, 40), 1.75, np.float32)
+    z = (3 * torch.randn(2, 3, 40, generator=gen)).numpy()
+    np.testing.assert_allclose(seqscan.forward_lerp(z, v, np.full((2, 3), 1.75, np.float32)), 1.75, rtol=1e-14)
+    # z = 0: every gate is 1/2; unit values from a zero state give 1 - 2^-(t+1)
+    T = 30
+    out = seqscan.forward_lerp(np.zeros((1, 1, T), np.float32), np.ones((1, 1, T), np.float32))
+    np.testing.assert_allclose(out[0, 0], 1.0 - 0.5 ** (np.arange(T) + 1), rtol=1e-15)
+    # saturated gates: z = -40 returns the values, z = +40 keeps the initial state
+    x = values[:1, :1, :50].numpy()
+    np.testing.assert_allclose(seqscan.forward_lerp(np.full_like(x, -40.0), x), x, rtol=1e-12, atol=1e-12)
+    np.testing.assert_allclose(seqscan.forward_lerp(np.full_like(x, 40.0), x, np.full((1, 1), 0.5, np.float32)), 0.5,
+                               rtol=1e-12, atol=1e-12)

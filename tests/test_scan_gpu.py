@@ -526,11 +526,14 @@ def test_config5_complex64_forward_backward():
     assert _rel_err(dg[:, rows], t_dg) <= 1e-5
 
 
-def test_target_shape_fp32_properties():
+@pytest.mark.parametrize("seqlen", [65536, 49152], ids=["T65536", "T49152_rows_192KiB_apart"])
+def test_target_shape_fp32_properties(seqlen):
     """(8, 1536, 65536) fp32, forward + backward, checked without a full-size oracle:
     sampled rows against the fp64 recurrence and the adjoint identity
-    <grad_out, scan(g, x)> = <d_tokens, x> (the scan is linear in the tokens)."""
-    shape = (8, 1536, 65536)
+    <grad_out, scan(g, x)> = <d_tokens, x> (the scan is linear in the tokens).
+    Also at T = 49152: the same mask-free kernels with rows that are not a power
+    of two bytes apart (three 64 KiB tiles per row)."""
+    shape = (8, 1536, seqlen)
     torch.manual_seed(12312323)
     gates = 0.999 + 0.001 * torch.rand(*shape, device=DEVICE)
     tokens = torch.rand(*shape, device=DEVICE)
