@@ -78,9 +78,12 @@ int backward_typed(const BackwardBuffers& b, int64_t rows, int64_t T, int act, c
     const Lead at = find_lead<Tr>(state_like, b.d_tokens);
     const bool same_lead = at.same;
     const int lead = at.lead;
-    Plan plan = choose_plan(T, SUB, kElem, kTrimPlan<Tr>);
+    // the interpolating gate's kernels (half-size tiles, a fourth input, more arithmetic per element) gain from a
+    // narrower plan for a mostly empty last tile whatever the dtype: fp32 (8,1536,9000) backward 4.9 -> 5.5 TB/s
+    const bool trim = kTrimPlan<Tr> || act == kGateSigmoidLerp;
+    Plan plan = choose_plan(T, SUB, kElem, trim);
     const Access access = choose_access(same_lead, lead, T, SUB * plan.waves_per_row);
-    if (access != Access::kRegular) plan = choose_plan(T, SUBG, kElem, kTrimPlan<Tr>);
+    if (access != Access::kRegular) plan = choose_plan(T, SUBG, kElem, trim);
     const int R = plan.rows_per_block;
     hipError_t err = hipSuccess;
     // 16-bit rows of 512 bytes and more, vectorised flavour, plenty of them: groups of the wider workgroup

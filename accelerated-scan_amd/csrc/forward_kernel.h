@@ -111,6 +111,25 @@ __global__ void __launch_bounds__(64 * kMaxWavesPerBlock)
                                         (int)(sub_base - lo), (int)SUB, stage_all + w * SUB, lane);
         }
 
+        // A sub-tile that holds nothing of the row (the waves past the row's end in its last
+        // tile step) contributes the identity to the scan: the wave passes the carry on and
+        // is done, instead of running both passes over filler values.  With one workgroup per
+        // compute unit that arithmetic is not hidden: four waves share a SIMD, and a tile step
+        // that moves a few elements would still cost the vector ALU time of a full one.
+        if constexpr (!FULL && !SPLIT) {
+            if (!touches) {  // wave-uniform
+                V totA[U], totX[U];
+#pragma unroll
+                for (int j = 0; j < U; ++j) {
+                    totA[j] = vone<V>();
+                    totX[j] = vzero<V>();
+                }
+                V c;
+                exchange_carries<V, W, U, PACKED>(totA, totX, carry, c, slots, (int)(k & 1), w, lane);
+                return;
+            }
+        }
+
         u32x4_t graw[U], traw[U];
         if (touches) {
 #pragma unroll

@@ -12,7 +12,10 @@
 //              long rows, without their barrier;
 //   pattern 2  row walk with one workgroup barrier per tile;
 //   pattern 3  linear sweep in the row walk's units: workgroup i moves the i-th
-//              tile of every tensor (barrier) and ends.
+//              tile of every tensor (barrier) and ends;
+//   pattern 4  row walk by `row_step` persistent workgroups: workgroup b walks
+//              rows b, b + row_step, ... (fewer rows in flight than compute units
+//              when row_step is below their number).
 // `blocks_per_wave` in {1, 2, 4, 8} sets the tile of patterns 1-3: that many KiB
 // per wave, 16 times as much per workgroup (the scan kernels: 4, 64 KiB tiles).
 // `row_step` > 1 (patterns 1, 2) hands consecutive workgroups rows that far apart.
@@ -56,14 +59,16 @@ __global__ void __launch_bounds__(kThreads) stream_probe_linear(Tensors t) {
 }
 
 template <int NR, int NW, bool BARRIER, int BPW>
-__global__ void __launch_bounds__(kThreads) stream_probe_rows(Tensors t, int64_t row_vectors, int row_step) {
+__global__ void __launch_bounds__(kThreads) stream_probe_rows(Tensors t, int64_t row_vectors, int row_step, int64_t rows) {
     constexpr int kBlocksPerWave = BPW;
     constexpr int64_t kTile = tile_bytes(BPW);
     const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
     // one row per workgroup; with row_vectors == one tile, the launch is a linear sweep in tiles.
-    // row_step > 1: consecutive workgroups take rows row_step apart (all rows are still covered)
-    const int64_t per_pass = gridDim.x / row_step;
-    const int64_t row_index = row_step > 1 ? (blockIdx.x % per_pass) * row_step + blockIdx.x / per_pass : blockIdx.x;
+    // row_step > 1: consecutive workgroups take rows row_step apart (all rows are still covered).
+    // rows > gridDim.x (pattern 4): the workgroups are persistent and take rows b, b + gridDim.x, ...
+    for (int64_t first = blockIdx.x; first < rows; first += gridDim.x) {
+    const int64_t per_pass = rows / row_step;
+    const int64_t row_index = row_step > 1 ? (first % per_pass) * row_step + first / per_pass : first;
     const int64_t row = row_index * row_vectors;
     for (int64_t tile = 0; tile < row_vectors; tile += kTile / 16) {
         const int64_t base = row + tile + (int64_t)wave * (64 * kBlocksPerWave) + lane;
@@ -82,6 +87,7 @@ __global__ void __launch_bounds__(kThreads) stream_probe_rows(Tensors t, int64_t
             if constexpr (NW == 0) keep(s[j], t.out[0] + base + j * 64);
         }
     }
+    }
 }
 
 template <class K>
@@ -99,14 +105,17 @@ hipError_t launch_rows(const Tensors& t, int64_t rows, int64_t row_bytes, int pa
     if (e != hipSuccess) return e;
     if (pattern == 1) {
         hipLaunchKernelGGL((stream_probe_rows<NR, NW, false, BPW>), dim3((unsigned)rows), dim3(kThreads), lds_bytes,
-                           stream, t, row_bytes / 16, row_step);
+                           stream, t, row_bytes / 16, row_step, rows);
     } else if (pattern == 2) {
         hipLaunchKernelGGL((stream_probe_rows<NR, NW, true, BPW>), dim3((unsigned)rows), dim3(kThreads), lds_bytes,
-                           stream, t, row_bytes / 16, row_step);
+                           stream, t, row_bytes / 16, row_step, rows);
+    } else if (pattern == 4) {  // row_step is the number of persistent workgroups
+        hipLaunchKernelGGL((stream_probe_rows<NR, NW, true, BPW>), dim3((unsigned)row_step), dim3(kThreads), lds_bytes,
+                           stream, t, row_bytes / 16, 1, rows);
     } else {
         const int64_t tiles = rows * row_bytes / tile_bytes(BPW);
         hipLaunchKernelGGL((stream_probe_rows<NR, NW, true, BPW>), dim3((unsigned)tiles), dim3(kThreads), lds_bytes,
-                           stream, t, tile_bytes(BPW) / 16, 1);
+                           stream, t, tile_bytes(BPW) / 16, 1, tiles);
     }
     return hipGetLastError();
 }
@@ -135,8 +144,8 @@ hipError_t launch(const Tensors& t, int64_t rows, int64_t row_bytes, int pattern
 extern "C" __attribute__((visibility("default"))) int stream_probe_launch(
     const void* in0, const void* in1, const void* in2, void* out0, void* out1, int64_t rows, int64_t row_bytes,
     int reads, int writes, int pattern, int blocks_per_wave, int row_step, unsigned lds_bytes, void* stream) {
-    if (row_step < 1 || rows % row_step != 0) return -1;
-    if (rows <= 0 || row_bytes <= 0 || pattern < 0 || pattern > 3 || lds_bytes > 160u * 1024u) return -1;
+    if (row_step < 1 || (pattern != 4 && rows % row_step != 0)) return -1;
+    if (rows <= 0 || row_bytes <= 0 || pattern < 0 || pattern > 4 || lds_bytes > 160u * 1024u) return -1;
     if (blocks_per_wave != 1 && blocks_per_wave != 2 && blocks_per_wave != 4 && blocks_per_wave != 8) return -1;
     if (pattern == 0 ? (rows * row_bytes) % kChunk != 0 : row_bytes % tile_bytes(blocks_per_wave) != 0) return -1;
     if (rows * row_bytes / kChunk > 2147483647LL || rows > 2147483647LL) return -1;
