@@ -66,18 +66,23 @@ const Plan& forced_plan() {
 // Measured on MI355X: what counts is how few rows are being streamed at any
 // one time.  With every wave on its own row the memory system sees thousands
 // of concurrent streams and tops out near 5.0 TB/s; with 16 waves marching
-// along one row it reaches the 5.7-6.1 TB/s of a plain linear sweep.  So a row
+// along one row it reaches 5.6-6.1 TB/s.  So a row
 // gets as many waves as it has sub-tiles (up to 16).  Short rows keep small
 // workgroups (256 threads, several rows each): packing more short rows into
 // one large workgroup measured slower.
 //
-// `trim`: a row is scanned in whole tiles of w sub-tiles, and when its last
-// tile would be mostly empty fewer waves per row leave fewer wave slots idle
-// (20000 bf16 elements in tiles of 16384: the second tile is a fifth full).  The
-// 16-bit and the complex kernels gain from a narrower plan when more than 30 %
-// of the slots would idle (bf16 backward at T = 20000: 0.65 -> 0.46 ms,
-// complex64 forward at T = 4500: 0.152 -> 0.121 ms; below that waste they lose
-// ~5 %); the fp32 kernels lose up to 10 % at every waste and keep w.
+// `trim`: a row is scanned in whole tiles of w sub-tiles, and the last tile may be mostly empty
+// (20000 bf16 elements in tiles of 16384: the second tile is a fifth full).  Waves without
+// any of the row in their sub-tile only pass the carry on, so the empty part costs little
+// arithmetic, but every tile step costs a round trip to memory and a barrier, and with 16 waves
+// per row nothing else runs on the compute unit meanwhile.  Measured over T = 2500..45000 with
+// every plan forced in turn (16-bit at (8,1536,T), complex64 at (8,768,T)), the fastest plan is
+// the widest one that (a) leaves at most a third of its wave slots empty (a quarter with 16 waves), (b) is not a single tile
+// step with more than a fifth of it empty (two steps of half the width do better: the second
+// step's loads overlap the first one's stores), and (c) is not a single step of 16 waves at all.
+// That rule is within 4 % of the best plan at every length tried but one (bf16 T = 6000, 12 %).
+// The fp32 kernels do less arithmetic per byte and are within 2 % of their best plan untrimmed
+// (fp32 T = 9000 forward: 6 %), so they keep w -- except the interpolating gate's backward kernel.
 template <class Tr>
 constexpr bool kTrimPlan = Tr::kNarrow || !std::is_same<typename Tr::V, float>::value;
 
@@ -87,19 +92,27 @@ Plan choose_plan(int64_t T, int64_t sub, int64_t element_bytes, bool trim) {
     int w = 1;
     while (w < kMaxWavesPerBlock && (int64_t)w * 4096 < T * element_bytes && (int64_t)w * sub < T) w *= 2;
     if (trim) {
+        auto steps = [&](int waves) { return (T + (int64_t)waves * sub - 1) / ((int64_t)waves * sub); };
         // wave slots (of `sub` elements each) a row occupies over all its tile steps
-        auto slots = [&](int waves) { return (T + (int64_t)waves * sub - 1) / ((int64_t)waves * sub) * waves; };
-        if (slots(w) * sub * 10 > T * 13) {
-            int best = w;
-            for (int v = w / 2; v >= 1; v /= 2) {
-                if (slots(v) * sub * 100 <= T * 115) {  // the widest plan that wastes at most 15 %
-                    best = v;
-                    break;
-                }
-                if (slots(v) < slots(best)) best = v;
+        auto slots = [&](int waves) { return steps(waves) * waves; };
+        auto acceptable = [&](int waves) {
+            const int64_t covered = slots(waves) * sub;
+            if (waves == kMaxWavesPerBlock ? covered * 3 > T * 4 : covered * 2 > T * 3) return false;  // (a)
+            if (steps(waves) == 1 && waves > 1 && covered * 5 > T * 6) return false;        // (b)
+            if (steps(waves) == 1 && waves == kMaxWavesPerBlock && covered > T) return false;  // (c)
+            return true;
+        };
+        int best = w;
+        bool found = false;
+        for (int v = w; v >= 1 && !found; v /= 2) {
+            if (acceptable(v)) {
+                best = v;
+                found = true;
+            } else if (slots(v) < slots(best)) {
+                best = v;  // nothing acceptable so far: remember the plan with the fewest slots
             }
-            w = best;
         }
+        w = best;
     }
     if (forced.waves_per_row) w = forced.waves_per_row;
     int r = w >= 4 ? 1 : 4 / w;
