@@ -149,12 +149,25 @@ __global__ void __launch_bounds__(64 * kMaxWavesPerBlock)
         // Pass 1: fold each vector into one (A, X) pair and scan the pairs.
         V totA[U], totX[U], exA[U], exX[U];
         CutAt<V> cut_found[PACKED ? U : 1];  // packed rows: where each vector is cut, kept for pass 2
+        // 16-bit storage with a gate non-linearity: eight exponentials and reciprocals per vector and
+        // pass make the vector ALU the limit (about 5.4 TB/s for the interpolating gate), so the
+        // activated gates and tokens of pass 1 are kept for pass 2; the raw vectors are dead by then.
+        // Everywhere else unpacking again is cheaper than the registers (the split-row kernels would spill).
+        constexpr bool KEEP = Tr::kNarrow && ACT != kGateIdentity && !PACKED && !SPLIT;
+        V gkeep[KEEP ? U : 1][EPV], tkeep[KEEP ? U : 1][EPV];
 #pragma unroll
         for (int j = 0; j < U; ++j) {
             V g[EPV], t[EPV];
             Tr::unpack(graw[j], g);
             Tr::unpack(traw[j], t);
             activate_pair<ACT>(g, t);
+            if constexpr (KEEP) {
+#pragma unroll
+                for (int e = 0; e < EPV; ++e) {
+                    gkeep[j][e] = g[e];
+                    tkeep[j][e] = t[e];
+                }
+            }
             if constexpr (PACKED) {
                 const int rel = (int)(sub_base - lo) + vec_offset<U, EPV, REV>(j, lane);
                 cut_found[j] = locate_cut<Tr, REV>(rel, cuts);
@@ -201,14 +214,22 @@ __global__ void __launch_bounds__(64 * kMaxWavesPerBlock)
         // Pass 2: the plain recurrence from the state entering each lane.
 #pragma unroll
         for (int j = 0; j < U; ++j) {
-            if constexpr (Tr::kNarrow) {
-                forget_unpacked(graw[j]);
-                forget_unpacked(traw[j]);
-            }
             V g[EPV], t[EPV];
-            Tr::unpack(graw[j], g);
-            Tr::unpack(traw[j], t);
-            activate_pair<ACT>(g, t);
+            if constexpr (KEEP) {
+#pragma unroll
+                for (int e = 0; e < EPV; ++e) {
+                    g[e] = gkeep[j][e];
+                    t[e] = tkeep[j][e];
+                }
+            } else {
+                if constexpr (Tr::kNarrow) {
+                    forget_unpacked(graw[j]);
+                    forget_unpacked(traw[j]);
+                }
+                Tr::unpack(graw[j], g);
+                Tr::unpack(traw[j], t);
+                activate_pair<ACT>(g, t);
+            }
             if constexpr (PACKED) {
                 cut_rows<Tr, REV>(g, t, (int)(sub_base - lo) + vec_offset<U, EPV, REV>(j, lane), cuts, cut_found[j]);
             }
