@@ -123,6 +123,13 @@ bool outputs_overlap(const Span (&inputs)[NI], const Span (&outputs)[NO]) {
 // Largest row count one launch can address: gridDim.x is limited to 2^31-1.
 constexpr int64_t kMaxBlocks = 2147483647LL;
 
+// rows and seqlen a call can have: non-negative, rows within the grid limit, and
+// the byte size of a tensor (plus a tile of slack for index arithmetic) within int64.
+bool shape_ok(int64_t rows, int64_t seqlen) {
+    if (rows < 0 || seqlen < 0 || rows > kMaxBlocks) return false;
+    return rows == 0 || seqlen <= (INT64_MAX >> 5) / rows;
+}
+
 bool activation_supported(int act, int dtype, bool reverse) {
     if (act == ASCAN_GATE_IDENTITY) return true;
     return (act == ASCAN_GATE_SIGMOID || act == ASCAN_GATE_SIGMOID_LERP) && !reverse &&
@@ -137,7 +144,7 @@ int forward_checked(const void* gates, const void* tokens, void* out, const void
     const size_t es = element_size(dtype);
     if (es == 0) return ASCAN_ERR_BAD_DTYPE;
     if (!activation_supported(act, dtype, reverse != 0)) return ASCAN_ERR_BAD_ACTIVATION;
-    if (rows < 0 || seqlen < 0 || rows > kMaxBlocks) return ASCAN_ERR_BAD_SHAPE;
+    if (!shape_ok(rows, seqlen)) return ASCAN_ERR_BAD_SHAPE;
     if (rows == 0 || seqlen == 0) return ASCAN_OK;
     if (!gates || !tokens || !out) return ASCAN_ERR_NULL_POINTER;
     if (!element_aligned(gates, es) || !element_aligned(tokens, token_size(dtype)) || !element_aligned(out, es) ||
@@ -167,7 +174,7 @@ int backward_checked(const void* gates, const void* states, const void* grad_out
     const size_t es = element_size(dtype);
     if (es == 0) return ASCAN_ERR_BAD_DTYPE;
     if (!activation_supported(act, dtype, false)) return ASCAN_ERR_BAD_ACTIVATION;
-    if (rows < 0 || seqlen < 0 || rows > kMaxBlocks) return ASCAN_ERR_BAD_SHAPE;
+    if (!shape_ok(rows, seqlen)) return ASCAN_ERR_BAD_SHAPE;
     if (rows == 0 || seqlen == 0) return ASCAN_OK;
     if (!gates || !states || !grad_out || !d_gates || !d_tokens) return ASCAN_ERR_NULL_POINTER;
     if (act == ASCAN_GATE_SIGMOID_LERP && !values) return ASCAN_ERR_NULL_POINTER;
@@ -215,7 +222,7 @@ int ascan_backward(const void* gates, const void* states, const void* grad_out, 
 
 size_t ascan_workspace_bytes(int64_t rows, int64_t seqlen, int dtype) {
     const size_t es = element_size(dtype);
-    if (es == 0 || rows <= 0 || seqlen <= 0) return 0;
+    if (es == 0 || rows <= 0 || seqlen <= 0 || !shape_ok(rows, seqlen)) return 0;
     // the smallest split tile any kernel uses for this dtype: 2 blocks of 64 vectors per wave
     const int64_t epv = 16 / (int64_t)es;
     const int64_t tile = (int64_t)kSplitWaves * 2 * 64 * epv;
@@ -296,7 +303,7 @@ const char* ascan_status_string(int status) {
     switch (status) {
         case ASCAN_OK: return "ok";
         case ASCAN_ERR_NULL_POINTER: return "a required buffer pointer is NULL";
-        case ASCAN_ERR_BAD_SHAPE: return "rows or seqlen is negative, or rows exceeds the grid limit";
+        case ASCAN_ERR_BAD_SHAPE: return "rows or seqlen is negative, rows exceeds the grid limit, or rows * seqlen does not fit the address space";
         case ASCAN_ERR_BAD_DTYPE: return "unsupported dtype: expecting float32, bfloat16, float16, complex64 or complex64 with float32 tokens";
         case ASCAN_ERR_MISALIGNED: return "a buffer is not aligned to its element size";
         case ASCAN_ERR_LAUNCH: return "the HIP runtime reported a launch error";

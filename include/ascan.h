@@ -87,7 +87,7 @@ enum ascan_dtype {
 enum ascan_status {
     ASCAN_OK                = 0,
     ASCAN_ERR_NULL_POINTER  = 1, /* a required buffer is NULL while rows*seqlen > 0 */
-    ASCAN_ERR_BAD_SHAPE     = 2, /* rows < 0, seqlen < 0, or rows too large for one grid */
+    ASCAN_ERR_BAD_SHAPE     = 2, /* rows < 0, seqlen < 0, rows too large for one grid, or rows * seqlen beyond 2^58 */
     ASCAN_ERR_BAD_DTYPE     = 3, /* dtype is not an ascan_dtype (warp.cuh:390-391) */
     ASCAN_ERR_MISALIGNED    = 4, /* a pointer is not aligned to its element size */
     ASCAN_ERR_LAUNCH        = 5, /* the HIP runtime refused the launch (see ascan_last_hip_error) */

@@ -56,6 +56,9 @@ def test_argument_validation_returns_codes():
     assert lib.ascan_forward(p, p, p, -1, 4, 0, 0, None) == 2
     assert lib.ascan_forward(p, p, p, 1, -4, 0, 0, None) == 2
     assert lib.ascan_forward(p, p, p, 2**31, 4, 0, 0, None) == 2
+    assert lib.ascan_forward(p, p, p, 2**31 - 1, 2**40, 0, 0, None) == 2  # rows * seqlen beyond the address space
+    assert lib.ascan_forward(p, p, p, 1, 2**63 - 1, 0, 0, None) == 2
+    assert lib.ascan_workspace_bytes(1, 2**63 - 1, 0) == 0
     assert lib.ascan_backward(p, p, p, p, p, 1, -1, 0, None) == 2
     # empty problems succeed without looking at the pointers
     assert lib.ascan_forward(None, None, None, 0, 4, 0, 0, None) == 0

@@ -567,6 +567,39 @@ def test_target_shape_fp32_properties(seqlen):
         assert _rel_err(out[bb, rr][None], t) <= 1e-5
 
 
+def test_target_shape_bf16_sampled_rows_and_flip_identity():
+    """(8, 1536, 65536) bf16 storage, forward + backward, the 16-bit point of the benchmark grid at full size:
+    sampled rows against the fp64 recurrence on the same bf16 values (one final rounding: rtol 2^-8), and the whole
+    tensor through the identity reverse_scan(g, x) = flip(scan(flip g, flip x)) (mirrored lanes do the same
+    arithmetic; at most the last bf16 rounding may differ)."""
+    shape = (8, 1536, 65536)
+    torch.manual_seed(20240611)
+    gates = torch.rand(*shape, device=DEVICE).bfloat16().requires_grad_(True)
+    tokens = torch.rand(*shape, device=DEVICE).bfloat16().requires_grad_(True)
+    grad_out = torch.randn(*shape, device=DEVICE).bfloat16()
+    out = scan_warp(gates, tokens)
+    dg, dx = torch.autograd.grad(out, (gates, tokens), grad_out)
+    out = out.detach()
+    assert out.dtype == dg.dtype == dx.dtype == torch.bfloat16
+
+    for b, rows in ((3, slice(5, 1536, 173)), (0, slice(0, 1)), (7, slice(1535, 1536))):
+        g32 = gates.detach()[b, rows].float().cpu().numpy()
+        x32 = tokens.detach()[b, rows].float().cpu().numpy()
+        d32 = grad_out[b, rows].float().cpu().numpy()
+        t_out = seqscan.forward(g32, x32)
+        t_dg, t_dx = seqscan.backward(g32, out[b, rows].float().cpu().numpy(), d32)
+        for name, got, want in (("out", out, t_out), ("d_tokens", dx, t_dx), ("d_gates", dg, t_dg)):
+            got = got[b, rows].float().cpu().numpy()
+            np.testing.assert_allclose(got, want, rtol=2.0**-8, atol=1e-5 * np.abs(want).max(), err_msg=name)
+
+    from accelerated_scan.warp import scan_forward
+
+    g, x = gates.detach(), tokens.detach()
+    rev = scan_forward(g, x, reverse=True)
+    flipped = scan_forward(g.flip(-1).contiguous(), x.flip(-1).contiguous()).flip(-1)
+    torch.testing.assert_close(rev.float(), flipped.float(), rtol=2.0**-7, atol=1e-6)
+
+
 # ---------------------------------------------------------------------------
 # Complex operator: the reference's matrix (tests/tests_eq_complex.py)
 # ---------------------------------------------------------------------------
