@@ -13,10 +13,10 @@ from pathlib import Path
 
 import torch
 
-ABI_VERSION = 6
+ABI_VERSION = 7
 
 # ascan_gate codes of include/ascan.h
-GATE_IDENTITY, GATE_SIGMOID, GATE_SIGMOID_LERP = 0, 1, 2
+GATE_IDENTITY, GATE_SIGMOID, GATE_SIGMOID_LERP, GATE_EXP = 0, 1, 2, 3
 
 # ascan_dtype codes of include/ascan.h
 F32, BF16, F16, C64, C64_REAL_TOKENS = 0, 1, 2, 3, 4

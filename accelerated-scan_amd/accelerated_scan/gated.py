@@ -1,4 +1,4 @@
-"""Scans whose gates come out of a sigmoid, with the sigmoid done inside the kernels.
+"""Scans whose gates come out of a non-linearity, with the non-linearity done inside the kernels.
 
 ``sigmoid_scan(gate_logits, tokens)`` equals
 ``warp.scan(torch.sigmoid(gate_logits), tokens)`` and is differentiable in the
@@ -16,6 +16,12 @@ tensor.
 logits and values (2 tensors in, 1 out, where the unfused sequence of sigmoid,
 multiply and scan moves 9), the backward kernel reads logits, values, states
 and the incoming gradient and writes both gradients (4 in, 2 out, against 21).
+
+``exp_scan(log_gates, tokens)`` equals ``warp.scan(torch.exp(log_gates), tokens)``
+the same way, for layers that keep their gates as logarithms (decay rates).  In
+16-bit storage that is also the accurate way to hold gates close to 1:
+bfloat16 has no value between 0.99609375 and 1, while a bfloat16 logarithm
+of -0.001 carries three significant digits.
 
 The reference's ``scan`` takes finished gates (accelerated_scan/warp.py:68-83);
 the linear-RNN layers that call it (README.md:8,42 of the reference) typically
@@ -48,33 +54,36 @@ def _check(gate_logits, tokens, initial):
         )
 
 
-class SigmoidScan(torch.autograd.Function):
-    """Autograd node: saves (gate_logits, states, initial); no gates tensor exists."""
+class GatedScan(torch.autograd.Function):
+    """Autograd node of a scan with an in-kernel gate non-linearity (``gate``: an
+    ascan_gate code other than the interpolating one): saves (gate_inputs, states,
+    initial); no gates tensor exists."""
 
     @staticmethod
-    def forward(ctx, gate_logits, tokens, initial):
-        _check(gate_logits, tokens, initial)
+    def forward(ctx, gate_inputs, tokens, initial, gate):
+        _check(gate_inputs, tokens, initial)
         initial = initial.contiguous()
         if _ops.capturing():
-            states = _ops.scan_forward_gated(gate_logits, tokens, initial, _abi.GATE_SIGMOID)
+            states = _ops.scan_forward_gated(gate_inputs, tokens, initial, gate)
         else:
-            states = torch.empty_like(gate_logits)
-            _abi.forward_gated(gate_logits, tokens, states, _abi.GATE_SIGMOID, initial=initial)
-        ctx.save_for_backward(gate_logits, states, initial)
+            states = torch.empty_like(gate_inputs)
+            _abi.forward_gated(gate_inputs, tokens, states, gate, initial=initial)
+        ctx.save_for_backward(gate_inputs, states, initial)
+        ctx.gate = gate
         return states
 
     @staticmethod
     def backward(ctx, grad_output):
-        gate_logits, states, initial = ctx.saved_tensors
+        gate_inputs, states, initial = ctx.saved_tensors
         grad_output = grad_output.contiguous()
         if _ops.capturing():
-            return _ops.scan_backward_gated(gate_logits, states, initial, grad_output, _abi.GATE_SIGMOID)
-        d_logits = torch.empty_like(gate_logits)
-        d_tokens = torch.empty_like(gate_logits)
+            return (*_ops.scan_backward_gated(gate_inputs, states, initial, grad_output, ctx.gate), None)
+        d_gate_inputs = torch.empty_like(gate_inputs)
+        d_tokens = torch.empty_like(gate_inputs)
         d_initial = torch.zeros_like(initial)  # stays zero for an empty sequence
-        _abi.backward_gated(gate_logits, states, grad_output, d_logits, d_tokens, _abi.GATE_SIGMOID,
+        _abi.backward_gated(gate_inputs, states, grad_output, d_gate_inputs, d_tokens, ctx.gate,
                             initial=initial, d_initial=d_initial)
-        return d_logits, d_tokens, d_initial
+        return d_gate_inputs, d_tokens, d_initial, None
 
 
 def sigmoid_scan(gate_logits, tokens, initial=None):
@@ -90,7 +99,23 @@ def sigmoid_scan(gate_logits, tokens, initial=None):
     """
     if initial is None:
         initial = torch.zeros(gate_logits.shape[:-1], dtype=gate_logits.dtype, device=gate_logits.device)
-    return SigmoidScan.apply(gate_logits, tokens, initial)
+    return GatedScan.apply(gate_logits, tokens, initial, _abi.GATE_SIGMOID)
+
+
+def exp_scan(log_gates, tokens, initial=None):
+    """Solve ``x[t] = exp(log_gates[t]) * x[t-1] + tokens[t]``.
+
+    Arguments:
+        log_gates (torch.Tensor): shape (B, C, T), contiguous; fp32, bf16 or fp16; logarithms of the gates.
+        tokens (torch.Tensor): shape (B, C, T), contiguous, same dtype.
+        initial (torch.Tensor, optional): shape (B, C), the state ``x[-1]`` (zero if absent).
+
+    Returns:
+        (torch.Tensor): the states, shape (B, C, T); differentiable in all arguments.
+    """
+    if initial is None:
+        initial = torch.zeros(log_gates.shape[:-1], dtype=log_gates.dtype, device=log_gates.device)
+    return GatedScan.apply(log_gates, tokens, initial, _abi.GATE_EXP)
 
 
 class SigmoidLerpScan(torch.autograd.Function):

@@ -132,11 +132,11 @@ bool shape_ok(int64_t rows, int64_t seqlen) {
 
 bool activation_supported(int act, int dtype, bool reverse) {
     if (act == ASCAN_GATE_IDENTITY) return true;
-    return (act == ASCAN_GATE_SIGMOID || act == ASCAN_GATE_SIGMOID_LERP) && !reverse &&
+    return (act == ASCAN_GATE_SIGMOID || act == ASCAN_GATE_SIGMOID_LERP || act == ASCAN_GATE_EXP) && !reverse &&
            (dtype == ASCAN_F32 || dtype == ASCAN_BF16 || dtype == ASCAN_F16);
 }
 static_assert(ASCAN_GATE_IDENTITY == kGateIdentity && ASCAN_GATE_SIGMOID == kGateSigmoid &&
-                  ASCAN_GATE_SIGMOID_LERP == kGateSigmoidLerp,
+                  ASCAN_GATE_SIGMOID_LERP == kGateSigmoidLerp && ASCAN_GATE_EXP == kGateExp,
               "the kernels' gate codes are the ABI's");
 
 int forward_checked(const void* gates, const void* tokens, void* out, const void* initial, int64_t rows,
@@ -308,7 +308,7 @@ const char* ascan_status_string(int status) {
         case ASCAN_ERR_MISALIGNED: return "a buffer is not aligned to its element size";
         case ASCAN_ERR_LAUNCH: return "the HIP runtime reported a launch error";
         case ASCAN_ERR_BAD_ACTIVATION:
-            return "unsupported gate activation: expecting identity, or a sigmoid gate with float32, bfloat16 or float16";
+            return "unsupported gate activation: expecting identity, or a sigmoid or exponential gate with float32, bfloat16 or float16";
         case ASCAN_ERR_OVERLAP: return "an output buffer overlaps an input or another output buffer of the call";
         case ASCAN_ERR_TOO_LARGE:
             return "the split-row table of this problem exceeds the library's static workspace (ASCAN_STATIC_WORKSPACE_BYTES)";

@@ -18,9 +18,13 @@ namespace {
 //   kGateSigmoidLerp: the same gate, and the token is (1 - gate) * stored value:
 //                     x[t] = gate * x[t-1] + (1 - gate) * v[t], the gated
 //                     interpolation of linear-RNN layers.  The tokens never
-//                     exist in memory either.
+//                     exist in memory either;
+//   kGateExp        : gate = exp(stored), real dtypes only: gates kept as
+//                     logarithms (decay rates).  A 16-bit logarithm carries a
+//                     gate close to 1 far more precisely than a 16-bit gate
+//                     does (bf16 has no value between 0.996 and 1).
 // ---------------------------------------------------------------------------
-constexpr int kGateIdentity = 0, kGateSigmoid = 1, kGateSigmoidLerp = 2;
+constexpr int kGateIdentity = 0, kGateSigmoid = 1, kGateSigmoidLerp = 2, kGateExp = 3;
 
 template <int ACT>
 constexpr bool kGateIsSigmoid = ACT == kGateSigmoid || ACT == kGateSigmoidLerp;
@@ -28,6 +32,10 @@ constexpr bool kGateIsSigmoid = ACT == kGateSigmoid || ACT == kGateSigmoidLerp;
 __device__ __forceinline__ float sigmoid(float v) {
     // v_exp_f32 computes 2^x; v_rcp_f32 is accurate to 1 ulp
     return __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(v * -1.4426950408889634f));
+}
+
+__device__ __forceinline__ float exp_gate(float v) {
+    return __builtin_amdgcn_exp2f(v * 1.4426950408889634f);
 }
 
 // sigmoid(v) and 1 - sigmoid(v) = sigmoid(-v), each to about 2 ulp of its own
@@ -49,6 +57,9 @@ __device__ __forceinline__ void activate(V (&g)[N]) {
     if constexpr (ACT == kGateSigmoid) {
 #pragma unroll
         for (int e = 0; e < N; ++e) g[e] = sigmoid(g[e]);
+    } else if constexpr (ACT == kGateExp) {
+#pragma unroll
+        for (int e = 0; e < N; ++e) g[e] = exp_gate(g[e]);
     }
 }
 // Gates and tokens of a vector from the stored values: g holds gate
@@ -91,6 +102,8 @@ __device__ __forceinline__ V activate1(V g) {
         float gate, complement;
         sigmoid_pair(g, gate, complement);
         return gate;
+    } else if constexpr (ACT == kGateExp) {
+        return exp_gate(g);
     } else {
         return g;
     }
@@ -100,6 +113,8 @@ template <int ACT, class V>
 __device__ __forceinline__ V identity_gate() {
     if constexpr (kGateIsSigmoid<ACT>) {
         return __builtin_inff();
+    } else if constexpr (ACT == kGateExp) {
+        return vzero<V>();
     } else {
         return vone<V>();
     }
@@ -109,6 +124,8 @@ template <int ACT, class V>
 __device__ __forceinline__ V gate_slope(V gate) {
     if constexpr (ACT == kGateSigmoid) {
         return gate * (1.0f - gate);
+    } else if constexpr (ACT == kGateExp) {
+        return gate;
     } else {
         return vone<V>();
     }

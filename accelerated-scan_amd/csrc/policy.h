@@ -310,7 +310,7 @@ Access choose_access(bool same_lead, int lead, int64_t T, int64_t tile) {
     return Access::kVector;
 }
 
-// Kernels with the sigmoid gates exist for the real dtypes, forward in time.
+// Kernels with a gate non-linearity exist for the real dtypes, forward in time.
 template <class Tr>
 constexpr bool kHasSigmoid = std::is_same<typename Tr::V, float>::value;
 
@@ -321,6 +321,7 @@ hipError_t with_gate(int act, F&& f) {
     if constexpr (kHasSigmoid<Tr>) {
         if (act == kGateSigmoid) return f(std::integral_constant<int, kGateSigmoid>{});
         if (act == kGateSigmoidLerp) return f(std::integral_constant<int, kGateSigmoidLerp>{});
+        if (act == kGateExp) return f(std::integral_constant<int, kGateExp>{});
     }
     return f(std::integral_constant<int, kGateIdentity>{});
 }

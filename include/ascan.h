@@ -62,7 +62,7 @@
 extern "C" {
 #endif
 
-#define ASCAN_ABI_VERSION 6
+#define ASCAN_ABI_VERSION 7
 
 /* Marks the exported entry points (the library is built with hidden visibility). */
 #define ASCAN_API __attribute__((visibility("default")))
@@ -106,7 +106,14 @@ enum ascan_gate {
      * gated interpolation of linear-RNN layers.  Forward: ascan_forward_gated;
      * backward: ascan_backward_lerp (it needs v).  float32, bfloat16, float16.
      */
-    ASCAN_GATE_SIGMOID_LERP = 2
+    ASCAN_GATE_SIGMOID_LERP = 2,
+    /*
+     * gate = exp(stored): the stored values are logarithms of the gates (decay
+     * rates; <= 0 for gates in (0, 1]).  A 16-bit logarithm holds a gate close
+     * to 1 far more precisely than a 16-bit gate can (bfloat16 has no value
+     * between 0.99609375 and 1).  float32, bfloat16, float16.
+     */
+    ASCAN_GATE_EXP = 3
 };
 
 /*
@@ -242,10 +249,11 @@ ASCAN_API int ascan_backward_from(const void* gates, const void* states, const v
  *
  * with g, d_tokens and d_initial as in ascan_backward_from.  No counterpart in
  * the reference.  gate = ASCAN_GATE_IDENTITY makes these calls the *_from ones
- * (forward in time only); the sigmoid gates need a real dtype, else
+ * (forward in time only); the sigmoid and exponential gates need a real dtype, else
  * ASCAN_ERR_BAD_ACTIVATION (as does ASCAN_GATE_SIGMOID_LERP in
  * ascan_backward_gated, which lacks the values: see ascan_backward_lerp).  The sigmoid is evaluated in fp32 with the
- * hardware's exp2 and reciprocal (about 2 ulp).
+ * hardware's exp2 and reciprocal (about 2 ulp), the exponential with exp2 (1 ulp
+ * of the result for arguments of moderate size).
  */
 ASCAN_API int ascan_forward_gated(const void* gate_inputs, const void* tokens, const void* initial, void* out,
                         int64_t rows, int64_t seqlen, int dtype, int gate,

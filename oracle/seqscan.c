@@ -274,6 +274,46 @@ void seq_backward_sigmoid_f32(const float* z, const float* state, const float* i
 }
 
 /*
+ * Scans whose gates are the exponential of stored logarithms (no counterpart
+ * in the reference, which is handed finished gates):
+ *   gate[t] = exp(z[t]),  out[t] = gate[t] * out[t-1] + x[t],  out[-1] = init
+ *   a[t] = dout[t] + gate[t+1] * a[t+1],  dx = a,
+ *   dz[t] = a[t] * state[t-1] * gate[t],  dinit = gate[0] * a[0]
+ * Pinned by tests/test_oracle.py: torch autograd through the plain float64 loop
+ * with torch.exp, the zero-start functions above on gates formed in float64,
+ * and closed forms (constant z = log q gives the geometric series of ratio q;
+ * x = delta at 0 gives exp of the running sum of z).
+ */
+void seq_forward_exp_f32(const float* z, const float* x, const float* init, double* out, int64_t rows, int64_t T) {
+#pragma omp parallel for schedule(static)
+    for (int64_t r = 0; r < rows; ++r) {
+        double s = init ? (double)init[r] : 0.0;
+        for (int64_t t = 0; t < T; ++t) {
+            s = exp((double)z[r * T + t]) * s + (double)x[r * T + t];
+            out[r * T + t] = s;
+        }
+    }
+}
+
+void seq_backward_exp_f32(const float* z, const float* state, const float* init, const float* dout, double* dz,
+                          double* dx, double* dinit, int64_t rows, int64_t T) {
+#pragma omp parallel for schedule(static)
+    for (int64_t r = 0; r < rows; ++r) {
+        const float* zr = z + r * T;
+        const float* sr = state + r * T;
+        const double x0 = init ? (double)init[r] : 0.0;
+        double a = 0.0;
+        for (int64_t t = T - 1; t >= 0; --t) {
+            const double gnext = (t + 1 < T) ? exp((double)zr[t + 1]) : 1.0;
+            a = (double)dout[r * T + t] + gnext * a;
+            dx[r * T + t] = a;
+            dz[r * T + t] = a * ((t > 0) ? (double)sr[t - 1] : x0) * exp((double)zr[t]);
+        }
+        if (dinit) dinit[r] = (T > 0) ? exp((double)zr[0]) * a : 0.0;
+    }
+}
+
+/*
  * Gated interpolation (no counterpart in the reference): the gate is the
  * sigmoid of a stored pre-activation and the token its complement times a
  * stored value,

@@ -38,13 +38,16 @@ def _load():
         lib.seq_backward_from_f32.argtypes = [p, p, p, p, p, p, p, i64, i64]
         lib.seq_backward_from_c64.argtypes = [p, p, p, p, p, p, p, i64, i64]
         lib.seq_forward_sigmoid_f32.argtypes = [p, p, p, p, i64, i64]
+        lib.seq_forward_exp_f32.argtypes = [p, p, p, p, i64, i64]
+        lib.seq_backward_exp_f32.argtypes = [p, p, p, p, p, p, p, i64, i64]
         lib.seq_backward_sigmoid_f32.argtypes = [p, p, p, p, p, p, p, i64, i64]
         lib.seq_forward_lerp_f32.argtypes = [p, p, p, p, i64, i64]
         lib.seq_backward_lerp_f32.argtypes = [p, p, p, p, p, p, p, p, i64, i64]
         for f in (lib.seq_forward_f32, lib.seq_forward_c64, lib.seq_backward_f32, lib.seq_backward_c64,
                   lib.seq_forward_from_f32, lib.seq_forward_from_c64, lib.seq_backward_from_f32,
                   lib.seq_backward_from_c64, lib.seq_forward_sigmoid_f32, lib.seq_backward_sigmoid_f32,
-                  lib.seq_forward_lerp_f32, lib.seq_backward_lerp_f32):
+                  lib.seq_forward_lerp_f32, lib.seq_backward_lerp_f32, lib.seq_forward_exp_f32,
+                  lib.seq_backward_exp_f32):
             f.restype = None
         _lib = lib
     return _lib
@@ -130,10 +133,9 @@ def backward_from(gates, states, initial, grad_out):
     return dg, dx, di
 
 
-def forward_sigmoid(gate_logits, tokens, initial=None):
-    """Sequential scan in fp64 with gates = sigmoid(gate_logits) (real inputs)."""
+def _forward_gated(name, gate_inputs, tokens, initial):
     lib = _load()
-    z, zp = _prep(gate_logits, np.float32)
+    z, zp = _prep(gate_inputs, np.float32)
     x, xp = _prep(tokens, np.float32)
     assert z.shape == x.shape
     ip = None
@@ -143,14 +145,13 @@ def forward_sigmoid(gate_logits, tokens, initial=None):
     T = z.shape[-1]
     rows = z.size // T if T else 0
     out = np.empty(z.shape, dtype=np.float64)
-    lib.seq_forward_sigmoid_f32(zp, xp, ip, out.ctypes.data_as(ctypes.c_void_p), rows, T)
+    getattr(lib, name)(zp, xp, ip, out.ctypes.data_as(ctypes.c_void_p), rows, T)
     return out
 
 
-def backward_sigmoid(gate_logits, states, grad_out, initial=None):
-    """(d_gate_logits, d_tokens, d_initial) of the sigmoid-gated scan, in fp64."""
+def _backward_gated(name, gate_inputs, states, grad_out, initial):
     lib = _load()
-    z, zp = _prep(gate_logits, np.float32)
+    z, zp = _prep(gate_inputs, np.float32)
     s, sp = _prep(states, np.float32)
     d, dp = _prep(grad_out, np.float32)
     assert z.shape == s.shape == d.shape
@@ -164,9 +165,29 @@ def backward_sigmoid(gate_logits, states, grad_out, initial=None):
     dx = np.empty(z.shape, dtype=np.float64)
     di = np.zeros(z.shape[:-1], dtype=np.float64)
     if rows:
-        lib.seq_backward_sigmoid_f32(zp, sp, ip, dp, dz.ctypes.data_as(ctypes.c_void_p),
-                                     dx.ctypes.data_as(ctypes.c_void_p), di.ctypes.data_as(ctypes.c_void_p), rows, T)
+        getattr(lib, name)(zp, sp, ip, dp, dz.ctypes.data_as(ctypes.c_void_p), dx.ctypes.data_as(ctypes.c_void_p),
+                           di.ctypes.data_as(ctypes.c_void_p), rows, T)
     return dz, dx, di
+
+
+def forward_sigmoid(gate_logits, tokens, initial=None):
+    """Sequential scan in fp64 with gates = sigmoid(gate_logits) (real inputs)."""
+    return _forward_gated("seq_forward_sigmoid_f32", gate_logits, tokens, initial)
+
+
+def backward_sigmoid(gate_logits, states, grad_out, initial=None):
+    """(d_gate_logits, d_tokens, d_initial) of the sigmoid-gated scan, in fp64."""
+    return _backward_gated("seq_backward_sigmoid_f32", gate_logits, states, grad_out, initial)
+
+
+def forward_exp(log_gates, tokens, initial=None):
+    """Sequential scan in fp64 with gates = exp(log_gates) (real inputs)."""
+    return _forward_gated("seq_forward_exp_f32", log_gates, tokens, initial)
+
+
+def backward_exp(log_gates, states, grad_out, initial=None):
+    """(d_log_gates, d_tokens, d_initial) of the exponentially gated scan, in fp64."""
+    return _backward_gated("seq_backward_exp_f32", log_gates, states, grad_out, initial)
 
 
 def forward_lerp(gate_logits, values, initial=None):

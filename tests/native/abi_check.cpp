@@ -21,6 +21,9 @@ void seq_backward_from_f32(const float* g, const float* state, const float* init
 void seq_forward_sigmoid_f32(const float* z, const float* x, const float* init, double* out, int64_t rows, int64_t T);
 void seq_backward_sigmoid_f32(const float* z, const float* state, const float* init, const float* dout, double* dz,
                               double* dx, double* dinit, int64_t rows, int64_t T);
+void seq_forward_exp_f32(const float* z, const float* x, const float* init, double* out, int64_t rows, int64_t T);
+void seq_backward_exp_f32(const float* z, const float* state, const float* init, const float* dout, double* dz,
+                          double* dx, double* dinit, int64_t rows, int64_t T);
 void seq_forward_lerp_f32(const float* z, const float* v, const float* init, double* out, int64_t rows, int64_t T);
 void seq_backward_lerp_f32(const float* z, const float* v, const float* state, const float* init, const float* dout,
                            double* dz, double* dv, double* dinit, int64_t rows, int64_t T);
@@ -193,6 +196,25 @@ void check_gated_and_static(int64_t rows, int64_t T, hipStream_t stream) {
     EXPECT(worst(download(d_z, n, stream), t_dz) <= tol);
     EXPECT(worst(download(d_x, n, stream), t_dx) <= tol);
     EXPECT(worst(download(d_init, rows, stream), t_di) <= tol);
+
+    // exponential gate: the stored values are logarithms of gates in (0, 1]
+    {
+        std::vector<float> logs(n);
+        for (size_t i = 0; i < n; ++i) logs[i] = -0.25f * std::fabs(z[i]);
+        upload(dz_in, logs, stream);
+        EXPECT(ascan_forward_gated(dz_in.p, dx_in.p, dinit_in.p, out.p, rows, T, ASCAN_F32, ASCAN_GATE_EXP, ws_ptr,
+                                   ws_bytes, stream) == ASCAN_OK);
+        EXPECT(ascan_backward_gated(dz_in.p, out.p, dinit_in.p, dd_in.p, d_z.p, d_x.p, d_init.p, rows, T, ASCAN_F32,
+                                    ASCAN_GATE_EXP, ws_ptr, ws_bytes, stream) == ASCAN_OK);
+        h_out = download(out, n, stream);
+        seq_forward_exp_f32(logs.data(), x.data(), init.data(), t_out.data(), rows, T);
+        seq_backward_exp_f32(logs.data(), h_out.data(), init.data(), d.data(), t_dz.data(), t_dx.data(), t_di.data(), rows,
+                             T);
+        EXPECT(worst(h_out, t_out) <= tol);
+        EXPECT(worst(download(d_z, n, stream), t_dz) <= tol);
+        EXPECT(worst(download(d_x, n, stream), t_dx) <= tol);
+        EXPECT(worst(download(d_init, rows, stream), t_di) <= tol);
+    }
 
     // static-table forward scan: stored values in [0, 1) as gates (x from a zero state)
     std::vector<float> g(n);

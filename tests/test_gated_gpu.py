@@ -34,9 +34,12 @@ def _need_gpu_and_library():
     _abi.load()  # raises if the HIP library is missing: no fallback exists
 
 
-def _inputs(rows, T, dtype, seed, logit_mean=0.0):
+def _inputs(rows, T, dtype, seed, logit_mean=0.0, gate="sigmoid"):
     gen = torch.Generator().manual_seed(seed)
-    logits = (logit_mean + 2.0 * torch.randn(rows, T, generator=gen)).to(dtype)
+    logits = logit_mean + 2.0 * torch.randn(rows, T, generator=gen)
+    if gate == "exp":  # logarithms of gates: mostly below zero (gates in (0, 1)), one in twenty a little above
+        logits = torch.where(torch.rand(rows, T, generator=gen) < 0.05, 0.05 * logits.abs(), -logits.abs())
+    logits = logits.to(dtype)
     tokens = torch.randn(rows, T, generator=gen).to(dtype)
     grad_out = torch.randn(rows, T, generator=gen).to(dtype)
     initial = (3.0 * torch.randn(rows, generator=gen)).to(dtype)
@@ -50,10 +53,15 @@ def _offset_copy(t, shape, k):
     return view
 
 
-def _run_and_compare(rows, T, dtype, seed, what, with_initial, offsets=(0, 0, 0), logit_mean=0.0, factor=2.0):
+def _run_and_compare(rows, T, dtype, seed, what, with_initial, offsets=(0, 0, 0), logit_mean=0.0, factor=2.0,
+                     gate="sigmoid"):
+    """``gate``: "sigmoid" (oracle functions *_sigmoid) or "exp" (*_exp; tests/test_exp_gate_gpu.py)."""
     from accelerated_scan import _abi
 
-    logits, tokens, grad_out, initial = _inputs(rows, T, dtype, seed, logit_mean)
+    code = {"sigmoid": _abi.GATE_SIGMOID, "exp": _abi.GATE_EXP}[gate]
+    truth_forward, truth_backward = {"sigmoid": (seqscan.forward_sigmoid, seqscan.backward_sigmoid),
+                                     "exp": (seqscan.forward_exp, seqscan.backward_exp)}[gate]
+    logits, tokens, grad_out, initial = _inputs(rows, T, dtype, seed, logit_mean, gate)
     og, ox, oo = offsets
     shape = (1, rows, T)
     z, x, d = _offset_copy(logits, shape, og), _offset_copy(tokens, shape, ox), _offset_copy(grad_out, shape, oo)
@@ -61,15 +69,15 @@ def _run_and_compare(rows, T, dtype, seed, what, with_initial, offsets=(0, 0, 0)
     out = _offset_copy(torch.zeros_like(logits), shape, oo)
     dz, dx = _offset_copy(torch.zeros_like(logits), shape, ox), _offset_copy(torch.zeros_like(tokens), shape, oo)
     di = torch.full((1, rows), float("nan"), dtype=dtype, device=DEVICE) if with_initial else None
-    _abi.forward_gated(z, x, out, _abi.GATE_SIGMOID, initial=init)
-    _abi.backward_gated(z, out, d, dz, dx, _abi.GATE_SIGMOID, initial=init, d_initial=di)
+    _abi.forward_gated(z, x, out, code, initial=init)
+    _abi.backward_gated(z, out, d, dz, dx, code, initial=init, d_initial=di)
     torch.cuda.synchronize()
 
     f32 = lambda t: t.float().numpy()
     init_host = f32(initial) if with_initial else None
-    t_out = seqscan.forward_sigmoid(f32(logits), f32(tokens), init_host)
+    t_out = truth_forward(f32(logits), f32(tokens), init_host)
     states = out.reshape(rows, T).cpu()  # backward consumes the states the GPU produced
-    t_dz, t_dx, t_di = seqscan.backward_sigmoid(f32(logits), f32(states), f32(grad_out), init_host)
+    t_dz, t_dx, t_di = truth_backward(f32(logits), f32(states), f32(grad_out), init_host)
     tol = factor * 2e-5 if dtype == torch.float32 else 2 * storage_ulp[dtype]
     pairs = [("out", out, t_out), ("d_tokens", dx, t_dx), ("d_logits", dz, t_dz)]
     if with_initial:

@@ -358,6 +358,59 @@ def test_sigmoid_vs_plain_scan_of_rounded_gates_and_closed_form():
 
 
 # ---------------------------------------------------------------------------
+# Exponentially gated scans, gate = exp(stored logarithm) (oracle functions *_exp)
+# ---------------------------------------------------------------------------
+@pytest.mark.parametrize("T", [1, 2, 9, 64])
+@pytest.mark.parametrize("with_initial", [False, True])
+def test_exp_vs_autograd_of_loop(T, with_initial):
+    gen = torch.Generator().manual_seed(450 + T)
+    log_gates = -torch.rand(2, 2, T, generator=gen) * 2.0 + 0.3  # a few gates above 1 as well
+    tokens, grad_out = (torch.randn(2, 2, T, generator=gen) for _ in range(2))
+    initial = torch.randn(2, 2, generator=gen) if with_initial else torch.zeros(2, 2)
+    zw, tw, iw = (t.double().requires_grad_(True) for t in (log_gates, tokens, initial))
+    out = _loop_scan_from(torch.exp(zw), tw, iw)
+    dz_ref, dt_ref, di_ref = torch.autograd.grad(out, (zw, tw, iw), grad_out.double())
+    init_arg = initial.numpy() if with_initial else None
+    fwd = seqscan.forward_exp(log_gates.numpy(), tokens.numpy(), init_arg)
+    np.testing.assert_allclose(fwd, out.detach().numpy(), rtol=1e-12, atol=1e-12)
+    dz, dt, di = seqscan.backward_exp(log_gates.numpy(), fwd.astype(np.float32), grad_out.numpy(), init_arg)
+    np.testing.assert_allclose(dt, dt_ref.numpy(), rtol=1e-12, atol=1e-12)
+    np.testing.assert_allclose(di, di_ref.numpy(), rtol=1e-12, atol=1e-12)
+    np.testing.assert_allclose(dz, dz_ref.numpy(), rtol=1e-5, atol=1e-5)  # states rounded to fp32 before the multiply
+
+
+def test_exp_vs_plain_scan_of_rounded_gates_and_closed_forms():
+    gen = torch.Generator().manual_seed(23)
+    log_gates = -torch.rand(3, 4, 200, generator=gen)
+    tokens, grad_out = (torch.randn(3, 4, 200, generator=gen) for _ in range(2))
+    gates = torch.exp(log_gates.double())
+    fwd = seqscan.forward_exp(log_gates.numpy(), tokens.numpy())
+    plain = seqscan.forward(gates.float().numpy(), tokens.numpy())
+    np.testing.assert_allclose(fwd, plain, rtol=1e-5, atol=1e-5)  # gates rounded to fp32 on one side
+    states = fwd.astype(np.float32)
+    dz, dx, _ = seqscan.backward_exp(log_gates.numpy(), states, grad_out.numpy())
+    dg, dx_plain = seqscan.backward(gates.float().numpy(), states, grad_out.numpy())
+    np.testing.assert_allclose(dx, dx_plain, rtol=1e-5, atol=1e-5)
+    np.testing.assert_allclose(dz, dg * gates.numpy(), rtol=1e-5, atol=1e-5)  # d exp(z) / dz = exp(z)
+    # constant logarithm log q, unit tokens: the geometric series (1 - q^(t+1)) / (1 - q)
+    T, q = 40, 0.75
+    z = np.full((1, 1, T), np.log(q), np.float32)
+    out = seqscan.forward_exp(z, np.ones((1, 1, T), np.float32))
+    qq = np.exp(np.float64(z[0, 0, 0]))
+    np.testing.assert_allclose(out[0, 0], (1 - qq ** (np.arange(T) + 1)) / (1 - qq), rtol=1e-13)
+    # a single unit token at t = 0: the state is exp of the running sum of the later logarithms
+    z = log_gates[:1, :1, :60].numpy()
+    x = np.zeros_like(z)
+    x[..., 0] = 1.0
+    running = np.concatenate([[0.0], np.cumsum(z[0, 0, 1:].astype(np.float64))])
+    np.testing.assert_allclose(seqscan.forward_exp(z, x)[0, 0], np.exp(running), rtol=1e-12)
+    # z = 0 is a running sum, z = -800 (gate 0 in fp64) returns the tokens
+    x = tokens[:1, :1, :50].numpy()
+    np.testing.assert_allclose(seqscan.forward_exp(np.zeros_like(x), x), np.cumsum(x.astype(np.float64), -1), rtol=1e-12, atol=1e-12)
+    np.testing.assert_allclose(seqscan.forward_exp(np.full_like(x, -800.0), x), x, rtol=1e-12, atol=1e-12)
+
+
+# ---------------------------------------------------------------------------
 # Gated interpolation x[t] = a x[t-1] + (1 - a) v[t], a = sigmoid(z) (oracle functions *_lerp)
 # ---------------------------------------------------------------------------
 @pytest.mark.parametrize("T", [1, 2, 9, 64])
