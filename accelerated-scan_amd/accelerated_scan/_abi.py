@@ -13,7 +13,7 @@ from pathlib import Path
 
 import torch
 
-ABI_VERSION = 7
+ABI_VERSION = 8
 
 # ascan_gate codes of include/ascan.h
 GATE_IDENTITY, GATE_SIGMOID, GATE_SIGMOID_LERP, GATE_EXP = 0, 1, 2, 3
@@ -66,6 +66,13 @@ _SIGNATURES = {
          ctypes.c_void_p, ctypes.c_size_t, ctypes.c_void_p],
     ),
     "ascan_backward_from": (
+        ctypes.c_int,
+        [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p,
+         ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p,
+         ctypes.c_int64, ctypes.c_int64, ctypes.c_int,
+         ctypes.c_void_p, ctypes.c_size_t, ctypes.c_void_p],
+    ),
+    "ascan_backward_reverse": (
         ctypes.c_int,
         [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p,
          ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p,
@@ -252,15 +259,23 @@ def forward(gates, tokens, out, reverse: bool, workspace=None, initial=None) -> 
                 seqlen, code, 1 if reverse else 0, workspace.data_ptr(), workspace.numel())
 
 
-def backward(gates, states, grad_out, d_gates, d_tokens, workspace=None, initial=None, d_initial=None) -> None:
+def backward(gates, states, grad_out, d_gates, d_tokens, workspace=None, initial=None, d_initial=None,
+             reverse: bool = False) -> None:
     """Enqueue the fused backward scan on the current stream of the tensors' device.
     ``initial`` is the state the forward scan started from; ``d_initial``
-    receives its gradient (left untouched for an empty sequence)."""
+    receives its gradient (left untouched for an empty sequence).  ``reverse``:
+    the scan being differentiated ran backwards in time (``forward(..., reverse=True)``)."""
     lib = _lib or load()
     rows, seqlen, code = _problem(gates, d_tokens)
     if workspace is None and _workspace_bytes(rows, seqlen, code):
         workspace = _workspace(rows, seqlen, code, gates.device)
-    if initial is not None or d_initial is not None:
+    if reverse:
+        _check_state(initial, states, "initial")
+        _check_state(d_initial, states, "d_initial")
+        _launch(gates.device, lib.ascan_backward_reverse, gates.data_ptr(), states.data_ptr(), _ptr(initial),
+                grad_out.data_ptr(), d_gates.data_ptr(), d_tokens.data_ptr(), _ptr(d_initial), rows, seqlen, code,
+                _ptr(workspace), workspace.numel() if workspace is not None else 0)
+    elif initial is not None or d_initial is not None:
         _check_state(initial, states, "initial")
         _check_state(d_initial, states, "d_initial")
         _launch(gates.device, lib.ascan_backward_from, gates.data_ptr(), states.data_ptr(), _ptr(initial),

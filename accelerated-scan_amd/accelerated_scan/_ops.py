@@ -112,6 +112,24 @@ def _(gates, states, initial, grad_out, real_tokens):
     return torch.empty_like(gates), _empty_token_grad(gates, real_tokens), torch.empty_like(initial)
 
 
+@torch.library.custom_op("accelerated_scan::scan_backward_reverse", mutates_args=())
+def scan_backward_reverse(
+    gates: torch.Tensor, states: torch.Tensor, initial: torch.Tensor, grad_out: torch.Tensor, real_tokens: bool
+) -> Tuple[torch.Tensor, torch.Tensor, torch.Tensor]:
+    """Backward pass of a reverse scan (``scan_forward`` / ``scan_forward_from`` with ``reverse=True``)."""
+    _check_dense(gates, (states, grad_out), states=(initial,))
+    d_gates = torch.empty_like(gates)
+    d_tokens = _empty_token_grad(gates, real_tokens)
+    d_initial = torch.zeros_like(initial)  # stays zero for an empty sequence
+    _abi.backward(gates, states, grad_out, d_gates, d_tokens, initial=initial, d_initial=d_initial, reverse=True)
+    return d_gates, d_tokens, d_initial
+
+
+@scan_backward_reverse.register_fake
+def _(gates, states, initial, grad_out, real_tokens):
+    return torch.empty_like(gates), _empty_token_grad(gates, real_tokens), torch.empty_like(initial)
+
+
 @torch.library.custom_op("accelerated_scan::scan_forward_gated", mutates_args=())
 def scan_forward_gated(gate_inputs: torch.Tensor, tokens: torch.Tensor, initial: torch.Tensor, gate: int) -> torch.Tensor:
     _check_dense(gate_inputs, (tokens,), states=(initial,))
@@ -177,13 +195,8 @@ def capturing() -> bool:
 # Autograd formulas of the forward operators.  The gradient of a scan is the
 # fused backward operator (accelerated_scan/warp.py:50-65 of the reference:
 # g[t] = grad[t] + gates[t+1] * g[t+1], d_tokens = g, d_gates[t] = g[t] * x[t-1]).
-# A reverse scan is the forward scan of the flipped sequences, flipped, so its
-# gradient is the flipped gradient of that scan.
+# A reverse scan has a fused backward operator of its own, the mirror image in time.
 # ---------------------------------------------------------------------------
-def _flip(t: torch.Tensor) -> torch.Tensor:
-    return t.flip(-1).contiguous()
-
-
 def _real_tokens(gates: torch.Tensor, tokens: torch.Tensor) -> bool:
     return gates.is_complex() and not tokens.is_complex()
 
@@ -199,8 +212,9 @@ def _backward_scan_forward(ctx, grad):
     gates, states = ctx.saved_tensors
     grad = grad.contiguous()
     if ctx.reverse:
-        d_gates, d_tokens = scan_backward(_flip(gates), _flip(states), _flip(grad), ctx.real_tokens)
-        return _flip(d_gates), _flip(d_tokens), None
+        zero = torch.zeros(gates.shape[:-1], dtype=gates.dtype, device=gates.device)
+        d_gates, d_tokens, _ = scan_backward_reverse(gates, states, zero, grad, ctx.real_tokens)
+        return d_gates, d_tokens, None
     d_gates, d_tokens = scan_backward(gates, states, grad, ctx.real_tokens)
     return d_gates, d_tokens, None
 
@@ -220,9 +234,8 @@ def _backward_scan_forward_from(ctx, grad):
     gates, states, initial = ctx.saved_tensors
     grad = grad.contiguous()
     if ctx.reverse:
-        d_gates, d_tokens, d_initial = scan_backward_from(
-            _flip(gates), _flip(states), initial, _flip(grad), ctx.real_tokens)
-        return _flip(d_gates), _flip(d_tokens), d_initial, None
+        d_gates, d_tokens, d_initial = scan_backward_reverse(gates, states, initial, grad, ctx.real_tokens)
+        return d_gates, d_tokens, d_initial, None
     d_gates, d_tokens, d_initial = scan_backward_from(gates, states, initial, grad, ctx.real_tokens)
     return d_gates, d_tokens, d_initial, None
 

@@ -50,11 +50,12 @@ class Scan(torch.autograd.Function):
     """Autograd node: saves (gates, states, initial), returns (d_gates, d_tokens, d_initial)."""
 
     @staticmethod
-    def forward(ctx, gates, tokens, initial):
+    def forward(ctx, gates, tokens, initial, reverse=False):
         initial = initial.contiguous()
-        states = scan_forward(gates, tokens, initial)
+        states = scan_forward(gates, tokens, initial, reverse)
         ctx.save_for_backward(gates, states, initial)
         ctx.real_tokens = gates.is_complex() and not tokens.is_complex()
+        ctx.reverse = reverse
         return states
 
     @staticmethod
@@ -62,28 +63,37 @@ class Scan(torch.autograd.Function):
         gates, states, initial = ctx.saved_tensors
         grad_output = grad_output.contiguous()
         if _ops.capturing():
-            return _ops.scan_backward_from(gates, states, initial, grad_output, ctx.real_tokens)
+            op = _ops.scan_backward_reverse if ctx.reverse else _ops.scan_backward_from
+            return (*op(gates, states, initial, grad_output, ctx.real_tokens), None)
         d_gates = torch.empty_like(gates)
         if ctx.real_tokens:
             d_tokens = torch.empty(gates.shape, dtype=gates.real.dtype, device=gates.device)
         else:
             d_tokens = torch.empty_like(gates)
         d_initial = torch.zeros_like(initial)  # stays zero for an empty sequence
-        _abi.backward(gates, states, grad_output, d_gates, d_tokens, initial=initial, d_initial=d_initial)
-        return d_gates, d_tokens, d_initial
+        _abi.backward(gates, states, grad_output, d_gates, d_tokens, initial=initial, d_initial=d_initial,
+                      reverse=ctx.reverse)
+        return d_gates, d_tokens, d_initial, None
 
 
-def scan(gates, tokens, initial):
-    """Solve ``x[t] = gates[t] * x[t-1] + tokens[t]`` from ``x[-1] = initial``.
+def scan(gates, tokens, initial=None, reverse=False):
+    """Solve ``x[t] = gates[t] * x[t-1] + tokens[t]`` from ``x[-1] = initial``, or with
+    ``reverse=True`` ``y[t] = gates[t] * y[t+1] + tokens[t]`` from ``y[T] = initial``.
 
     Arguments:
         gates (torch.Tensor): shape (B, C, T), contiguous; fp32, bf16, fp16 or complex64.
         tokens (torch.Tensor): shape (B, C, T), contiguous, the dtype of gates
             (or float32 with complex64 gates).
-        initial (torch.Tensor): shape (B, C), the dtype of gates.
+        initial (torch.Tensor, optional): shape (B, C), the dtype of gates; zeros if absent.
+        reverse (bool): scan from the last element to the first.  The reference's reverse
+            scan (accelerated_scan/warp.py:32-35) is not differentiable; this one is, through
+            a fused backward kernel of its own, so a sequence can be scanned in both directions.
 
     Returns:
-        (torch.Tensor): states of shape (B, C, T); ``states[..., -1]`` is the
-        state to hand to the next chunk.
+        (torch.Tensor): states of shape (B, C, T), differentiable in gates, tokens and
+        initial; ``states[..., -1]`` (``states[..., 0]`` for a reverse scan) is the state
+        to hand to the next chunk.
     """
-    return Scan.apply(gates, tokens, initial)
+    if initial is None:
+        initial = torch.zeros(gates.shape[:-1], dtype=gates.dtype, device=gates.device)
+    return Scan.apply(gates, tokens, initial, reverse)

@@ -111,7 +111,7 @@ class Scan(torch.autograd.Function):
         return d_gates, d_tokens
 
 
-def scan(gates, tokens, initial=None):
+def scan(gates, tokens, initial=None, reverse=False):
     """Solve the first-order recurrence ``x[t] = gates[t] * x[t-1] + tokens[t]``.
 
     Arguments:
@@ -119,12 +119,15 @@ def scan(gates, tokens, initial=None):
         tokens (torch.Tensor): shape (B, C, T), contiguous, same dtype.
         initial (torch.Tensor, optional): shape (B, C), the state ``x[-1]`` to
             start from (not in the reference, which starts from zero).
+        reverse (bool, optional): solve ``x[t] = gates[t] * x[t+1] + tokens[t]`` from the
+            last element down instead (``initial`` is then ``x[T]``); differentiable like
+            the forward scan (not in the reference, whose reverse scan has no gradient).
 
     Returns:
         (torch.Tensor): shape (B, C, T), the states ``x``; differentiable in
         all arguments.
     """
-    if initial is not None:
+    if initial is not None or reverse:
         _check_dtype(gates)
-        return stateful.scan(gates, tokens, initial)
+        return stateful.scan(gates, tokens, initial, reverse)
     return Scan.apply(gates, tokens)

@@ -167,13 +167,14 @@ int forward_checked(const void* gates, const void* tokens, void* out, const void
     }
 }
 
-// `values` is the fourth input of the interpolating gate and null for every other gate.
+// `values` is the fourth input of the interpolating gate and null for every other gate;
+// `reverse` says that the scan being differentiated ran backwards in time (identity gate only).
 int backward_checked(const void* gates, const void* states, const void* grad_out, void* d_gates, void* d_tokens,
                      const void* initial, void* d_initial, const void* values, int64_t rows, int64_t seqlen,
-                     int dtype, int act, const Workspace& ws, void* stream) {
+                     int dtype, int act, bool reverse, const Workspace& ws, void* stream) {
     const size_t es = element_size(dtype);
     if (es == 0) return ASCAN_ERR_BAD_DTYPE;
-    if (!activation_supported(act, dtype, false)) return ASCAN_ERR_BAD_ACTIVATION;
+    if (!activation_supported(act, dtype, reverse)) return ASCAN_ERR_BAD_ACTIVATION;
     if (!shape_ok(rows, seqlen)) return ASCAN_ERR_BAD_SHAPE;
     if (rows == 0 || seqlen == 0) return ASCAN_OK;
     if (!gates || !states || !grad_out || !d_gates || !d_tokens) return ASCAN_ERR_NULL_POINTER;
@@ -192,6 +193,15 @@ int backward_checked(const void* gates, const void* states, const void* grad_out
     }
     const BackwardCall call{gates, states, grad_out, d_gates, d_tokens, initial, d_initial, values, rows, seqlen, act,
                             ws, static_cast<hipStream_t>(stream)};
+    if (reverse) {
+        switch (dtype) {
+            case ASCAN_F32: return backward_reverse_f32(call);
+            case ASCAN_BF16: return backward_reverse_bf16(call);
+            case ASCAN_F16: return backward_reverse_f16(call);
+            case ASCAN_C64: return backward_reverse_c64(call);
+            default: return backward_reverse_c64_real_tokens(call);
+        }
+    }
     switch (dtype) {
         case ASCAN_F32: return backward_f32(call);
         case ASCAN_BF16: return backward_bf16(call);
@@ -217,7 +227,7 @@ int ascan_forward(const void* gates, const void* tokens, void* out, int64_t rows
 int ascan_backward(const void* gates, const void* states, const void* grad_out, void* d_gates, void* d_tokens,
                    int64_t rows, int64_t seqlen, int dtype, void* stream) {
     return backward_checked(gates, states, grad_out, d_gates, d_tokens, nullptr, nullptr, nullptr, rows, seqlen, dtype,
-                            ASCAN_GATE_IDENTITY, Workspace{nullptr, 0}, stream);
+                            ASCAN_GATE_IDENTITY, false, Workspace{nullptr, 0}, stream);
 }
 
 size_t ascan_workspace_bytes(int64_t rows, int64_t seqlen, int dtype) {
@@ -257,7 +267,7 @@ int ascan_backward_split(const void* gates, const void* states, const void* grad
                          void* d_tokens, int64_t rows, int64_t seqlen, int dtype, void* workspace,
                          size_t workspace_bytes, void* stream) {
     return backward_checked(gates, states, grad_out, d_gates, d_tokens, nullptr, nullptr, nullptr, rows, seqlen, dtype,
-                            ASCAN_GATE_IDENTITY, Workspace{workspace, workspace_bytes}, stream);
+                            ASCAN_GATE_IDENTITY, false, Workspace{workspace, workspace_bytes}, stream);
 }
 
 int ascan_forward_from(const void* gates, const void* tokens, const void* initial, void* out, int64_t rows,
@@ -271,7 +281,14 @@ int ascan_backward_from(const void* gates, const void* states, const void* initi
                         void* d_gates, void* d_tokens, void* d_initial, int64_t rows, int64_t seqlen, int dtype,
                         void* workspace, size_t workspace_bytes, void* stream) {
     return backward_checked(gates, states, grad_out, d_gates, d_tokens, initial, d_initial, nullptr, rows, seqlen, dtype,
-                            ASCAN_GATE_IDENTITY, Workspace{workspace, workspace_bytes}, stream);
+                            ASCAN_GATE_IDENTITY, false, Workspace{workspace, workspace_bytes}, stream);
+}
+
+int ascan_backward_reverse(const void* gates, const void* states, const void* initial, const void* grad_out,
+                           void* d_gates, void* d_tokens, void* d_initial, int64_t rows, int64_t seqlen, int dtype,
+                           void* workspace, size_t workspace_bytes, void* stream) {
+    return backward_checked(gates, states, grad_out, d_gates, d_tokens, initial, d_initial, nullptr, rows, seqlen, dtype,
+                            ASCAN_GATE_IDENTITY, true, Workspace{workspace, workspace_bytes}, stream);
 }
 
 int ascan_forward_gated(const void* gate_inputs, const void* tokens, const void* initial, void* out, int64_t rows,
@@ -285,14 +302,14 @@ int ascan_backward_gated(const void* gate_inputs, const void* states, const void
                          int dtype, int gate, void* workspace, size_t workspace_bytes, void* stream) {
     if (gate == ASCAN_GATE_SIGMOID_LERP) return ASCAN_ERR_BAD_ACTIVATION;  // needs the values: ascan_backward_lerp
     return backward_checked(gate_inputs, states, grad_out, d_gate_inputs, d_tokens, initial, d_initial, nullptr, rows,
-                            seqlen, dtype, gate, Workspace{workspace, workspace_bytes}, stream);
+                            seqlen, dtype, gate, false, Workspace{workspace, workspace_bytes}, stream);
 }
 
 int ascan_backward_lerp(const void* gate_inputs, const void* values, const void* states, const void* initial,
                         const void* grad_out, void* d_gate_inputs, void* d_values, void* d_initial, int64_t rows,
                         int64_t seqlen, int dtype, void* workspace, size_t workspace_bytes, void* stream) {
     return backward_checked(gate_inputs, states, grad_out, d_gate_inputs, d_values, initial, d_initial, values, rows,
-                            seqlen, dtype, ASCAN_GATE_SIGMOID_LERP, Workspace{workspace, workspace_bytes}, stream);
+                            seqlen, dtype, ASCAN_GATE_SIGMOID_LERP, false, Workspace{workspace, workspace_bytes}, stream);
 }
 
 unsigned int ascan_workspace_timeouts(const void* workspace_header_copy) {

@@ -20,7 +20,8 @@ struct BackwardBuffers {
     const void* values;  // the interpolating gate's fourth input, else null
 };
 
-template <class Tr, int W, bool ALIGNED, bool REGULAR, int ACT>
+// REV is the backward kernel's own direction: true for the backward pass of a forward-time scan.
+template <class Tr, bool REV, int W, bool ALIGNED, bool REGULAR, int ACT>
 hipError_t launch_backward(const BackwardBuffers& b, int64_t rows, int64_t T, int grid, int rows_per_block,
                            hipStream_t stream) {
     using S = typename Tr::S;
@@ -28,20 +29,20 @@ hipError_t launch_backward(const BackwardBuffers& b, int64_t rows, int64_t T, in
     constexpr int U = backward_blocks<ACT>(REGULAR ? Tuning<Tr>::UB : Tuning<Tr>::UBG);
     const unsigned blocks = (unsigned)((rows + rows_per_block - 1) / rows_per_block);
     const unsigned threads = 64u * W * rows_per_block;
-    return launch(scan_backward_kernel<Tr, W, U, ALIGNED, REGULAR, false, ACT, false>, blocks, threads, stream,
+    return launch(scan_backward_kernel<Tr, W, U, REV, ALIGNED, REGULAR, false, ACT, false>, blocks, threads, stream,
                   static_cast<const S*>(b.gates), static_cast<const S*>(b.states), static_cast<const S*>(b.grad_out),
                   static_cast<S*>(b.d_gates), static_cast<TokS*>(b.d_tokens), rows, T,
                   static_cast<SplitHeader*>(nullptr), static_cast<const S*>(b.initial), static_cast<S*>(b.d_initial),
                   grid, 0, static_cast<const S*>(b.values));
 }
 
-template <class Tr, bool REGULAR, int ACT>
+template <class Tr, bool REV, bool REGULAR, int ACT>
 hipError_t launch_backward_split(const BackwardBuffers& b, int64_t rows, int64_t T, int grid, int64_t ntiles,
                                  const Workspace& ws, hipStream_t stream) {
     using S = typename Tr::S;
     using TokS = typename Tr::TokS;
     constexpr int U = backward_blocks<ACT>(REGULAR ? SplitTuning<Tr>::UB : SplitTuning<Tr>::UBG);
-    auto kernel = scan_backward_kernel<Tr, kSplitWaves, U, true, REGULAR, true, ACT, false>;
+    auto kernel = scan_backward_kernel<Tr, kSplitWaves, U, REV, true, REGULAR, true, ACT, false>;
     const unsigned resident = resident_workgroups(kernel, 64 * kSplitWaves);
     if (resident == 0) return hipErrorInvalidConfiguration;
     const hipError_t e = reset_split_table(ws, rows, ntiles, stream);
@@ -54,20 +55,20 @@ hipError_t launch_backward_split(const BackwardBuffers& b, int64_t rows, int64_t
                   grid, 0, static_cast<const S*>(b.values));
 }
 
-template <class Tr, int PW, bool ALIGNED, int ACT>
+template <class Tr, bool REV, int PW, bool ALIGNED, int ACT>
 hipError_t launch_backward_packed(const BackwardBuffers& b, int64_t rows, int64_t T, int grid, int group,
                                   hipStream_t stream) {
     using S = typename Tr::S;
     using TokS = typename Tr::TokS;
     const unsigned blocks = (unsigned)((rows + group - 1) / group);
-    return launch(scan_backward_kernel<Tr, PW, Tuning<Tr>::UBG, ALIGNED, false, false, ACT, true>, blocks,
+    return launch(scan_backward_kernel<Tr, PW, Tuning<Tr>::UBG, REV, ALIGNED, false, false, ACT, true>, blocks,
                   64u * PW, stream, static_cast<const S*>(b.gates), static_cast<const S*>(b.states),
                   static_cast<const S*>(b.grad_out), static_cast<S*>(b.d_gates), static_cast<TokS*>(b.d_tokens), rows,
                   T, static_cast<SplitHeader*>(nullptr), static_cast<const S*>(b.initial),
                   static_cast<S*>(b.d_initial), grid, group, static_cast<const S*>(b.values));
 }
 
-template <class Tr>
+template <class Tr, bool REV>
 int backward_typed(const BackwardBuffers& b, int64_t rows, int64_t T, int act, const Workspace& ws,
                    hipStream_t stream) {
     constexpr int64_t kElem = (int64_t)sizeof(typename Tr::S);
@@ -91,8 +92,8 @@ int backward_typed(const BackwardBuffers& b, int64_t rows, int64_t T, int act, c
         if (same_lead && T * kElem >= kPackedWideRowBytes) {
             const int group = packed_group(rows, T, kElem, SUBG * kPackedWavesWide, at.grid);
             if (group != 0 && rows / group >= kPackedWideMinGroups) {
-                err = with_gate<Tr>(act, [&](auto gate) {
-                    return launch_backward_packed<Tr, kPackedWavesWide, true, decltype(gate)::value>(b, rows, T, at.grid,
+                err = with_gate<Tr, REV>(act, [&](auto gate) {
+                    return launch_backward_packed<Tr, REV, kPackedWavesWide, true, decltype(gate)::value>(b, rows, T, at.grid,
                                                                                                      group, stream);
                 });
                 return launch_status(err);
@@ -100,10 +101,10 @@ int backward_typed(const BackwardBuffers& b, int64_t rows, int64_t T, int act, c
         }
     }
     if (const int group = packed_group(rows, T, kElem, SUBG * kPackedWaves, same_lead ? at.grid : 1)) {
-        err = with_gate<Tr>(act, [&](auto gate) {
+        err = with_gate<Tr, REV>(act, [&](auto gate) {
             constexpr int ACT = decltype(gate)::value;
-            return same_lead ? launch_backward_packed<Tr, kPackedWaves, true, ACT>(b, rows, T, at.grid, group, stream)
-                             : launch_backward_packed<Tr, kPackedWaves, false, ACT>(b, rows, T, at.grid, group, stream);
+            return same_lead ? launch_backward_packed<Tr, REV, kPackedWaves, true, ACT>(b, rows, T, at.grid, group, stream)
+                             : launch_backward_packed<Tr, REV, kPackedWaves, false, ACT>(b, rows, T, at.grid, group, stream);
         });
         return launch_status(err);
     }
@@ -113,24 +114,24 @@ int backward_typed(const BackwardBuffers& b, int64_t rows, int64_t T, int act, c
         const bool regular = lead == 0 && T % (SUBS * kSplitWaves) == 0;
         const int64_t ntiles = host_tiles_per_row<Tr>(T, (regular ? SUBS : SUBSG) * kSplitWaves, regular, at);
         if (want_split(rows, ntiles) && workspace_fits(ws, rows, ntiles)) {
-            err = with_gate<Tr>(act, [&](auto gate) {
+            err = with_gate<Tr, REV>(act, [&](auto gate) {
                 constexpr int ACT = decltype(gate)::value;
-                return regular ? launch_backward_split<Tr, true, ACT>(b, rows, T, at.grid, ntiles, ws, stream)
-                               : launch_backward_split<Tr, false, ACT>(b, rows, T, at.grid, ntiles, ws, stream);
+                return regular ? launch_backward_split<Tr, REV, true, ACT>(b, rows, T, at.grid, ntiles, ws, stream)
+                               : launch_backward_split<Tr, REV, false, ACT>(b, rows, T, at.grid, ntiles, ws, stream);
             });
             return launch_status(err);
         }
     }
     auto with_waves = [&](auto aligned, auto reg) {
-        return with_gate<Tr>(act, [&](auto gate) {
+        return with_gate<Tr, REV>(act, [&](auto gate) {
             constexpr int ACT = decltype(gate)::value;
             constexpr bool AL = decltype(aligned)::value, REG = decltype(reg)::value;
             switch (plan.waves_per_row) {
-                case 1: return launch_backward<Tr, 1, AL, REG, ACT>(b, rows, T, at.grid, R, stream);
-                case 2: return launch_backward<Tr, 2, AL, REG, ACT>(b, rows, T, at.grid, R, stream);
-                case 4: return launch_backward<Tr, 4, AL, REG, ACT>(b, rows, T, at.grid, R, stream);
-                case 8: return launch_backward<Tr, 8, AL, REG, ACT>(b, rows, T, at.grid, R, stream);
-                default: return launch_backward<Tr, 16, AL, REG, ACT>(b, rows, T, at.grid, R, stream);
+                case 1: return launch_backward<Tr, REV, 1, AL, REG, ACT>(b, rows, T, at.grid, R, stream);
+                case 2: return launch_backward<Tr, REV, 2, AL, REG, ACT>(b, rows, T, at.grid, R, stream);
+                case 4: return launch_backward<Tr, REV, 4, AL, REG, ACT>(b, rows, T, at.grid, R, stream);
+                case 8: return launch_backward<Tr, REV, 8, AL, REG, ACT>(b, rows, T, at.grid, R, stream);
+                default: return launch_backward<Tr, REV, 16, AL, REG, ACT>(b, rows, T, at.grid, R, stream);
             }
         });
     };
@@ -147,12 +148,13 @@ int backward_typed(const BackwardBuffers& b, int64_t rows, int64_t T, int act, c
 }  // namespace
 }  // namespace ascan
 
-// Defines ascan::NAME, the backward entry of one dtype, in the including file.
-#define ASCAN_DEFINE_BACKWARD(NAME, TRAITS)                                                                     \
+// Defines ascan::NAME, the backward entry of one dtype, in the including file;
+// REV = true for the backward pass of forward-time scans, false for that of reverse scans.
+#define ASCAN_DEFINE_BACKWARD(NAME, TRAITS, REV)                                                                \
     int ascan::NAME(const ascan::BackwardCall& c) {                                                             \
         const ascan::BackwardBuffers b{c.gates, c.states, c.grad_out, c.d_gates, c.d_tokens, c.initial, c.d_initial, \
                                        c.values};                                                               \
-        return ascan::backward_typed<ascan::TRAITS>(b, c.rows, c.seqlen, c.gate, c.workspace, c.stream);        \
+        return ascan::backward_typed<ascan::TRAITS, REV>(b, c.rows, c.seqlen, c.gate, c.workspace, c.stream);   \
     }
 
 #endif  // ASCAN_BACKWARD_DISPATCH_H_

@@ -17,11 +17,17 @@ namespace {
 // ---------------------------------------------------------------------------
 // Fused backward kernel: reverse-time scan over gate[t+1] producing d_tokens,
 // and d_gates[t] = d_tokens[t] * conj(x[t-1]) in the same pass.
+// REV says which way the kernel's scan runs through memory.  REV = true is the
+// case above, the backward pass of a forward-time scan: the gradient scan runs
+// down the addresses.  REV = false is its mirror image, the backward pass of a
+// reverse scan x[t] = gate[t] x[t+1] + token[t]: g[t] = grad_out[t] + conj(gate[t-1]) g[t-1]
+// runs up the addresses and d_gates[t] = g[t] conj(x[t+1]).  Below, "after" and
+// "before" are meant in the order of the scan being differentiated.
 // With the interpolating gate (x[t] = a x[t-1] + (1 - a) v[t], a = sigmoid(z))
 // the kernel also reads the values v and writes, for the same g,
 // d_v[t] = g[t] (1 - a[t]) and d_z[t] = g[t] (x[t-1] - v[t]) a[t] (1 - a[t]).
 // ---------------------------------------------------------------------------
-template <class Tr, int W, int U, bool ALIGNED, bool REGULAR, bool SPLIT, int ACT, bool PACKED>
+template <class Tr, int W, int U, bool REV, bool ALIGNED, bool REGULAR, bool SPLIT, int ACT, bool PACKED>
 __global__ void __launch_bounds__(64 * kMaxWavesPerBlock)
     scan_backward_kernel(const typename Tr::S* __restrict__ gates, const typename Tr::S* __restrict__ states,
                          const typename Tr::S* __restrict__ grad_out, typename Tr::S* __restrict__ d_gates,
@@ -34,7 +40,11 @@ __global__ void __launch_bounds__(64 * kMaxWavesPerBlock)
     constexpr int64_t SUB = (int64_t)U * 64 * EPV;
     constexpr int64_t TILE = SUB * W;
     static_assert(!PACKED || (!SPLIT && !REGULAR), "packed rows use the general kernels, one group per workgroup");
+    static_assert(REV || ACT == kGateIdentity, "the gated scans run forward in time only");
     constexpr bool LERP = ACT == kGateSigmoidLerp;  // `values` is a fourth input
+    // index, inside a vector, of the element the gradient scan reaches first / last
+    constexpr int E_FIRST = REV ? Tr::EPV - 1 : 0;
+    constexpr int E_LAST = REV ? 0 : Tr::EPV - 1;
     constexpr int NIN = LERP ? 4 : 3;
 
     const int lane = threadIdx.x & 63;
@@ -91,19 +101,26 @@ __global__ void __launch_bounds__(64 * kMaxWavesPerBlock)
     // below: kept per lane they would sit in vector registers across the tile loop
     const int64_t row_scalar = (int64_t)__builtin_amdgcn_readfirstlane((int)row);
 
-    // Gradient of x[-1], conj(gate[0]) * g[0], from g at position 0 of the row's
-    // first tile.  Positions below the row's first element (position lo) carry
-    // gate 1 and grad_out 0, so with lo > 0 that g already is the gradient;
-    // with lo == 0 the last factor is still missing.
-    auto store_start_gradient = [&](V g_low) {
-        if (lo == 0) g_low = vmul(vconj(activate1<ACT>(Tr::load1(arow))), g_low);
-        if (lane == 0) Tr::store1(d_initial + row_scalar, g_low);
+    // Gradient of the state the differentiated scan started from (x[-1]; x[T] for a
+    // reverse scan), conj(gate) * g at the row's first (last) element, from g at the
+    // position where the gradient scan ends: position 0 of the row's first tile (the
+    // top of its last tile).  Positions outside the row carry gate 1 and grad_out 0,
+    // and the first of them past the row's end takes the row's outermost gate as the
+    // gate that "follows" it -- inside the sub-tile that holds that end.  So if that
+    // sub-tile goes on beyond the row, g already is the gradient when it leaves it;
+    // with the row flush against the sub-tile's edge the last factor is still missing
+    // (sub-tiles that hold nothing of the row are the identity, see a_edge below).
+    auto store_start_gradient = [&](V g_end) {
+        if (REV ? lo == 0 : hi % SUB == 0) {
+            g_end = vmul(vconj(activate1<ACT>(Tr::load1(arow + (REV ? 0 : hi - 1)))), g_end);
+        }
+        if (lane == 0) Tr::store1(d_initial + row_scalar, g_end);
     };
 
-    // Position of this wave's sub-tile in tile step k (reverse time).
+    // Position of this wave's sub-tile in tile step k of the gradient scan.
     auto sub_tile_base = [&](int64_t k) {
-        const int64_t tile = ntiles - 1 - k;
-        return tile * TILE + (int64_t)(W - 1 - w) * SUB;
+        const int64_t tile = REV ? ntiles - 1 - k : k;
+        return tile * TILE + (int64_t)(REV ? W - 1 - w : w) * SUB;
     };
     // One tile step of this wave; FULL as in the forward kernel.
     auto tile_step = [&](int64_t k, auto full_tag) {
@@ -124,10 +141,11 @@ __global__ void __launch_bounds__(64 * kMaxWavesPerBlock)
         S* __restrict__ dgsub = dgrow + sub_base;
         typename Tr::TokS* __restrict__ dtsub = dtrow + sub_base;
 
-        // x[-1], the state the forward scan started from (absent = zero), is
-        // needed by the sub-tile that holds the row's first element
+        // the state the differentiated scan started from (absent = zero) is needed by
+        // the sub-tile that holds the row's first element (last, for a reverse scan)
         V x_start = vzero<V>();
-        if (!PACKED && initial != nullptr && sub_base <= lo && lo < sub_end) x_start = Tr::load1(initial + row_scalar);  // wave-uniform
+        const int64_t start_at = REV ? lo : hi - 1;
+        if (!PACKED && initial != nullptr && sub_base <= start_at && start_at < sub_end) x_start = Tr::load1(initial + row_scalar);  // wave-uniform
         Cuts<Tr> cuts;  // packed rows take their initial states at the cuts instead
         if constexpr (PACKED) {
             cuts = stage_row_starts<Tr>(initial != nullptr ? initial + first_row : nullptr, (int)T, (int)len,
@@ -157,7 +175,7 @@ __global__ void __launch_bounds__(64 * kMaxWavesPerBlock)
         if (touches) {
 #pragma unroll
             for (int j = 0; j < U; ++j) {
-                const int off = vec_offset<U, EPV, true>(j, lane);
+                const int off = vec_offset<U, EPV, REV>(j, lane);
                 araw[j] = load_raw<Tr, ALIGNED, FULL>(asub, off, win, identity_gate<ACT, V>());
                 draw[j] = load_raw<Tr, ALIGNED, FULL>(dsub, off, win, vzero<V>());
                 xraw[j] = load_raw<Tr, ALIGNED, FULL>(xsub, off, win, x_start);
@@ -173,26 +191,30 @@ __global__ void __launch_bounds__(64 * kMaxWavesPerBlock)
             }
         }
 
-        // The two elements just outside the sub-tile: gate at sub_end and x at
-        // sub_base-1.  Addresses are clamped into the row so the loads are
-        // unconditional; out-of-row positions take the identity gate and x[-1].
+        // The two elements just outside the sub-tile: the gate where the gradient
+        // scan comes from (sub_end; sub_base-1 when it runs upwards) and x where it
+        // goes next (sub_base-1; sub_end).  Addresses are clamped into the row so the
+        // loads are unconditional; out-of-row positions take the identity gate and
+        // the state the differentiated scan started from.
         V a_edge, x_edge;
         {
-            const int64_t ia = sub_end < hi ? (sub_end > lo ? sub_end : lo) : hi - 1;
-            int64_t ix = sub_base - 1;
-            ix = ix < lo ? lo : (ix < hi ? ix : hi - 1);
+            const int64_t pa = REV ? sub_end : sub_base - 1;
+            const int64_t px = REV ? sub_base - 1 : sub_end;
+            const int64_t ia = pa < lo ? lo : (pa < hi ? pa : hi - 1);
+            const int64_t ix = px < lo ? lo : (px < hi ? px : hi - 1);
             const V av = activate1<ACT>(Tr::load1(arow + ia));
             const V xv = Tr::load1(xrow + ix);
-            a_edge = vselect(sub_end >= lo && sub_end < hi, av, vone<V>());
-            x_edge = vselect(sub_base - 1 >= lo && sub_base - 1 < hi, xv, x_start);
+            a_edge = vselect(touches && pa >= lo && pa < hi, av, vone<V>());
+            x_edge = vselect(px >= lo && px < hi, xv, x_start);
         }
 
         // Pass 1.  Gates are needed one element later (gate[t+1]) and states one
-        // element earlier (x[t-1]).  In scan order the vector at the next higher
-        // address belongs to lane-1 and the one at the next lower address to
-        // lane+1, so each block needs one value from each neighbour: a_next (the
-        // first gate of the vector above) and x_prev (the last state of the
-        // vector below).
+        // element earlier (x[t-1]) in the order of the differentiated scan.  The
+        // gradient scan runs the other way: the vector it visited just before this
+        // lane's belongs to lane-1 and the one it visits next to lane+1, so each
+        // block needs one value from each neighbour: a_next (the nearest gate of the
+        // vector visited before) and x_prev (the nearest state of the vector visited
+        // next).
         V a_next[U], x_prev[U];
         V totA[U], totX[U], exA[U], exX[U];
 #pragma unroll
@@ -208,35 +230,41 @@ __global__ void __launch_bounds__(64 * kMaxWavesPerBlock)
             } else {
                 V above[EPV];
                 Tr::unpack(araw[j > 0 ? j - 1 : 0], above);
-                hi_edge = read_lane<63>(activate1<ACT>(above[0]));
+                hi_edge = read_lane<63>(activate1<ACT>(above[E_LAST]));
             }
             if (j == U - 1) {
                 lo_edge = x_edge;
             } else {
                 V below[EPV];
                 Tr::unpack(xraw[j < U - 1 ? j + 1 : j], below);
-                lo_edge = read_lane<0>(below[EPV - 1]);
+                lo_edge = read_lane<0>(below[E_FIRST]);
             }
-            a_next[j] = shift_up1(a[0], hi_edge);
-            x_prev[j] = shift_down1(x[EPV - 1], lo_edge);
+            a_next[j] = shift_up1(a[E_LAST], hi_edge);
+            x_prev[j] = shift_down1(x[E_FIRST], lo_edge);
 
             // after[e]: the gate that follows element e; before[e]: the state that precedes it
             V after[EPV], before[EPV];
 #pragma unroll
             for (int e = 0; e < EPV; ++e) {
-                after[e] = e < EPV - 1 ? a[e + 1] : a_next[j];
-                before[e] = e > 0 ? x[e - 1] : x_prev[j];
+                if constexpr (REV) {
+                    after[e] = e < EPV - 1 ? a[e + 1] : a_next[j];
+                    before[e] = e > 0 ? x[e - 1] : x_prev[j];
+                } else {
+                    after[e] = e > 0 ? a[e - 1] : a_next[j];
+                    before[e] = e < EPV - 1 ? x[e + 1] : x_prev[j];
+                }
             }
             if constexpr (PACKED) {
                 bool is_first[EPV];
                 int row_of[EPV];
-                cut_rows_backward<Tr>(after, before, is_first, row_of,
-                                      (int)(sub_base - lo) + vec_offset<U, EPV, true>(j, lane), cuts);
+                cut_rows_backward<Tr, REV>(after, before, is_first, row_of,
+                                           (int)(sub_base - lo) + vec_offset<U, EPV, REV>(j, lane), cuts);
             }
-            V A = vconj(after[EPV - 1]);
-            V X = d[EPV - 1];
+            V A = vconj(after[E_FIRST]);
+            V X = d[E_FIRST];
 #pragma unroll
-            for (int e = EPV - 2; e >= 0; --e) {
+            for (int i = 1; i < EPV; ++i) {
+                const int e = REV ? EPV - 1 - i : i;
                 const V ga = vconj(after[e]);
                 X = carry_in<PACKED>(ga, X, d[e]);
                 A = gate_product<PACKED>(A, ga);
@@ -296,23 +324,29 @@ __global__ void __launch_bounds__(64 * kMaxWavesPerBlock)
             Tr::unpack(draw[j], d);
             Tr::unpack(xraw[j], x);
             if constexpr (LERP) Tr::unpack(vraw[j], v);
-            V gr = carry_in<PACKED>(exA[j], c, exX[j]);  // g entering this lane's vector from above
+            V gr = carry_in<PACKED>(exA[j], c, exX[j]);  // g entering this lane's vector
             c = carry_in<PACKED>(totA[j], c, totX[j]);
-            const int off = vec_offset<U, EPV, true>(j, lane);
+            const int off = vec_offset<U, EPV, REV>(j, lane);
             V after[EPV], before[EPV];
 #pragma unroll
             for (int e = 0; e < EPV; ++e) {
-                after[e] = e < EPV - 1 ? a[e + 1] : a_next[j];
-                before[e] = e > 0 ? x[e - 1] : x_prev[j];
+                if constexpr (REV) {
+                    after[e] = e < EPV - 1 ? a[e + 1] : a_next[j];
+                    before[e] = e > 0 ? x[e - 1] : x_prev[j];
+                } else {
+                    after[e] = e > 0 ? a[e - 1] : a_next[j];
+                    before[e] = e < EPV - 1 ? x[e + 1] : x_prev[j];
+                }
             }
             bool is_first[EPV];
             int row_of[EPV];
             if constexpr (PACKED) {
-                cut_rows_backward<Tr>(after, before, is_first, row_of, (int)(sub_base - lo) + off, cuts);
+                cut_rows_backward<Tr, REV>(after, before, is_first, row_of, (int)(sub_base - lo) + off, cuts);
             }
             V dt[EPV], dg[EPV], gs[PACKED ? EPV : 1];  // gs: g itself, for the rows' initial states
 #pragma unroll
-            for (int e = EPV - 1; e >= 0; --e) {
+            for (int i = 0; i < EPV; ++i) {
+                const int e = REV ? EPV - 1 - i : i;
                 gr = carry_in<PACKED>(vconj(after[e]), gr, d[e]);
                 if constexpr (PACKED) gs[e] = gr;
                 if constexpr (LERP) {
@@ -340,8 +374,8 @@ __global__ void __launch_bounds__(64 * kMaxWavesPerBlock)
             }
         }
 
-        // A split row's last tile step ends at the row's first element: after
-        // pass 2, c is g at the lowest position of this wave's sub-tile.
+        // A split row's last tile step ends where the differentiated scan started: after
+        // pass 2, c is g at the last position this wave's sub-tile holds in the gradient scan.
         if constexpr (SPLIT) {
             if (d_initial != nullptr && k == ntiles - 1 && w == W - 1) store_start_gradient(c);  // wave-uniform
         }
@@ -359,7 +393,7 @@ __global__ void __launch_bounds__(64 * kMaxWavesPerBlock)
             }
         }
     }
-    // after the last tile step the carry is g at position 0 of the first tile
+    // after the last tile step the carry is g at the position where the gradient scan ends
     if constexpr (!SPLIT && !PACKED) {
         if (d_initial != nullptr && w == 0) store_start_gradient(carry);  // wave-uniform
     }

@@ -1,0 +1,4 @@
+// Backward kernels of reverse scans and their dispatch for one dtype (TraitsC64RealTokens).
+#include "backward_dispatch.h"
+
+ASCAN_DEFINE_BACKWARD(backward_reverse_c64_real_tokens, TraitsC64RealTokens, false)

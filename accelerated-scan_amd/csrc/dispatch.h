@@ -1,6 +1,7 @@
-// What the C entry points (ascan.hip) call: one forward and one backward
-// function per dtype, each compiled in a translation unit of its own
-// (forward_<dtype>.hip, backward_<dtype>.hip) together with its kernels.
+// What the C entry points (ascan.hip) call: one forward function and two backward
+// functions (for forward-time and for reverse scans) per dtype, each compiled in a
+// translation unit of its own (forward_<dtype>.hip, backward_<dtype>.hip,
+// backward_reverse_<dtype>.hip) together with its kernels.
 #ifndef ASCAN_DISPATCH_H_
 #define ASCAN_DISPATCH_H_
 
@@ -55,6 +56,12 @@ int backward_bf16(const BackwardCall& call);
 int backward_f16(const BackwardCall& call);
 int backward_c64(const BackwardCall& call);
 int backward_c64_real_tokens(const BackwardCall& call);
+// Backward passes of reverse scans (identity gate only).
+int backward_reverse_f32(const BackwardCall& call);
+int backward_reverse_bf16(const BackwardCall& call);
+int backward_reverse_f16(const BackwardCall& call);
+int backward_reverse_c64(const BackwardCall& call);
+int backward_reverse_c64_real_tokens(const BackwardCall& call);
 
 // hipError_t of the calling thread's last failed launch (defined in ascan.hip).
 extern thread_local int g_last_hip_error;

@@ -103,12 +103,14 @@ __device__ __forceinline__ void cut_rows(typename Tr::V (&g)[Tr::EPV], typename 
 }
 
 // Backward scan: `after[e]` is the gate that follows element e in its row and
-// `before[e]` the state that precedes it; at a row's last element nothing
-// follows (0), at its first the state before it is the row's initial state.
-// is_first[e] / row_of[e] tell the caller where to put the gradient of that
-// initial state.  Rows at least as long as a vector have at most one first and
-// one last element in a vector (as above).
-template <class Tr>
+// `before[e]` the state that precedes it, both in the order of the scan being
+// differentiated (REV = true: forward in time, as the backward kernel names its
+// own direction; false: a reverse scan, whose first element is the row's last in
+// memory); at a row's last element nothing follows (0), at its first the state
+// before it is the row's initial state.  is_first[e] / row_of[e] tell the caller
+// where to put the gradient of that initial state.  Rows at least as long as a
+// vector have at most one first and one last element in a vector (as above).
+template <class Tr, bool REV>
 __device__ __forceinline__ void cut_rows_backward(typename Tr::V (&after)[Tr::EPV], typename Tr::V (&before)[Tr::EPV],
                                                   bool (&is_first)[Tr::EPV], int (&row_of)[Tr::EPV], int rel0,
                                                   const Cuts<Tr>& cuts) {
@@ -116,9 +118,13 @@ __device__ __forceinline__ void cut_rows_backward(typename Tr::V (&after)[Tr::EP
     int row, pos;
     split_position(rel0, cuts.T, cuts.inv_T, row, pos);
     if (cuts.T >= Tr::EPV) {  // wave-uniform
-        const int first_e = pos == 0 ? 0 : cuts.T - pos;
-        const int last_e = cuts.T - 1 - pos;
-        const int first_row = row + (pos != 0);
+        // where a row starts (pos 0) and where a row ends (pos T-1) inside this vector, in memory order
+        const int low_e = pos == 0 ? 0 : cuts.T - pos;
+        const int high_e = cuts.T - 1 - pos;
+        const int low_row = row + (pos != 0);
+        const int first_e = REV ? low_e : high_e;  // first element of its row in the differentiated scan's order
+        const int last_e = REV ? high_e : low_e;
+        const int first_row = REV ? low_row : row;
         const bool first_valid = first_e < Tr::EPV && (unsigned)(rel0 + first_e) < (unsigned)cuts.len;
         const bool last_valid = last_e < Tr::EPV && (unsigned)(rel0 + last_e) < (unsigned)cuts.len;
         const int first_at = first_valid ? first_e : -1;
@@ -138,8 +144,8 @@ __device__ __forceinline__ void cut_rows_backward(typename Tr::V (&after)[Tr::EP
 #pragma unroll
     for (int e = 0; e < Tr::EPV; ++e) {
         const bool valid = (unsigned)(rel0 + e) < (unsigned)cuts.len;
-        const bool first = valid && pos == 0;
-        const bool last = valid && pos == cuts.T - 1;
+        const bool first = valid && pos == (REV ? 0 : cuts.T - 1);
+        const bool last = valid && pos == (REV ? cuts.T - 1 : 0);
         V start = vzero<V>();
         if (cuts.stage != nullptr && first) start = Tr::load1(cuts.stage + (row - cuts.first_row));
         before[e] = vselect(first, start, before[e]);

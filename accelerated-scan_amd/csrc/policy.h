@@ -315,10 +315,11 @@ template <class Tr>
 constexpr bool kHasSigmoid = std::is_same<typename Tr::V, float>::value;
 
 // Calls f(std::integral_constant<int, ACT>) for the gate code `act`, which the
-// entry points have validated against the dtype.
-template <class Tr, class F>
+// entry points have validated against the dtype.  SCAN_FORWARD = false (reverse
+// scans and their backward pass) has the identity gate only.
+template <class Tr, bool SCAN_FORWARD = true, class F>
 hipError_t with_gate(int act, F&& f) {
-    if constexpr (kHasSigmoid<Tr>) {
+    if constexpr (kHasSigmoid<Tr> && SCAN_FORWARD) {
         if (act == kGateSigmoid) return f(std::integral_constant<int, kGateSigmoid>{});
         if (act == kGateSigmoidLerp) return f(std::integral_constant<int, kGateSigmoidLerp>{});
         if (act == kGateExp) return f(std::integral_constant<int, kGateExp>{});

@@ -62,7 +62,7 @@
 extern "C" {
 #endif
 
-#define ASCAN_ABI_VERSION 7
+#define ASCAN_ABI_VERSION 8
 
 /* Marks the exported entry points (the library is built with hidden visibility). */
 #define ASCAN_API __attribute__((visibility("default")))
@@ -234,6 +234,27 @@ ASCAN_API int ascan_backward_from(const void* gates, const void* states, const v
                         const void* grad_out, void* d_gates, void* d_tokens, void* d_initial,
                         int64_t rows, int64_t seqlen, int dtype,
                         void* workspace, size_t workspace_bytes, void* stream);
+
+/*
+ * Backward pass of a reverse scan, y[t] = gate[t] * y[t+1] + token[t] with
+ * y[seqlen] = initial (NULL: 0), i.e. of ascan_forward / ascan_forward_from /
+ * ascan_forward_split called with reverse != 0.  `states` is that call's output.
+ *
+ *     g[t]        = grad_out[t] + conj(gate[t-1]) * g[t-1]     (a forward-time scan, g[-1] = 0)
+ *     d_tokens[t] = g[t]
+ *     d_gates[t]  = g[t] * conj(y[t+1])                        (y[seqlen] = initial)
+ *     d_initial   = conj(gate[seqlen-1]) * g[seqlen-1]
+ *
+ * One fused pass like ascan_backward, mirrored in time.  No counterpart in the
+ * reference: its reverse scan (warp.py:32-35, the `reverse` argument of
+ * warp.cuh:395) exists to compute gradients and is not differentiable itself;
+ * layers that scan a sequence in both directions need this.  Arguments as for
+ * ascan_backward_from; initial, d_initial and workspace may each be NULL.
+ */
+ASCAN_API int ascan_backward_reverse(const void* gates, const void* states, const void* initial,
+                           const void* grad_out, void* d_gates, void* d_tokens, void* d_initial,
+                           int64_t rows, int64_t seqlen, int dtype,
+                           void* workspace, size_t workspace_bytes, void* stream);
 
 /*
  * Scans whose gates come out of a non-linearity, applied in registers: the

@@ -110,8 +110,14 @@ def forward_from(gates, tokens, initial, reverse=False):
     return out
 
 
-def backward_from(gates, states, initial, grad_out):
-    """(d_gates, d_tokens, d_initial) of the scan started from ``initial``, in fp64."""
+def backward_from(gates, states, initial, grad_out, reverse=False):
+    """(d_gates, d_tokens, d_initial) of the scan started from ``initial``, in fp64.
+    ``reverse``: of the reverse scan ``forward_from(..., reverse=True)``, which is the forward scan of the
+    sequences flipped in time, flipped: its gradients are those of that scan, flipped."""
+    if reverse:
+        flip = lambda a: np.ascontiguousarray(np.flip(np.asarray(a), -1))
+        dg, dx, di = backward_from(flip(gates), flip(states), initial, flip(grad_out))
+        return flip(dg), flip(dx), di
     lib = _load()
     cplx = any(np.iscomplexobj(a) for a in (gates, states, initial, grad_out))
     dt = np.complex64 if cplx else np.float32

@@ -139,6 +139,29 @@ void check_problem(int64_t rows, int64_t T, bool with_initial, hipStream_t strea
     EXPECT(worst(h_dx, t_dx) <= tol);
     EXPECT(worst(h_dg, t_dg) <= tol);
     if (with_initial) EXPECT(worst(download(d_init, rows, stream), t_di) <= tol);
+
+    // Backward pass of the reverse scan: the loops run on the sequences flipped in time.
+    {
+        EXPECT(ascan_backward_reverse(dg_in.p, rev.p, init_dev, dd_in.p, d_gates.p, d_tokens.p, with_initial ? d_init.p : nullptr,
+                                      rows, T, ASCAN_F32, ws_ptr, ws_bytes, stream) == ASCAN_OK);
+        auto flipped = [&](const std::vector<float>& v) {
+            std::vector<float> f(v.size());
+            for (int64_t r = 0; r < rows; ++r)
+                for (int64_t t = 0; t < T; ++t) f[r * T + t] = v[r * T + (T - 1 - t)];
+            return f;
+        };
+        const std::vector<float> fg = flipped(g), fs = flipped(h_rev), fd = flipped(d);
+        std::vector<double> f_dg(n), f_dx(n);
+        seq_backward_from_f32(fg.data(), fs.data(), init_host, fd.data(), f_dg.data(), f_dx.data(), t_di.data(), rows, T);
+        for (int64_t r = 0; r < rows; ++r)
+            for (int64_t t = 0; t < T; ++t) {
+                t_dg[r * T + t] = f_dg[r * T + (T - 1 - t)];
+                t_dx[r * T + t] = f_dx[r * T + (T - 1 - t)];
+            }
+        EXPECT(worst(download(d_tokens, n, stream), t_dx) <= tol);
+        EXPECT(worst(download(d_gates, n, stream), t_dg) <= tol);
+        if (with_initial) EXPECT(worst(download(d_init, rows, stream), t_di) <= tol);
+    }
     if (ws_bytes) {
         unsigned char header[64];
         HIP_OK(hipMemcpy(header, ws.p, sizeof(header), hipMemcpyDeviceToHost));

@@ -73,6 +73,12 @@ def test_argument_validation_returns_codes():
     assert lib.ascan_forward(p + 1, p, p, 1, 4, 1, 0, None) == 4
     assert lib.ascan_forward(p + 4, p, p, 1, 4, 3, 0, None) == 4
     assert lib.ascan_backward(p, p, p, p + 2, p, 1, 4, 0, None) == 4
+    # the reverse scan's backward pass validates like the forward-time one
+    assert lib.ascan_backward_reverse(p, p, None, p, p, p, None, -1, 4, 0, None, 0, None) == 2
+    assert lib.ascan_backward_reverse(None, None, None, None, None, None, None, 0, 4, 0, None, 0, None) == 0
+    assert lib.ascan_backward_reverse(p, p, None, p, None, p, None, 1, 4, 0, None, 0, None) == 1
+    assert lib.ascan_backward_reverse(p, p, None, p, p + 2, p, None, 1, 4, 0, None, 0, None) == 4
+    assert lib.ascan_backward_reverse(p, p, None, p, p, p, None, 1, 4, 9, None, 0, None) == 3
 
 
 def test_overlapping_buffers_are_refused():
@@ -90,6 +96,7 @@ def test_overlapping_buffers_are_refused():
     assert lib.ascan_backward(p, p + 64, p + 128, p + 128, p + 256, 1, n, 0, None) == 7      # d_gates is grad_out
     assert lib.ascan_backward(p, p + 64, p + 128, p + 256, p + 256 + 32, 1, n, 0, None) == 7  # the two outputs overlap
     assert lib.ascan_backward_from(p, p + 64, None, p + 128, p + 192, p + 256, p + 192 + 8, 1, n, 0, None, 0, None) == 7
+    assert lib.ascan_backward_reverse(p, p + 64, None, p + 128, p + 192, p + 256, p + 192 + 8, 1, n, 0, None, 0, None) == 7
     # complex gates with real tokens: the token buffers are half as long
     assert lib.ascan_forward(p, p + 256, p + 256 + 56, 1, n, 4, 0, None) == 7   # 16 c64 = 128 bytes, tokens 64 bytes
     # bf16: 32 bytes per row; ranges that only touch are fine for the check (the

@@ -122,6 +122,8 @@ def test_opcheck_stateful_ops():
     torch.library.opcheck(_ops.scan_forward_from, (g, x, initial, True))
     states = _ops.scan_forward_from(g, x, initial, False)
     torch.library.opcheck(_ops.scan_backward_from, (g, states, initial, weight, False))
+    reverse_states = _ops.scan_forward_from(g, x, initial, True)
+    torch.library.opcheck(_ops.scan_backward_reverse, (g, reverse_states, initial, weight, False))
     gc = torch.polar(g, x)
     ic = torch.complex(initial, initial.flip(0))
     sc = _ops.scan_forward_from(gc, x, ic, False)

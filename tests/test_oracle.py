@@ -310,6 +310,14 @@ def test_from_vs_autograd_of_loop(T, cplx):
     np.testing.assert_allclose(dt, dt_ref.numpy(), rtol=1e-12, atol=1e-12)
     np.testing.assert_allclose(di, di_ref.numpy(), rtol=1e-12, atol=1e-12)
     np.testing.assert_allclose(dg, dg_ref.numpy(), rtol=1e-5, atol=1e-5)  # states rounded to fp32 before the multiply
+    # the reverse scan's gradients against autograd through the loop run from the last element down
+    out_rev = _loop_scan_from(gw, tw, iw, reverse=True)
+    rdg_ref, rdt_ref, rdi_ref = torch.autograd.grad(out_rev, (gw, tw, iw), grad_out.to(wide))
+    rdg, rdt, rdi = seqscan.backward_from(gates.numpy(), rev.astype(gates.numpy().dtype), initial.numpy(), grad_out.numpy(),
+                                          reverse=True)
+    np.testing.assert_allclose(rdt, rdt_ref.numpy(), rtol=1e-12, atol=1e-12)
+    np.testing.assert_allclose(rdi, rdi_ref.numpy(), rtol=1e-12, atol=1e-12)
+    np.testing.assert_allclose(rdg, rdg_ref.numpy(), rtol=1e-5, atol=1e-5)
 
 
 # ---------------------------------------------------------------------------

@@ -155,8 +155,9 @@ def _tolerance(dtype):
     return dict(rtol=2 * storage_ulp[dtype], atol=2 * storage_ulp[dtype])
 
 
-def _compare_with_truth(gates, tokens, grad_out, out, rev, dg, dx, dtype, what=""):
-    """GPU results (any layout with rows*T elements) against the fp64 loops."""
+def _compare_with_truth(gates, tokens, grad_out, out, rev, dg, dx, dtype, what="", reverse_grads=None):
+    """GPU results (any layout with rows*T elements) against the fp64 loops.
+    ``reverse_grads``: (d_gates, d_tokens) of the reverse scan, computed from ``rev``."""
     rows, T = gates.shape
     tol = _tolerance(dtype)
     tok = _np32(tokens).astype(np.complex64) if dtype == C64_REAL_TOKENS else _np32(tokens)
@@ -168,7 +169,17 @@ def _compare_with_truth(gates, tokens, grad_out, out, rev, dg, dx, dtype, what="
     if dtype == C64_REAL_TOKENS:
         t_dx = t_dx.real  # real tokens keep the real part of their gradient
         assert dx.dtype == torch.float32
-    for name, got, want in (("out", out, t_out), ("rev", rev, t_rev), ("d_tokens", dx, t_dx), ("d_gates", dg, t_dg)):
+    pairs = [("out", out, t_out), ("rev", rev, t_rev), ("d_tokens", dx, t_dx), ("d_gates", dg, t_dg)]
+    if reverse_grads is not None:
+        rdg, rdx = reverse_grads
+        zero = np.zeros(rows, dtype=_np32(gates).dtype)
+        t_rdg, t_rdx, _ = seqscan.backward_from(_np32(gates), _np32(rev.reshape(rows, T).cpu()), zero, _np32(grad_out),
+                                                reverse=True)
+        if dtype == C64_REAL_TOKENS:
+            t_rdx = t_rdx.real
+            assert rdx.dtype == torch.float32
+        pairs += [("reverse d_tokens", rdx, t_rdx), ("reverse d_gates", rdg, t_rdg)]
+    for name, got, want in pairs:
         got = _np32(got.reshape(rows, T).cpu())
         scale = max(1.0, float(np.abs(want).max()))
         np.testing.assert_allclose(
@@ -189,8 +200,11 @@ def _check_against_truth(gates, tokens, grad_out, dtype, what=""):
     dg = torch.empty_like(g)
     dx = torch.empty_like(x)
     _abi.backward(g, out, d, dg, dx)
+    rdg = torch.empty_like(g)
+    rdx = torch.empty_like(x)
+    _abi.backward(g, rev, d, rdg, rdx, reverse=True)
     torch.cuda.synchronize()
-    _compare_with_truth(gates, tokens, grad_out, out, rev, dg, dx, dtype, what)
+    _compare_with_truth(gates, tokens, grad_out, out, rev, dg, dx, dtype, what, reverse_grads=(rdg, rdx))
 
 
 ALL_DTYPES = [torch.float32, torch.bfloat16, torch.float16, torch.complex64, C64_REAL_TOKENS]
@@ -265,10 +279,14 @@ def test_unaligned_base_pointer(dtype, offsets, rows, T):
     _abi.forward(g, x, out, False)
     _abi.forward(g, x, rev, True)
     _abi.backward(g, out, d, dg, dx)
+    rdg, rdx = offset_copy(torch.zeros_like(gates), ox), offset_copy(torch.zeros_like(tokens), oo)
+    for t in (rdg, rdx):
+        t.untyped_storage().fill_(0)
+    _abi.backward(g, rev, d, rdg, rdx, reverse=True)
     torch.cuda.synchronize()
-    _compare_with_truth(gates, tokens, grad_out, out, rev, dg, dx, dtype, what="offset views")
+    _compare_with_truth(gates, tokens, grad_out, out, rev, dg, dx, dtype, what="offset views", reverse_grads=(rdg, rdx))
     # nothing was written outside the row range of any output
-    for t in (out, rev, dg, dx):
+    for t in (out, rev, dg, dx, rdg, rdx):
         k = t.storage_offset()
         whole = torch.empty(0, dtype=t.dtype, device=DEVICE).set_(t.untyped_storage())
         assert whole[:k].abs().sum().item() == 0 and whole[k + rows * T:].abs().sum().item() == 0
@@ -761,13 +779,15 @@ def test_split_rows(dtype, rows, T):
     out, rev, dg = (torch.empty_like(g) for _ in range(3))
     dx = torch.empty_like(x)
     # zeroed, because a shape the library decides not to split leaves the table untouched
-    spaces = [torch.zeros(nbytes, dtype=torch.uint8, device=DEVICE) for _ in range(3)]
+    spaces = [torch.zeros(nbytes, dtype=torch.uint8, device=DEVICE) for _ in range(4)]
     _abi.forward(g, x, out, False, workspace=spaces[0])
     _abi.forward(g, x, rev, True, workspace=spaces[1])
     _abi.backward(g, out, d, dg, dx, workspace=spaces[2])
+    rdg, rdx = torch.empty_like(g), torch.empty_like(x)
+    _abi.backward(g, rev, d, rdg, rdx, workspace=spaces[3], reverse=True)
     torch.cuda.synchronize()
-    assert [_abi.workspace_timeouts(w) for w in spaces] == [0, 0, 0]
-    _compare_with_truth(gates, tokens, grad_out, out, rev, dg, dx, dtype, what="split")
+    assert [_abi.workspace_timeouts(w) for w in spaces] == [0, 0, 0, 0]
+    _compare_with_truth(gates, tokens, grad_out, out, rev, dg, dx, dtype, what="split", reverse_grads=(rdg, rdx))
 
 
 def test_split_matches_unsplit_and_autograd_path():
@@ -908,9 +928,12 @@ def test_random_shapes_and_offsets(case):
     _abi.forward(g, x, out, False)
     _abi.forward(g, x, rev, True)
     _abi.backward(g, out, d, dg, dx)
+    rdg, rdx = offset_copy(torch.zeros_like(gates), offsets[5]), offset_copy(torch.zeros_like(tokens), offsets[6])
+    _abi.backward(g, rev, d, rdg, rdx, reverse=True)
     torch.cuda.synchronize()
-    _compare_with_truth(gates, tokens, grad_out, out, rev, dg, dx, dtype, what=f"random case {case}")
-    for t in (out, rev, dg, dx):
+    _compare_with_truth(gates, tokens, grad_out, out, rev, dg, dx, dtype, what=f"random case {case}",
+                        reverse_grads=(rdg, rdx))
+    for t in (out, rev, dg, dx, rdg, rdx):
         k = t.storage_offset()
         whole = torch.empty(0, dtype=t.dtype, device=DEVICE).set_(t.untyped_storage())
         assert whole[:k].abs().sum().item() == 0 and whole[k + rows * T:].abs().sum().item() == 0

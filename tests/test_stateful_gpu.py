@@ -62,7 +62,7 @@ def _tolerance(dtype):
     return 2 * storage_ulp[dtype]
 
 
-def _compare(gates, tokens, grad_out, initial, out, rev, dg, dx, di, dtype, what):
+def _compare(gates, tokens, grad_out, initial, out, rev, dg, dx, di, dtype, what, reverse_grads=None):
     rows, T = gates.shape
     tol = _tolerance(dtype)
     tok = _np32(tokens).astype(np.complex64) if dtype == C64_REAL_TOKENS else _np32(tokens)
@@ -73,8 +73,17 @@ def _compare(gates, tokens, grad_out, initial, out, rev, dg, dx, di, dtype, what
     if dtype == C64_REAL_TOKENS:
         t_dx = t_dx.real
         assert dx.dtype == torch.float32
-    pairs = (("out", out, t_out), ("rev", rev, t_rev), ("d_tokens", dx, t_dx), ("d_gates", dg, t_dg),
-             ("d_initial", di, t_di))
+    pairs = [("out", out, t_out), ("rev", rev, t_rev), ("d_tokens", dx, t_dx), ("d_gates", dg, t_dg),
+             ("d_initial", di, t_di)]
+    if reverse_grads is not None:  # backward pass of the reverse scan, from the reverse states the GPU produced
+        rdg, rdx, rdi = reverse_grads
+        rev_states = rev.reshape(rows, T).cpu()
+        t_rdg, t_rdx, t_rdi = seqscan.backward_from(_np32(gates), _np32(rev_states), _np32(initial), _np32(grad_out),
+                                                    reverse=True)
+        if dtype == C64_REAL_TOKENS:
+            t_rdx = t_rdx.real
+            assert rdx.dtype == torch.float32
+        pairs += [("reverse d_tokens", rdx, t_rdx), ("reverse d_gates", rdg, t_rdg), ("reverse d_initial", rdi, t_rdi)]
     for name, got, want in pairs:
         got = _np32(got.reshape(want.shape).cpu())
         scale = max(1.0, float(np.abs(want).max()))
@@ -104,8 +113,11 @@ def _run_and_compare(rows, T, dtype, seed, what, offsets=(0, 0, 0)):
     _abi.forward(g, x, out, False, initial=init)
     _abi.forward(g, x, rev, True, initial=init)
     _abi.backward(g, out, d, dg, dx, initial=init, d_initial=di)
+    rdg, rdx = _offset_copy(torch.zeros_like(gates), shape, ox), _offset_copy(torch.zeros_like(tokens), shape, oo)
+    rdi = _offset_copy(torch.full_like(initial, float("nan")), (1, rows), 2)
+    _abi.backward(g, rev, d, rdg, rdx, initial=init, d_initial=rdi, reverse=True)
     torch.cuda.synchronize()
-    _compare(gates, tokens, grad_out, initial, out, rev, dg, dx, di, dtype, what)
+    _compare(gates, tokens, grad_out, initial, out, rev, dg, dx, di, dtype, what, reverse_grads=(rdg, rdx, rdi))
 
 
 @pytest.mark.parametrize("dtype", ALL_DTYPES, ids=ALL_IDS)
@@ -246,6 +258,55 @@ def test_chunked_scan_equals_whole_scan(module, dtype):
     torch.testing.assert_close(dx_parts, dx_whole, **gtol)
     gtol = dict(rtol=tol["rtol"], atol=tol["rtol"] * max(1.0, dg_whole.abs().max().item()))
     torch.testing.assert_close(dg_parts, dg_whole, **gtol)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.complex64, C64_REAL_TOKENS],
+                         ids=["fp32", "bf16", "c64", "c64_real_tokens"])
+@pytest.mark.parametrize("mode", ["eager", "aot_eager"])
+def test_bidirectional_scan_through_autograd(dtype, mode):
+    """A sequence scanned in both directions, ``scan(g, x, h) + scan(g, x, h, reverse=True)``, through the
+    modules' autograd nodes: values and all gradients against the fp64 loops (the reverse scan has a fused
+    backward kernel of its own)."""
+    from accelerated_scan import stateful
+    from accelerated_scan.warp import scan as warp_scan
+
+    B, C, T = 2, 40, 20011
+    gates, tokens, grad_out, initial = _inputs(B * C, T, dtype, seed=21)
+    g = gates.reshape(B, C, T).to(DEVICE).requires_grad_(True)
+    x = tokens.reshape(B, C, T).to(DEVICE).requires_grad_(True)
+    h = initial.reshape(B, C).to(DEVICE).requires_grad_(True)
+    d = grad_out.reshape(B, C, T).to(DEVICE)
+
+    def both(g, x, h):
+        return stateful.scan(g, x, h), stateful.scan(g, x, h, reverse=True)
+
+    fn = torch.compile(both, backend=mode, fullgraph=True) if mode != "eager" else both
+    fwd, rev = fn(g, x, h)
+    dg, dx, dh = torch.autograd.grad(fwd + rev, (g, x, h), d)
+
+    tol = _tolerance(dtype)
+    G, X, H, D = _np32(gates), _np32(tokens), _np32(initial), _np32(grad_out)
+    tok = X.astype(np.complex64) if dtype == C64_REAL_TOKENS else X
+    t_fwd = seqscan.forward_from(G, tok, H)
+    t_rev = seqscan.forward_from(G, tok, H, reverse=True)
+    f_dg, f_dx, f_dh = seqscan.backward_from(G, _np32(fwd.detach().reshape(B * C, T).cpu()), H, D)
+    r_dg, r_dx, r_dh = seqscan.backward_from(G, _np32(rev.detach().reshape(B * C, T).cpu()), H, D, reverse=True)
+    t_dx = f_dx + r_dx
+    if dtype == C64_REAL_TOKENS:
+        t_dx = t_dx.real
+    # the two gradients are summed by autograd in storage precision: one more rounding for 16-bit
+    gtol = tol if dtype != torch.bfloat16 else 2 * tol
+    for name, got, want, t in (("forward states", fwd, t_fwd, tol), ("reverse states", rev, t_rev, tol),
+                               ("d_tokens", dx, t_dx, gtol), ("d_gates", dg, f_dg + r_dg, gtol),
+                               ("d_initial", dh, f_dh + r_dh, gtol)):
+        got = _np32(got.detach().reshape(want.shape).cpu())
+        scale = max(1.0, float(np.abs(want).max()))
+        np.testing.assert_allclose(got, want, rtol=t, atol=t * scale, err_msg=f"{name} {dtype} {mode}")
+    # the keyword of warp.scan reaches the same operator
+    if dtype in (torch.float32, torch.bfloat16):
+        assert torch.equal(warp_scan(g, x, h, reverse=True), rev)
+        torch.testing.assert_close(warp_scan(g, x, reverse=True).float(),
+                                   stateful.scan(g, x, torch.zeros_like(h), reverse=True).float(), rtol=0, atol=0)
 
 
 def test_gradient_of_initial_against_autograd_of_the_loop():
