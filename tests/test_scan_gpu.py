@@ -743,6 +743,70 @@ def test_raw_c_abi_on_a_side_stream():
     np.testing.assert_allclose(dg.cpu().numpy(), t_dg, rtol=2e-5, atol=2e-5 * np.abs(t_dg).max())
 
 
+def test_host_threads_call_concurrently():
+    """The entry points are re-entrant: four host threads, each on its own stream,
+    issue forward + backward calls of different dtypes and launch plans (packed,
+    one wave per row, sixteen waves, split rows) at the same time -- ctypes drops
+    the GIL for the duration of a call -- and every result equals that of the same
+    call made alone.  The reference's operator is entered from the user's thread
+    and from autograd's backward thread alike (warp.py:38-65)."""
+    import threading
+
+    from accelerated_scan import _abi
+
+    lib = _abi.load()
+    cases = [(5000, 24, torch.float32, 0), (700, 1031, torch.bfloat16, 1), (9, 70000, torch.float16, 2),
+             (4, 1 << 18, torch.float32, 0)]
+    work = []
+    for i, (rows, T, dtype, code) in enumerate(cases):
+        gen = torch.Generator().manual_seed(100 + i)
+        g, x, d = (torch.rand(rows, T, generator=gen).to(dtype).to(DEVICE) for _ in range(3))
+        nbytes = lib.ascan_workspace_bytes(rows, T, code)
+        table = torch.empty(max(nbytes, 64), dtype=torch.uint8, device=DEVICE)
+        alone = [torch.empty_like(g) for _ in range(3)]
+        together = [torch.empty_like(g) for _ in range(3)]
+        work.append((rows, T, code, g, x, d, table, nbytes, alone, together, torch.cuda.Stream()))
+
+    def run(item, which, repeats):
+        rows, T, code, g, x, d, table, nbytes, alone, together, stream = item
+        out, dg, dx = alone if which == 0 else together
+        for _ in range(repeats):
+            rc = lib.ascan_forward_split(g.data_ptr(), x.data_ptr(), out.data_ptr(), rows, T, code, 0,
+                                         table.data_ptr() if nbytes else None, nbytes, stream.cuda_stream)
+            assert rc == 0, rc
+            rc = lib.ascan_backward_split(g.data_ptr(), out.data_ptr(), d.data_ptr(), dg.data_ptr(), dx.data_ptr(), rows,
+                                          T, code, table.data_ptr() if nbytes else None, nbytes, stream.cuda_stream)
+            assert rc == 0, rc
+        stream.synchronize()
+
+    torch.cuda.synchronize()
+    for item in work:
+        run(item, 0, 1)
+    failures = []
+
+    def guarded(item):
+        try:
+            run(item, 1, 40)
+        except BaseException as e:  # noqa: BLE001 - reported by the main thread
+            failures.append(repr(e))
+
+    threads = [threading.Thread(target=guarded, args=(item,)) for item in work]
+    for t in threads:
+        t.start()
+    for t in threads:
+        t.join()
+    torch.cuda.synchronize()
+    assert not failures, failures
+    for item in work:
+        for a, b in zip(item[8], item[9]):
+            if item[7]:  # split rows: the look-back folds whatever its predecessors have published by then
+                torch.testing.assert_close(a, b, rtol=2e-6, atol=2e-6 * a.abs().max().item())
+            else:
+                assert torch.equal(a, b)
+        if item[7]:
+            assert _abi.workspace_timeouts(item[6]) == 0
+
+
 def test_linearity_and_concatenation():
     """Size-independent properties: linear in tokens; a scan restarted from the
     state at a cut equals the uncut scan."""
