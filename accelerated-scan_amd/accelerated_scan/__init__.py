@@ -2,8 +2,8 @@
 
 Same module layout as the reference package (accelerated_scan/__init__.py:1):
 ``warp`` (fp32 / bf16 / fp16), ``scalar`` (same operator, any sequence length)
-and ``complex`` (complex64), all backed by one HIP shared library reached
-through a C ABI.
+``complex`` (complex64) and ``ref`` (the reference scan's signature, reverse
+included), all backed by one HIP shared library reached through a C ABI.
 """
 
 __version__ = "0.3.1"
