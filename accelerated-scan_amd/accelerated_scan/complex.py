@@ -81,7 +81,7 @@ class Scan(torch.autograd.Function):
         return d_forget, d_inputs
 
 
-def scan(forget, inputs, initial=None):
+def scan(forget, inputs, initial=None, reverse=False):
     """Solve ``x[t] = forget[t] * x[t-1] + inputs[t]`` over complex numbers.
 
     Arguments:
@@ -89,12 +89,15 @@ def scan(forget, inputs, initial=None):
         inputs (torch.Tensor): shape (B, C, T), complex64 or float32, contiguous.
         initial (torch.Tensor, optional): shape (B, C), complex64, the state
             ``x[-1]`` to start from (not in the reference, which starts from zero).
+        reverse (bool, optional): solve ``x[t] = forget[t] * x[t+1] + inputs[t]`` from the
+            last element down (``initial`` is then ``x[T]``); differentiable like the
+            forward scan (not in the reference).
 
     Returns:
         (torch.Tensor): complex64 states of shape (B, C, T).
     """
-    if initial is not None:
+    if initial is not None or reverse:
         if not torch.is_complex(forget):
             raise TypeError("forget must be a complex tensor")
-        return stateful.scan(forget, inputs, initial)
+        return stateful.scan(forget, inputs, initial, reverse)
     return Scan.apply(forget, inputs)

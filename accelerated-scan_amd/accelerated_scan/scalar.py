@@ -44,9 +44,11 @@ class Scan(torch.autograd.Function):
         return d_forget, d_inputs
 
 
-def scan(forget, inputs, initial=None):
+def scan(forget, inputs, initial=None, reverse=False):
     """Solve ``x[t] = forget[t] * x[t-1] + inputs[t]`` for (B, C, T) tensors of any T.
-    ``initial`` (shape (B, C), optional, not in the reference) is the state ``x[-1]``."""
-    if initial is not None:
-        return warp.scan(forget, inputs, initial)
+    ``initial`` (shape (B, C), optional, not in the reference) is the state ``x[-1]``;
+    ``reverse=True`` (not in the reference either) scans from the last element down,
+    ``x[t] = forget[t] * x[t+1] + inputs[t]`` with ``x[T] = initial``, and is differentiable too."""
+    if initial is not None or reverse:
+        return warp.scan(forget, inputs, initial, reverse)
     return Scan.apply(forget, inputs)

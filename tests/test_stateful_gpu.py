@@ -302,7 +302,17 @@ def test_bidirectional_scan_through_autograd(dtype, mode):
         got = _np32(got.detach().reshape(want.shape).cpu())
         scale = max(1.0, float(np.abs(want).max()))
         np.testing.assert_allclose(got, want, rtol=t, atol=t * scale, err_msg=f"{name} {dtype} {mode}")
-    # the keyword of warp.scan reaches the same operator
+    # the keyword of warp.scan / scalar.scan / complex.scan reaches the same operator
+    if dtype in (torch.float32, torch.bfloat16):
+        from accelerated_scan.scalar import scan as scalar_scan
+
+        assert torch.equal(scalar_scan(g, x, h, reverse=True), rev)
+        assert torch.equal(scalar_scan(g, x, reverse=True), warp_scan(g, x, reverse=True))
+    else:
+        from accelerated_scan.complex import scan as complex_scan
+
+        assert torch.equal(complex_scan(g, x, h, reverse=True), rev)
+        assert torch.equal(complex_scan(g, x, reverse=True), stateful.scan(g, x, None, reverse=True))
     if dtype in (torch.float32, torch.bfloat16):
         assert torch.equal(warp_scan(g, x, h, reverse=True), rev)
         torch.testing.assert_close(warp_scan(g, x, reverse=True).float(),
