@@ -13,10 +13,12 @@ from pathlib import Path
 
 import torch
 
-ABI_VERSION = 8
+ABI_VERSION = 9
 
 # ascan_gate codes of include/ascan.h
-GATE_IDENTITY, GATE_SIGMOID, GATE_SIGMOID_LERP, GATE_EXP = 0, 1, 2, 3
+GATE_IDENTITY, GATE_SIGMOID, GATE_SIGMOID_LERP, GATE_EXP, GATE_EXP_NORM = 0, 1, 2, 3, 4
+# gates whose second input holds values: the backward pass reads them again
+GATES_WITH_VALUES = (GATE_SIGMOID_LERP, GATE_EXP_NORM)
 
 # ascan_dtype codes of include/ascan.h
 F32, BF16, F16, C64, C64_REAL_TOKENS = 0, 1, 2, 3, 4
@@ -97,6 +99,13 @@ _SIGNATURES = {
         [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p,
          ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p,
          ctypes.c_int64, ctypes.c_int64, ctypes.c_int,
+         ctypes.c_void_p, ctypes.c_size_t, ctypes.c_void_p],
+    ),
+    "ascan_backward_gated_values": (
+        ctypes.c_int,
+        [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p,
+         ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p,
+         ctypes.c_int64, ctypes.c_int64, ctypes.c_int, ctypes.c_int,
          ctypes.c_void_p, ctypes.c_size_t, ctypes.c_void_p],
     ),
     "ascan_status_string": (ctypes.c_char_p, [ctypes.c_int]),
@@ -315,10 +324,27 @@ def backward_gated(gate_inputs, states, grad_out, d_gate_inputs, d_tokens, gate:
             gate, _ptr(workspace), workspace.numel() if workspace is not None else 0)
 
 
+def backward_gated_values(gate_inputs, values, states, grad_out, d_gate_inputs, d_values, gate: int, workspace=None,
+                          initial=None, d_initial=None) -> None:
+    """Backward of ``forward_gated`` for a gate with values (``GATE_SIGMOID_LERP``:
+    x[t] = a x[t-1] + (1 - a) values[t], a = sigmoid(gate_inputs); ``GATE_EXP_NORM``:
+    x[t] = a x[t-1] + sqrt(1 - a^2) values[t], a = exp(gate_inputs)): gradients of the gate inputs,
+    the values and the initial state."""
+    lib = _lib or load()
+    rows, seqlen, code = _problem(gate_inputs, d_values)
+    if workspace is None:
+        workspace = _workspace(rows, seqlen, code, gate_inputs.device)
+    _check_state(initial, states, "initial")
+    _check_state(d_initial, states, "d_initial")
+    _launch(gate_inputs.device, lib.ascan_backward_gated_values, gate_inputs.data_ptr(), values.data_ptr(),
+            states.data_ptr(), _ptr(initial), grad_out.data_ptr(), d_gate_inputs.data_ptr(), d_values.data_ptr(),
+            _ptr(d_initial), rows, seqlen, code, gate, _ptr(workspace),
+            workspace.numel() if workspace is not None else 0)
+
+
 def backward_lerp(gate_inputs, values, states, grad_out, d_gate_inputs, d_values, workspace=None,
                   initial=None, d_initial=None) -> None:
-    """Backward of ``forward_gated(..., GATE_SIGMOID_LERP)``: gradients of the gate inputs, the values and
-    the initial state of x[t] = a x[t-1] + (1 - a) values[t], a = sigmoid(gate_inputs)."""
+    """``backward_gated_values`` for the interpolating gate, through the library's ``ascan_backward_lerp``."""
     lib = _lib or load()
     rows, seqlen, code = _problem(gate_inputs, d_values)
     if workspace is None:

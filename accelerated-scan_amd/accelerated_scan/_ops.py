@@ -179,6 +179,25 @@ def _(gate_inputs, values, states, initial, grad_out):
     return torch.empty_like(gate_inputs), torch.empty_like(gate_inputs), torch.empty_like(initial)
 
 
+@torch.library.custom_op("accelerated_scan::scan_backward_gated_values", mutates_args=())
+def scan_backward_gated_values(
+    gate_inputs: torch.Tensor, values: torch.Tensor, states: torch.Tensor, initial: torch.Tensor,
+    grad_out: torch.Tensor, gate: int
+) -> Tuple[torch.Tensor, torch.Tensor, torch.Tensor]:
+    _check_dense(gate_inputs, (values, states, grad_out), states=(initial,))
+    d_gate_inputs = torch.empty_like(gate_inputs)
+    d_values = torch.empty_like(gate_inputs)
+    d_initial = torch.zeros_like(initial)  # stays zero for an empty sequence
+    _abi.backward_gated_values(gate_inputs, values, states, grad_out, d_gate_inputs, d_values, gate, initial=initial,
+                               d_initial=d_initial)
+    return d_gate_inputs, d_values, d_initial
+
+
+@scan_backward_gated_values.register_fake
+def _(gate_inputs, values, states, initial, grad_out, gate):
+    return torch.empty_like(gate_inputs), torch.empty_like(gate_inputs), torch.empty_like(initial)
+
+
 def _empty_token_grad(gates: torch.Tensor, real_tokens: bool) -> torch.Tensor:
     """Token gradient buffer: real when complex gates were scanned over real tokens."""
     if real_tokens and gates.is_complex():
@@ -246,7 +265,7 @@ torch.library.register_autograd(
 
 def _setup_scan_forward_gated(ctx, inputs, output):
     gate_inputs, tokens, initial, gate = inputs
-    if gate == _abi.GATE_SIGMOID_LERP:  # the second input holds values, and the backward pass reads them
+    if gate in _abi.GATES_WITH_VALUES:  # the second input holds values, and the backward pass reads them
         ctx.save_for_backward(gate_inputs, output, initial, tokens)
     else:
         ctx.save_for_backward(gate_inputs, output, initial)
@@ -254,9 +273,10 @@ def _setup_scan_forward_gated(ctx, inputs, output):
 
 
 def _backward_scan_forward_gated(ctx, grad):
-    if ctx.gate == _abi.GATE_SIGMOID_LERP:
+    if ctx.gate in _abi.GATES_WITH_VALUES:
         gate_inputs, states, initial, values = ctx.saved_tensors
-        d_gate_inputs, d_values, d_initial = scan_backward_lerp(gate_inputs, values, states, initial, grad.contiguous())
+        d_gate_inputs, d_values, d_initial = scan_backward_gated_values(gate_inputs, values, states, initial,
+                                                                        grad.contiguous(), ctx.gate)
         return d_gate_inputs, d_values, d_initial, None
     gate_inputs, states, initial = ctx.saved_tensors
     d_gate_inputs, d_tokens, d_initial = scan_backward_gated(gate_inputs, states, initial, grad.contiguous(), ctx.gate)

@@ -23,6 +23,13 @@ the same way, for layers that keep their gates as logarithms (decay rates).  In
 bfloat16 has no value between 0.99609375 and 1, while a bfloat16 logarithm
 of -0.001 carries three significant digits.
 
+``exp_norm_scan(log_gates, values)`` solves
+``x[t] = a[t] * x[t-1] + sqrt(1 - a[t]**2) * values[t]`` with ``a = exp(log_gates)``,
+the update of RG-LRU / Hawk-style layers: the input scale keeps the variance of
+the state at that of the values whatever the decay.  Gates, scales and scaled
+tokens exist in registers only, and ``1 - a**2`` is evaluated without
+cancellation for gates close to 1.
+
 The reference's ``scan`` takes finished gates (accelerated_scan/warp.py:68-83);
 the linear-RNN layers that call it (README.md:8,42 of the reference) typically
 compute them with a sigmoid just before the scan.
@@ -118,33 +125,35 @@ def exp_scan(log_gates, tokens, initial=None):
     return GatedScan.apply(log_gates, tokens, initial, _abi.GATE_EXP)
 
 
-class SigmoidLerpScan(torch.autograd.Function):
-    """Autograd node of the gated interpolation: saves (gate_logits, values, states, initial)."""
+class ValuesScan(torch.autograd.Function):
+    """Autograd node of the scans whose second input holds values (``gate``: the interpolating
+    or the normalised exponential ascan_gate code): saves (gate_inputs, values, states, initial)."""
 
     @staticmethod
-    def forward(ctx, gate_logits, values, initial):
-        _check(gate_logits, values, initial)
+    def forward(ctx, gate_inputs, values, initial, gate):
+        _check(gate_inputs, values, initial)
         initial = initial.contiguous()
         if _ops.capturing():
-            states = _ops.scan_forward_gated(gate_logits, values, initial, _abi.GATE_SIGMOID_LERP)
+            states = _ops.scan_forward_gated(gate_inputs, values, initial, gate)
         else:
-            states = torch.empty_like(gate_logits)
-            _abi.forward_gated(gate_logits, values, states, _abi.GATE_SIGMOID_LERP, initial=initial)
-        ctx.save_for_backward(gate_logits, values, states, initial)
+            states = torch.empty_like(gate_inputs)
+            _abi.forward_gated(gate_inputs, values, states, gate, initial=initial)
+        ctx.save_for_backward(gate_inputs, values, states, initial)
+        ctx.gate = gate
         return states
 
     @staticmethod
     def backward(ctx, grad_output):
-        gate_logits, values, states, initial = ctx.saved_tensors
+        gate_inputs, values, states, initial = ctx.saved_tensors
         grad_output = grad_output.contiguous()
         if _ops.capturing():
-            return _ops.scan_backward_lerp(gate_logits, values, states, initial, grad_output)
-        d_logits = torch.empty_like(gate_logits)
-        d_values = torch.empty_like(gate_logits)
+            return (*_ops.scan_backward_gated_values(gate_inputs, values, states, initial, grad_output, ctx.gate), None)
+        d_gate_inputs = torch.empty_like(gate_inputs)
+        d_values = torch.empty_like(gate_inputs)
         d_initial = torch.zeros_like(initial)  # stays zero for an empty sequence
-        _abi.backward_lerp(gate_logits, values, states, grad_output, d_logits, d_values, initial=initial,
-                           d_initial=d_initial)
-        return d_logits, d_values, d_initial
+        _abi.backward_gated_values(gate_inputs, values, states, grad_output, d_gate_inputs, d_values, ctx.gate,
+                                   initial=initial, d_initial=d_initial)
+        return d_gate_inputs, d_values, d_initial, None
 
 
 def sigmoid_lerp_scan(gate_logits, values, initial=None):
@@ -160,4 +169,21 @@ def sigmoid_lerp_scan(gate_logits, values, initial=None):
     """
     if initial is None:
         initial = torch.zeros(gate_logits.shape[:-1], dtype=gate_logits.dtype, device=gate_logits.device)
-    return SigmoidLerpScan.apply(gate_logits, values, initial)
+    return ValuesScan.apply(gate_logits, values, initial, _abi.GATE_SIGMOID_LERP)
+
+
+def exp_norm_scan(log_gates, values, initial=None):
+    """Solve ``x[t] = a[t] * x[t-1] + sqrt(1 - a[t]**2) * values[t]`` with ``a = exp(log_gates)``.
+
+    Arguments:
+        log_gates (torch.Tensor): shape (B, C, T), contiguous; fp32, bf16 or fp16; logarithms of the
+            gates, strictly negative (at 0 the input scale vanishes and its derivative is unbounded).
+        values (torch.Tensor): shape (B, C, T), contiguous, same dtype.
+        initial (torch.Tensor, optional): shape (B, C), the state ``x[-1]`` (zero if absent).
+
+    Returns:
+        (torch.Tensor): the states, shape (B, C, T); differentiable in all arguments.
+    """
+    if initial is None:
+        initial = torch.zeros(log_gates.shape[:-1], dtype=log_gates.dtype, device=log_gates.device)
+    return ValuesScan.apply(log_gates, values, initial, _abi.GATE_EXP_NORM)

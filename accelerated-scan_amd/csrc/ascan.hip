@@ -132,11 +132,13 @@ bool shape_ok(int64_t rows, int64_t seqlen) {
 
 bool activation_supported(int act, int dtype, bool reverse) {
     if (act == ASCAN_GATE_IDENTITY) return true;
-    return (act == ASCAN_GATE_SIGMOID || act == ASCAN_GATE_SIGMOID_LERP || act == ASCAN_GATE_EXP) && !reverse &&
+    return (act == ASCAN_GATE_SIGMOID || act == ASCAN_GATE_SIGMOID_LERP || act == ASCAN_GATE_EXP ||
+            act == ASCAN_GATE_EXP_NORM) && !reverse &&
            (dtype == ASCAN_F32 || dtype == ASCAN_BF16 || dtype == ASCAN_F16);
 }
 static_assert(ASCAN_GATE_IDENTITY == kGateIdentity && ASCAN_GATE_SIGMOID == kGateSigmoid &&
-                  ASCAN_GATE_SIGMOID_LERP == kGateSigmoidLerp && ASCAN_GATE_EXP == kGateExp,
+                  ASCAN_GATE_SIGMOID_LERP == kGateSigmoidLerp && ASCAN_GATE_EXP == kGateExp &&
+                  ASCAN_GATE_EXP_NORM == kGateExpNorm,
               "the kernels' gate codes are the ABI's");
 
 int forward_checked(const void* gates, const void* tokens, void* out, const void* initial, int64_t rows,
@@ -167,7 +169,7 @@ int forward_checked(const void* gates, const void* tokens, void* out, const void
     }
 }
 
-// `values` is the fourth input of the interpolating gate and null for every other gate;
+// `values` is the fourth input of the gates with values and null for every other gate;
 // `reverse` says that the scan being differentiated ran backwards in time (identity gate only).
 int backward_checked(const void* gates, const void* states, const void* grad_out, void* d_gates, void* d_tokens,
                      const void* initial, void* d_initial, const void* values, int64_t rows, int64_t seqlen,
@@ -178,7 +180,7 @@ int backward_checked(const void* gates, const void* states, const void* grad_out
     if (!shape_ok(rows, seqlen)) return ASCAN_ERR_BAD_SHAPE;
     if (rows == 0 || seqlen == 0) return ASCAN_OK;
     if (!gates || !states || !grad_out || !d_gates || !d_tokens) return ASCAN_ERR_NULL_POINTER;
-    if (act == ASCAN_GATE_SIGMOID_LERP && !values) return ASCAN_ERR_NULL_POINTER;
+    if (gate_takes_values(act) && !values) return ASCAN_ERR_NULL_POINTER;
     if (!element_aligned(gates, es) || !element_aligned(states, es) || !element_aligned(grad_out, es) ||
         !element_aligned(d_gates, es) || !element_aligned(d_tokens, token_size(dtype)) ||
         !element_aligned(initial, es) || !element_aligned(d_initial, es) || !element_aligned(values, es))
@@ -300,7 +302,7 @@ int ascan_forward_gated(const void* gate_inputs, const void* tokens, const void*
 int ascan_backward_gated(const void* gate_inputs, const void* states, const void* initial, const void* grad_out,
                          void* d_gate_inputs, void* d_tokens, void* d_initial, int64_t rows, int64_t seqlen,
                          int dtype, int gate, void* workspace, size_t workspace_bytes, void* stream) {
-    if (gate == ASCAN_GATE_SIGMOID_LERP) return ASCAN_ERR_BAD_ACTIVATION;  // needs the values: ascan_backward_lerp
+    if (gate_takes_values(gate)) return ASCAN_ERR_BAD_ACTIVATION;  // needs the values: ascan_backward_gated_values
     return backward_checked(gate_inputs, states, grad_out, d_gate_inputs, d_tokens, initial, d_initial, nullptr, rows,
                             seqlen, dtype, gate, false, Workspace{workspace, workspace_bytes}, stream);
 }
@@ -310,6 +312,15 @@ int ascan_backward_lerp(const void* gate_inputs, const void* values, const void*
                         int64_t seqlen, int dtype, void* workspace, size_t workspace_bytes, void* stream) {
     return backward_checked(gate_inputs, states, grad_out, d_gate_inputs, d_values, initial, d_initial, values, rows,
                             seqlen, dtype, ASCAN_GATE_SIGMOID_LERP, false, Workspace{workspace, workspace_bytes}, stream);
+}
+
+int ascan_backward_gated_values(const void* gate_inputs, const void* values, const void* states, const void* initial,
+                                const void* grad_out, void* d_gate_inputs, void* d_values, void* d_initial,
+                                int64_t rows, int64_t seqlen, int dtype, int gate, void* workspace,
+                                size_t workspace_bytes, void* stream) {
+    if (!gate_takes_values(gate)) return ASCAN_ERR_BAD_ACTIVATION;
+    return backward_checked(gate_inputs, states, grad_out, d_gate_inputs, d_values, initial, d_initial, values, rows,
+                            seqlen, dtype, gate, false, Workspace{workspace, workspace_bytes}, stream);
 }
 
 unsigned int ascan_workspace_timeouts(const void* workspace_header_copy) {

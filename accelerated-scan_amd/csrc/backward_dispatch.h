@@ -17,7 +17,7 @@ struct BackwardBuffers {
     void* d_tokens;
     const void* initial;
     void* d_initial;
-    const void* values;  // the interpolating gate's fourth input, else null
+    const void* values;  // the fourth input of a gate with values, else null
 };
 
 // REV is the backward kernel's own direction: true for the backward pass of a forward-time scan.
@@ -81,7 +81,7 @@ int backward_typed(const BackwardBuffers& b, int64_t rows, int64_t T, int act, c
     const int lead = at.lead;
     // the interpolating gate's kernels (half-size tiles, a fourth input, more arithmetic per element) gain from a
     // narrower plan for a mostly empty last tile whatever the dtype: fp32 (8,1536,9000) backward 4.9 -> 5.5 TB/s
-    const bool trim = kTrimPlan<Tr> || act == kGateSigmoidLerp;
+    const bool trim = kTrimPlan<Tr> || gate_takes_values(act);
     Plan plan = choose_plan(T, SUB, kElem, trim);
     const Access access = choose_access(same_lead, lead, T, SUB * plan.waves_per_row);
     if (access != Access::kRegular) plan = choose_plan(T, SUBG, kElem, trim);

@@ -25,7 +25,9 @@ namespace {
 // "before" are meant in the order of the scan being differentiated.
 // With the interpolating gate (x[t] = a x[t-1] + (1 - a) v[t], a = sigmoid(z))
 // the kernel also reads the values v and writes, for the same g,
-// d_v[t] = g[t] (1 - a[t]) and d_z[t] = g[t] (x[t-1] - v[t]) a[t] (1 - a[t]).
+// d_v[t] = g[t] (1 - a[t]) and d_z[t] = g[t] (x[t-1] - v[t]) a[t] (1 - a[t]); with the
+// normalised exponential gate (x[t] = a x[t-1] + b v[t], a = exp(z), b = sqrt(1 - a^2))
+// d_v[t] = g[t] b[t] and d_z[t] = g[t] (a[t] x[t-1] - v[t] a[t]^2 / b[t]).
 // ---------------------------------------------------------------------------
 template <class Tr, int W, int U, bool REV, bool ALIGNED, bool REGULAR, bool SPLIT, int ACT, bool PACKED>
 __global__ void __launch_bounds__(64 * kMaxWavesPerBlock)
@@ -41,7 +43,7 @@ __global__ void __launch_bounds__(64 * kMaxWavesPerBlock)
     constexpr int64_t TILE = SUB * W;
     static_assert(!PACKED || (!SPLIT && !REGULAR), "packed rows use the general kernels, one group per workgroup");
     static_assert(REV || ACT == kGateIdentity, "the gated scans run forward in time only");
-    constexpr bool LERP = ACT == kGateSigmoidLerp;  // `values` is a fourth input
+    constexpr bool LERP = kGateTakesValues<ACT>;  // `values` is a fourth input
     // index, inside a vector, of the element the gradient scan reaches first / last
     constexpr int E_FIRST = REV ? Tr::EPV - 1 : 0;
     constexpr int E_LAST = REV ? 0 : Tr::EPV - 1;
@@ -349,10 +351,14 @@ __global__ void __launch_bounds__(64 * kMaxWavesPerBlock)
                 const int e = REV ? EPV - 1 - i : i;
                 gr = carry_in<PACKED>(vconj(after[e]), gr, d[e]);
                 if constexpr (PACKED) gs[e] = gr;
-                if constexpr (LERP) {
+                if constexpr (ACT == kGateSigmoidLerp) {
                     // token = (1 - a) v:  d_v = g (1 - a);  d_a = g (x[t-1] - v);  d_z = d_a a (1 - a)
                     dt[e] = gr * a_rest[e];
                     dg[e] = (gr * (before[e] - v[e])) * (a[e] * a_rest[e]);
+                } else if constexpr (ACT == kGateExpNorm) {
+                    // token = b v, b = sqrt(1 - a^2):  d_v = g b;  d_z = g (a x[t-1] + v db/dz),  db/dz = -a^2 / b
+                    dt[e] = gr * a_rest[e];
+                    dg[e] = gr * (a[e] * (before[e] - v[e] * (a[e] * __builtin_amdgcn_rcpf(a_rest[e]))));
                 } else {
                     dt[e] = gr;
                     dg[e] = vmul(gr, vconj(before[e]));

@@ -38,7 +38,7 @@ struct BackwardCall {
     void* d_tokens;
     const void* initial;  // or null
     void* d_initial;      // or null
-    const void* values;   // the interpolating gate's values v (then d_tokens receives d_v), else null
+    const void* values;   // values v of a gate with values (then d_tokens receives d_v), else null
     int64_t rows, seqlen;
     int gate;
     Workspace workspace;

@@ -26,7 +26,7 @@ hipError_t launch_forward_split(const void* gates, const void* tokens, void* out
                                 int64_t T, int grid, int64_t ntiles, const Workspace& ws, hipStream_t stream) {
     using S = typename Tr::S;
     using TokS = typename Tr::TokS;
-    constexpr int U = REGULAR ? SplitTuning<Tr>::U : SplitTuning<Tr>::UG;
+    constexpr int U = forward_split_blocks<ACT>(REGULAR ? SplitTuning<Tr>::U : SplitTuning<Tr>::UG);
     auto kernel = scan_forward_kernel<Tr, kSplitWaves, U, REV, true, REGULAR, true, ACT, false>;
     const unsigned resident = resident_workgroups(kernel, 64 * kSplitWaves);
     if (resident == 0) return hipErrorInvalidConfiguration;
@@ -73,13 +73,16 @@ int forward_typed(const void* gates, const void* tokens, void* out, const void* 
     constexpr int64_t kElem = (int64_t)sizeof(typename Tr::S);
     constexpr int64_t SUB = (int64_t)Tuning<Tr>::U * 64 * Tr::EPV;    // regular kernels
     constexpr int64_t SUBG = (int64_t)Tuning<Tr>::UG * 64 * Tr::EPV;  // kernels with masking code
-    Plan plan = choose_plan(T, SUB, kElem, kTrimPlan<Tr>);
+    // gates that form the token from values as well do more arithmetic per byte and, like the 16-bit kernels,
+    // gain from a narrower plan when the last tile step would be mostly empty
+    const bool trim = kTrimPlan<Tr> || gate_takes_values(act);
+    Plan plan = choose_plan(T, SUB, kElem, trim);
     const void* const state_like[] = {gates, out};
     const Lead at = find_lead<Tr>(state_like, tokens);
     const bool same_lead = at.same;
     const int lead = at.lead;
     const Access access = choose_access(same_lead, lead, T, SUB * plan.waves_per_row);
-    if (access != Access::kRegular) plan = choose_plan(T, SUBG, kElem, kTrimPlan<Tr>);
+    if (access != Access::kRegular) plan = choose_plan(T, SUBG, kElem, trim);
     const int R = plan.rows_per_block;
     hipError_t err = hipSuccess;
     // Gated kernels run forward in time only (validated by the entry points); REV below is a
@@ -93,8 +96,8 @@ int forward_typed(const void* gates, const void* tokens, void* out, const void* 
         return launch_status(err);
     }
     if (same_lead && ws.ptr != nullptr) {
-        constexpr int64_t SUBS = (int64_t)SplitTuning<Tr>::U * 64 * Tr::EPV;
-        constexpr int64_t SUBSG = (int64_t)SplitTuning<Tr>::UG * 64 * Tr::EPV;
+        const int64_t SUBS = (int64_t)forward_split_blocks_of(act, SplitTuning<Tr>::U) * 64 * Tr::EPV;
+        const int64_t SUBSG = (int64_t)forward_split_blocks_of(act, SplitTuning<Tr>::UG) * 64 * Tr::EPV;
         const bool regular = lead == 0 && T % (SUBS * kSplitWaves) == 0;
         const int64_t ntiles = host_tiles_per_row<Tr>(T, (regular ? SUBS : SUBSG) * kSplitWaves, regular, at);
         if (want_split(rows, ntiles) && workspace_fits(ws, rows, ntiles)) {

@@ -22,9 +22,19 @@ namespace {
 //   kGateExp        : gate = exp(stored), real dtypes only: gates kept as
 //                     logarithms (decay rates).  A 16-bit logarithm carries a
 //                     gate close to 1 far more precisely than a 16-bit gate
-//                     does (bf16 has no value between 0.996 and 1).
+//                     does (bf16 has no value between 0.996 and 1);
+//   kGateExpNorm    : gate = exp(stored), and the token is sqrt(1 - gate^2) * stored
+//                     value: x[t] = a x[t-1] + sqrt(1 - a^2) v[t], the update of
+//                     RG-LRU / Hawk-style layers, whose input scale keeps the
+//                     state's variance at that of the values.
 // ---------------------------------------------------------------------------
-constexpr int kGateIdentity = 0, kGateSigmoid = 1, kGateSigmoidLerp = 2, kGateExp = 3;
+constexpr int kGateIdentity = 0, kGateSigmoid = 1, kGateSigmoidLerp = 2, kGateExp = 3, kGateExpNorm = 4;
+
+// Gates whose second input holds values v rather than tokens: the token is
+// formed in registers from v and the gate, and the backward pass reads v again.
+template <int ACT>
+constexpr bool kGateTakesValues = ACT == kGateSigmoidLerp || ACT == kGateExpNorm;
+inline bool gate_takes_values(int act) { return act == kGateSigmoidLerp || act == kGateExpNorm; }
 
 template <int ACT>
 constexpr bool kGateIsSigmoid = ACT == kGateSigmoid || ACT == kGateSigmoidLerp;
@@ -51,9 +61,27 @@ __device__ __forceinline__ void sigmoid_pair(float v, float& gate, float& comple
     complement = positive ? small : large;
 }
 
+// exp(v) and sqrt(1 - exp(2 v)) for v <= 0 (0 for v > 0).  1 - exp(w), w = 2 v, loses
+// its leading digits to cancellation as w approaches 0, where the gates of long
+// memories live; for w > -1/16 it is summed as -w (1 + w/2 (1 + w/3 (1 + w/4 (1 + w/5))))
+// instead (truncation below 2e-9 relative; the difference 1 - a^2 is good to 1e-6 relative
+// below that), so the scale keeps fp32 accuracy for every gate.  v = 0, the
+// out-of-row fill, gives exactly (1, 0).
+__device__ __forceinline__ void exp_norm_pair(float v, float& gate, float& scale) {
+    gate = exp_gate(v);
+    const float w = v + v;
+    float series = __builtin_fmaf(w, 0.2f, 1.0f);
+    series = __builtin_fmaf(w * 0.25f, series, 1.0f);
+    series = __builtin_fmaf(w * (1.0f / 3.0f), series, 1.0f);
+    series = __builtin_fmaf(w * 0.5f, series, 1.0f);
+    const float direct = __builtin_fmaf(-gate, gate, 1.0f);
+    const float m = w > -0.0625f ? -w * series : direct;
+    scale = __builtin_amdgcn_sqrtf(__builtin_fmaxf(m, 0.0f));
+}
+
 template <int ACT, class V, int N>
 __device__ __forceinline__ void activate(V (&g)[N]) {
-    static_assert(ACT != kGateSigmoidLerp, "the interpolating gate goes through activate_pair / activate_with_complement");
+    static_assert(!kGateTakesValues<ACT>, "gates with values go through activate_pair / activate_with_complement");
     if constexpr (ACT == kGateSigmoid) {
 #pragma unroll
         for (int e = 0; e < N; ++e) g[e] = sigmoid(g[e]);
@@ -75,11 +103,20 @@ __device__ __forceinline__ void activate_pair(V (&g)[N], V (&t)[N]) {
             g[e] = gate;
             t[e] = complement * t[e];
         }
+    } else if constexpr (ACT == kGateExpNorm) {
+#pragma unroll
+        for (int e = 0; e < N; ++e) {
+            float gate, scale;
+            exp_norm_pair(g[e], gate, scale);
+            g[e] = gate;
+            t[e] = scale * t[e];
+        }
     } else {
         activate<ACT>(g);
     }
 }
-// Gates and their complements 1 - gate (the interpolating gate's backward pass).
+// Gates and the factor their values are weighted by -- 1 - gate for the interpolating
+// gate, sqrt(1 - gate^2) for the normalised exponential one (the backward pass of both).
 template <int ACT, class V, int N>
 __device__ __forceinline__ void activate_with_complement(V (&g)[N], V (&c)[N]) {
     if constexpr (ACT == kGateSigmoidLerp) {
@@ -89,6 +126,14 @@ __device__ __forceinline__ void activate_with_complement(V (&g)[N], V (&c)[N]) {
             sigmoid_pair(g[e], gate, complement);
             g[e] = gate;
             c[e] = complement;
+        }
+    } else if constexpr (ACT == kGateExpNorm) {
+#pragma unroll
+        for (int e = 0; e < N; ++e) {
+            float gate, scale;
+            exp_norm_pair(g[e], gate, scale);
+            g[e] = gate;
+            c[e] = scale;
         }
     } else {
         activate<ACT>(g);
@@ -102,7 +147,7 @@ __device__ __forceinline__ V activate1(V g) {
         float gate, complement;
         sigmoid_pair(g, gate, complement);
         return gate;
-    } else if constexpr (ACT == kGateExp) {
+    } else if constexpr (ACT == kGateExp || ACT == kGateExpNorm) {
         return exp_gate(g);
     } else {
         return g;
@@ -113,7 +158,7 @@ template <int ACT, class V>
 __device__ __forceinline__ V identity_gate() {
     if constexpr (kGateIsSigmoid<ACT>) {
         return __builtin_inff();
-    } else if constexpr (ACT == kGateExp) {
+    } else if constexpr (ACT == kGateExp || ACT == kGateExpNorm) {
         return vzero<V>();
     } else {
         return vone<V>();

@@ -323,17 +323,26 @@ hipError_t with_gate(int act, F&& f) {
         if (act == kGateSigmoid) return f(std::integral_constant<int, kGateSigmoid>{});
         if (act == kGateSigmoidLerp) return f(std::integral_constant<int, kGateSigmoidLerp>{});
         if (act == kGateExp) return f(std::integral_constant<int, kGateExp>{});
+        if (act == kGateExpNorm) return f(std::integral_constant<int, kGateExpNorm>{});
     }
     return f(std::integral_constant<int, kGateIdentity>{});
 }
 
-// The backward kernel of the interpolating gate holds a fourth input tensor in
+// The backward kernel of a gate with values holds a fourth input tensor in
 // registers and takes 2 KiB per wave and tile at most.
 template <int ACT>
 constexpr int backward_blocks(int blocks) {
-    return ACT == kGateSigmoidLerp && blocks > 2 ? 2 : blocks;
+    return kGateTakesValues<ACT> && blocks > 2 ? 2 : blocks;
 }
-inline int backward_blocks_of(int act, int blocks) { return act == kGateSigmoidLerp && blocks > 2 ? 2 : blocks; }
+inline int backward_blocks_of(int act, int blocks) { return gate_takes_values(act) && blocks > 2 ? 2 : blocks; }
+
+// The split-row forward kernel of the normalised exponential gate (two activations
+// per element next to the look-back's registers) takes 2 KiB per wave and tile as well.
+template <int ACT>
+constexpr int forward_split_blocks(int blocks) {
+    return ACT == kGateExpNorm && blocks > 2 ? 2 : blocks;
+}
+inline int forward_split_blocks_of(int act, int blocks) { return act == kGateExpNorm && blocks > 2 ? 2 : blocks; }
 
 }  // namespace
 }  // namespace ascan

@@ -62,7 +62,7 @@
 extern "C" {
 #endif
 
-#define ASCAN_ABI_VERSION 8
+#define ASCAN_ABI_VERSION 9
 
 /* Marks the exported entry points (the library is built with hidden visibility). */
 #define ASCAN_API __attribute__((visibility("default")))
@@ -113,7 +113,17 @@ enum ascan_gate {
      * to 1 far more precisely than a 16-bit gate can (bfloat16 has no value
      * between 0.99609375 and 1).  float32, bfloat16, float16.
      */
-    ASCAN_GATE_EXP = 3
+    ASCAN_GATE_EXP = 3,
+    /*
+     * The same gate, and the second input holds values v rather than tokens:
+     * token = sqrt(1 - gate^2) * v, i.e. x[t] = a * x[t-1] + sqrt(1 - a^2) * v[t]
+     * with a = exp(stored), the update of RG-LRU / Hawk-style layers (the scale
+     * keeps the state's variance at that of the values).  Stored values must be
+     * negative: at 0 the scale is 0 and its derivative unbounded.  Forward:
+     * ascan_forward_gated; backward: ascan_backward_gated_values (it needs v).
+     * float32, bfloat16, float16.
+     */
+    ASCAN_GATE_EXP_NORM = 4
 };
 
 /*
@@ -271,8 +281,8 @@ ASCAN_API int ascan_backward_reverse(const void* gates, const void* states, cons
  * with g, d_tokens and d_initial as in ascan_backward_from.  No counterpart in
  * the reference.  gate = ASCAN_GATE_IDENTITY makes these calls the *_from ones
  * (forward in time only); the sigmoid and exponential gates need a real dtype, else
- * ASCAN_ERR_BAD_ACTIVATION (as does ASCAN_GATE_SIGMOID_LERP in
- * ascan_backward_gated, which lacks the values: see ascan_backward_lerp).  The sigmoid is evaluated in fp32 with the
+ * ASCAN_ERR_BAD_ACTIVATION (as do ASCAN_GATE_SIGMOID_LERP and ASCAN_GATE_EXP_NORM in
+ * ascan_backward_gated, which lacks the values: see ascan_backward_gated_values).  The sigmoid is evaluated in fp32 with the
  * hardware's exp2 and reciprocal (about 2 ulp), the exponential with exp2 (1 ulp
  * of the result for arguments of moderate size).
  */
@@ -304,6 +314,28 @@ ASCAN_API int ascan_backward_lerp(const void* gate_inputs, const void* values, c
                         const void* grad_out, void* d_gate_inputs, void* d_values, void* d_initial,
                         int64_t rows, int64_t seqlen, int dtype,
                         void* workspace, size_t workspace_bytes, void* stream);
+
+/*
+ * Backward pass of ascan_forward_gated for the gates whose second input holds
+ * values: gate = ASCAN_GATE_SIGMOID_LERP is ascan_backward_lerp, and
+ * gate = ASCAN_GATE_EXP_NORM differentiates
+ *
+ *     a[t] = exp(gate_inputs[t]),   b[t] = sqrt(1 - a[t]^2)
+ *     forward          : x[t] = a[t] * x[t-1] + b[t] * values[t],   x[-1] = initial (NULL: 0)
+ *     g[t]             = grad_out[t] + a[t+1] * g[t+1]
+ *     d_values[t]      = g[t] * b[t]
+ *     d_gate_inputs[t] = g[t] * (a[t] * x[t-1] - values[t] * a[t]^2 / b[t])
+ *     d_initial        = a[0] * g[0]
+ *
+ * in one fused reverse-time pass (4 tensors read, 2 written).  1 - a^2 is
+ * evaluated without cancellation for gates close to 1 (a series in
+ * 2 * gate_inputs above -0.25).  Any other gate: ASCAN_ERR_BAD_ACTIVATION.
+ * No counterpart in the reference.
+ */
+ASCAN_API int ascan_backward_gated_values(const void* gate_inputs, const void* values, const void* states,
+                                const void* initial, const void* grad_out, void* d_gate_inputs, void* d_values,
+                                void* d_initial, int64_t rows, int64_t seqlen, int dtype, int gate,
+                                void* workspace, size_t workspace_bytes, void* stream);
 
 /* Static, human-readable text for an ascan_status code. */
 ASCAN_API const char* ascan_status_string(int status);

@@ -358,3 +358,55 @@ void seq_backward_lerp_f32(const float* z, const float* v, const float* state, c
         if (dinit) dinit[r] = (T > 0) ? sigmoid64((double)zr[0]) * g : 0.0;
     }
 }
+
+/*
+ * Exponential gate with a variance-preserving input scale (no counterpart in
+ * the reference; the update of RG-LRU / Hawk-style layers): the gate is the
+ * exponential of a stored logarithm z <= 0 and the token the stored value
+ * times sqrt(1 - gate^2),
+ *   a[t] = exp(z[t]),  b[t] = sqrt(1 - a[t]^2),  out[t] = a[t] * out[t-1] + b[t] * v[t],  out[-1] = init
+ *   g[t] = dout[t] + a[t+1] * g[t+1]
+ *   dv[t] = g[t] * b[t],  dz[t] = g[t] * (a[t] * state[t-1] - v[t] * a[t]^2 / b[t]),  dinit = a[0] * g[0]
+ * 1 - a^2 is taken as -expm1(2 z), which keeps its relative accuracy for z
+ * close to 0 (clamped at 0 for z > 0).  Pinned by tests/test_oracle.py: torch
+ * autograd through the plain float64 loop with torch.exp, torch.expm1 and
+ * torch.sqrt, the exponential-gate functions above on tokens b * v formed in
+ * float64 plus the chain rule, and closed forms (a = 0.6 gives b = 0.8; a
+ * constant value c tends to c * sqrt((1 + a) / (1 - a)); z = -800 returns the values).
+ */
+static double expnorm_scale(double z) {
+    const double m = -expm1(2.0 * z);
+    return m > 0.0 ? sqrt(m) : 0.0;
+}
+
+void seq_forward_expnorm_f32(const float* z, const float* v, const float* init, double* out, int64_t rows, int64_t T) {
+#pragma omp parallel for schedule(static)
+    for (int64_t r = 0; r < rows; ++r) {
+        double s = init ? (double)init[r] : 0.0;
+        for (int64_t t = 0; t < T; ++t) {
+            const double zt = (double)z[r * T + t];
+            s = exp(zt) * s + expnorm_scale(zt) * (double)v[r * T + t];
+            out[r * T + t] = s;
+        }
+    }
+}
+
+void seq_backward_expnorm_f32(const float* z, const float* v, const float* state, const float* init, const float* dout,
+                              double* dz, double* dv, double* dinit, int64_t rows, int64_t T) {
+#pragma omp parallel for schedule(static)
+    for (int64_t r = 0; r < rows; ++r) {
+        const float* zr = z + r * T;
+        const float* vr = v + r * T;
+        const float* sr = state + r * T;
+        const double x0 = init ? (double)init[r] : 0.0;
+        double g = 0.0;
+        for (int64_t t = T - 1; t >= 0; --t) {
+            const double gnext = (t + 1 < T) ? exp((double)zr[t + 1]) : 1.0;
+            g = (double)dout[r * T + t] + gnext * g;
+            const double a = exp((double)zr[t]), b = expnorm_scale((double)zr[t]);
+            dv[r * T + t] = g * b;
+            dz[r * T + t] = g * (a * ((t > 0) ? (double)sr[t - 1] : x0) - (double)vr[t] * a * a / b);
+        }
+        if (dinit) dinit[r] = (T > 0) ? exp((double)zr[0]) * g : 0.0;
+    }
+}

@@ -43,11 +43,13 @@ def _load():
         lib.seq_backward_sigmoid_f32.argtypes = [p, p, p, p, p, p, p, i64, i64]
         lib.seq_forward_lerp_f32.argtypes = [p, p, p, p, i64, i64]
         lib.seq_backward_lerp_f32.argtypes = [p, p, p, p, p, p, p, p, i64, i64]
+        lib.seq_forward_expnorm_f32.argtypes = [p, p, p, p, i64, i64]
+        lib.seq_backward_expnorm_f32.argtypes = [p, p, p, p, p, p, p, p, i64, i64]
         for f in (lib.seq_forward_f32, lib.seq_forward_c64, lib.seq_backward_f32, lib.seq_backward_c64,
                   lib.seq_forward_from_f32, lib.seq_forward_from_c64, lib.seq_backward_from_f32,
                   lib.seq_backward_from_c64, lib.seq_forward_sigmoid_f32, lib.seq_backward_sigmoid_f32,
                   lib.seq_forward_lerp_f32, lib.seq_backward_lerp_f32, lib.seq_forward_exp_f32,
-                  lib.seq_backward_exp_f32):
+                  lib.seq_backward_exp_f32, lib.seq_forward_expnorm_f32, lib.seq_backward_expnorm_f32):
             f.restype = None
         _lib = lib
     return _lib
@@ -196,11 +198,9 @@ def backward_exp(log_gates, states, grad_out, initial=None):
     return _backward_gated("seq_backward_exp_f32", log_gates, states, grad_out, initial)
 
 
-def forward_lerp(gate_logits, values, initial=None):
-    """Sequential gated interpolation in fp64:
-    x[t] = a[t] * x[t-1] + (1 - a[t]) * values[t], a = sigmoid(gate_logits) (real inputs)."""
+def _forward_values(name, gate_inputs, values, initial):
     lib = _load()
-    z, zp = _prep(gate_logits, np.float32)
+    z, zp = _prep(gate_inputs, np.float32)
     v, vp = _prep(values, np.float32)
     assert z.shape == v.shape
     ip = None
@@ -210,14 +210,13 @@ def forward_lerp(gate_logits, values, initial=None):
     T = z.shape[-1]
     rows = z.size // T if T else 0
     out = np.empty(z.shape, dtype=np.float64)
-    lib.seq_forward_lerp_f32(zp, vp, ip, out.ctypes.data_as(ctypes.c_void_p), rows, T)
+    getattr(lib, name)(zp, vp, ip, out.ctypes.data_as(ctypes.c_void_p), rows, T)
     return out
 
 
-def backward_lerp(gate_logits, values, states, grad_out, initial=None):
-    """(d_gate_logits, d_values, d_initial) of the gated interpolation, in fp64."""
+def _backward_values(name, gate_inputs, values, states, grad_out, initial):
     lib = _load()
-    z, zp = _prep(gate_logits, np.float32)
+    z, zp = _prep(gate_inputs, np.float32)
     v, vp = _prep(values, np.float32)
     s, sp = _prep(states, np.float32)
     d, dp = _prep(grad_out, np.float32)
@@ -232,6 +231,28 @@ def backward_lerp(gate_logits, values, states, grad_out, initial=None):
     dv = np.empty(z.shape, dtype=np.float64)
     di = np.zeros(z.shape[:-1], dtype=np.float64)
     if rows:
-        lib.seq_backward_lerp_f32(zp, vp, sp, ip, dp, dz.ctypes.data_as(ctypes.c_void_p),
-                                  dv.ctypes.data_as(ctypes.c_void_p), di.ctypes.data_as(ctypes.c_void_p), rows, T)
+        getattr(lib, name)(zp, vp, sp, ip, dp, dz.ctypes.data_as(ctypes.c_void_p), dv.ctypes.data_as(ctypes.c_void_p),
+                           di.ctypes.data_as(ctypes.c_void_p), rows, T)
     return dz, dv, di
+
+
+def forward_lerp(gate_logits, values, initial=None):
+    """Sequential gated interpolation in fp64:
+    x[t] = a[t] * x[t-1] + (1 - a[t]) * values[t], a = sigmoid(gate_logits) (real inputs)."""
+    return _forward_values("seq_forward_lerp_f32", gate_logits, values, initial)
+
+
+def backward_lerp(gate_logits, values, states, grad_out, initial=None):
+    """(d_gate_logits, d_values, d_initial) of the gated interpolation, in fp64."""
+    return _backward_values("seq_backward_lerp_f32", gate_logits, values, states, grad_out, initial)
+
+
+def forward_expnorm(log_gates, values, initial=None):
+    """Sequential scan in fp64 with an exponential gate and the input scale that goes with it:
+    x[t] = a[t] * x[t-1] + sqrt(1 - a[t]^2) * values[t], a = exp(log_gates) (real inputs, log_gates <= 0)."""
+    return _forward_values("seq_forward_expnorm_f32", log_gates, values, initial)
+
+
+def backward_expnorm(log_gates, values, states, grad_out, initial=None):
+    """(d_log_gates, d_values, d_initial) of that scan, in fp64."""
+    return _backward_values("seq_backward_expnorm_f32", log_gates, values, states, grad_out, initial)

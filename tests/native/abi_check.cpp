@@ -27,6 +27,9 @@ void seq_backward_exp_f32(const float* z, const float* state, const float* init,
 void seq_forward_lerp_f32(const float* z, const float* v, const float* init, double* out, int64_t rows, int64_t T);
 void seq_backward_lerp_f32(const float* z, const float* v, const float* state, const float* init, const float* dout,
                            double* dz, double* dv, double* dinit, int64_t rows, int64_t T);
+void seq_forward_expnorm_f32(const float* z, const float* v, const float* init, double* out, int64_t rows, int64_t T);
+void seq_backward_expnorm_f32(const float* z, const float* v, const float* state, const float* init, const float* dout,
+                           double* dz, double* dv, double* dinit, int64_t rows, int64_t T);
 }
 
 #define HIP_OK(call)                                                                          \
@@ -169,7 +172,7 @@ void check_problem(int64_t rows, int64_t T, bool with_initial, hipStream_t strea
     }
 }
 
-// The gated entry points (sigmoid gate; sigmoid gate with interpolated values) and the
+// The gated entry points (sigmoid gate; sigmoid gate with interpolated values; exponential gates) and the
 // split-row forward scan whose table is the library's static array.
 void check_gated_and_static(int64_t rows, int64_t T, hipStream_t stream) {
     std::printf("gated rows=%lld T=%lld\n", (long long)rows, (long long)T);
@@ -239,6 +242,25 @@ void check_gated_and_static(int64_t rows, int64_t T, hipStream_t stream) {
         EXPECT(worst(download(d_init, rows, stream), t_di) <= tol);
     }
 
+    // exponential gate with the input scale sqrt(1 - gate^2): logarithms strictly below zero
+    {
+        std::vector<float> logs(n);
+        for (size_t i = 0; i < n; ++i) logs[i] = -0.25f * std::fabs(z[i]) - 1e-3f;
+        upload(dz_in, logs, stream);
+        EXPECT(ascan_forward_gated(dz_in.p, dx_in.p, dinit_in.p, out.p, rows, T, ASCAN_F32, ASCAN_GATE_EXP_NORM, ws_ptr,
+                                   ws_bytes, stream) == ASCAN_OK);
+        EXPECT(ascan_backward_gated_values(dz_in.p, dx_in.p, out.p, dinit_in.p, dd_in.p, d_z.p, d_x.p, d_init.p, rows, T,
+                                           ASCAN_F32, ASCAN_GATE_EXP_NORM, ws_ptr, ws_bytes, stream) == ASCAN_OK);
+        h_out = download(out, n, stream);
+        seq_forward_expnorm_f32(logs.data(), x.data(), init.data(), t_out.data(), rows, T);
+        seq_backward_expnorm_f32(logs.data(), x.data(), h_out.data(), init.data(), d.data(), t_dz.data(), t_dx.data(),
+                                 t_di.data(), rows, T);
+        EXPECT(worst(h_out, t_out) <= tol);
+        EXPECT(worst(download(d_z, n, stream), t_dz) <= tol);
+        EXPECT(worst(download(d_x, n, stream), t_dx) <= tol);
+        EXPECT(worst(download(d_init, rows, stream), t_di) <= tol);
+    }
+
     // static-table forward scan: stored values in [0, 1) as gates (x from a zero state)
     std::vector<float> g(n);
     for (size_t i = 0; i < n; ++i) g[i] = rng.uniform();
@@ -280,6 +302,13 @@ void check_status_codes(hipStream_t stream) {
                                 ASCAN_GATE_SIGMOID_LERP, nullptr, 0, stream) == ASCAN_ERR_BAD_ACTIVATION);
     EXPECT(ascan_backward_lerp(a.p, nullptr, b.p, nullptr, c.p, (char*)a.p + 1024, (char*)a.p + 2048, nullptr, 1, 16,
                                ASCAN_F32, nullptr, 0, stream) == ASCAN_ERR_NULL_POINTER);
+    EXPECT(ascan_backward_gated(a.p, b.p, nullptr, c.p, (char*)a.p + 1024, (char*)a.p + 2048, nullptr, 1, 16, ASCAN_F32,
+                                ASCAN_GATE_EXP_NORM, nullptr, 0, stream) == ASCAN_ERR_BAD_ACTIVATION);
+    EXPECT(ascan_backward_gated_values(a.p, (char*)a.p + 3072, b.p, nullptr, c.p, (char*)a.p + 1024, (char*)a.p + 2048,
+                                       nullptr, 1, 16, ASCAN_F32, ASCAN_GATE_EXP, nullptr, 0, stream) ==
+           ASCAN_ERR_BAD_ACTIVATION);
+    EXPECT(ascan_backward_gated_values(a.p, nullptr, b.p, nullptr, c.p, (char*)a.p + 1024, (char*)a.p + 2048, nullptr, 1,
+                                       16, ASCAN_F32, ASCAN_GATE_EXP_NORM, nullptr, 0, stream) == ASCAN_ERR_NULL_POINTER);
     // the static-table entry point refuses what does not fit its array
     EXPECT(ascan_forward_split_static(a.p, b.p, c.p, 128, 1 << 24, ASCAN_F32, 0, stream) == ASCAN_ERR_TOO_LARGE);
 }

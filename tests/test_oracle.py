@@ -475,3 +475,80 @@ def test_lerp_vs_sigmoid_scan_of_formed_tokens_and_closed_forms():
     np.testing.assert_allclose(seqscan.forward_lerp(np.full_like(x, -40.0), x), x, rtol=1e-12, atol=1e-12)
     np.testing.assert_allclose(seqscan.forward_lerp(np.full_like(x, 40.0), x, np.full((1, 1), 0.5, np.float32)), 0.5,
                                rtol=1e-12, atol=1e-12)
+
+
+# ---------------------------------------------------------------------------
+# Exponential gate with the input scale sqrt(1 - a^2): x[t] = a x[t-1] + sqrt(1 - a^2) v[t], a = exp(z)
+# (oracle functions *_expnorm)
+# ---------------------------------------------------------------------------
+@pytest.mark.parametrize("T", [1, 2, 9, 64])
+@pytest.mark.parametrize("with_initial", [False, True])
+def test_expnorm_vs_autograd_of_loop(T, with_initial):
+    """Values and all three gradients against torch autograd through the explicit
+    float64 loop written with torch.exp, torch.expm1 and torch.sqrt."""
+    gen = torch.Generator().manual_seed(1300 + T)
+    log_gates = -torch.rand(2, 2, T, generator=gen).mul(6.0).exp().mul(1e-3)  # -1e-3 ... -0.4: gates 0.67 ... 0.999
+    values, grad_out = (torch.randn(2, 2, T, generator=gen) for _ in range(2))
+    initial = torch.randn(2, 2, generator=gen) if with_initial else torch.zeros(2, 2)
+    zw, vw, iw = (t.double().requires_grad_(True) for t in (log_gates, values, initial))
+    a = torch.exp(zw)
+    b = torch.sqrt(-torch.expm1(2 * zw))
+    state, outs = iw, []
+    for t in range(T):
+        state = a[..., t] * state + b[..., t] * vw[..., t]
+        outs.append(state)
+    out = torch.stack(outs, dim=-1)
+    dz_ref, dv_ref, di_ref = torch.autograd.grad(out, (zw, vw, iw), grad_out.double())
+    init_arg = initial.numpy() if with_initial else None
+    fwd = seqscan.forward_expnorm(log_gates.numpy(), values.numpy(), init_arg)
+    np.testing.assert_allclose(fwd, out.detach().numpy(), rtol=1e-12, atol=1e-12)
+    dz, dv, di = seqscan.backward_expnorm(log_gates.numpy(), values.numpy(), fwd.astype(np.float32), grad_out.numpy(),
+                                          init_arg)
+    np.testing.assert_allclose(dv, dv_ref.numpy(), rtol=1e-12, atol=1e-12)
+    np.testing.assert_allclose(di, di_ref.numpy(), rtol=1e-12, atol=1e-12)
+    # states rounded to fp32 before they meet the gate; the a^2 / b term is exact on both sides
+    np.testing.assert_allclose(dz, dz_ref.numpy(), rtol=1e-6, atol=1e-6 * np.abs(dz_ref.numpy()).max())
+
+
+def test_expnorm_vs_exp_scan_of_formed_tokens_and_closed_forms():
+    gen = torch.Generator().manual_seed(29)
+    log_gates = -torch.rand(3, 4, 200, generator=gen).mul(5.0).exp().mul(2e-3)
+    values, grad_out = (torch.randn(3, 4, 200, generator=gen) for _ in range(2))
+    z64 = log_gates.double()
+    a = torch.exp(z64)
+    b = torch.sqrt(-torch.expm1(2 * z64))
+    tokens = b * values.double()
+    fwd = seqscan.forward_expnorm(log_gates.numpy(), values.numpy())
+    # the exponentially gated scan of the tokens b v formed outside (rounded to fp32 on that side)
+    np.testing.assert_allclose(fwd, seqscan.forward_exp(log_gates.numpy(), tokens.float().numpy()), rtol=1e-5, atol=1e-5)
+    states = fwd.astype(np.float32)
+    dz, dv, di = seqscan.backward_expnorm(log_gates.numpy(), values.numpy(), states, grad_out.numpy())
+    dz_scan, dt, di_scan = seqscan.backward_exp(log_gates.numpy(), states, grad_out.numpy())
+    # chain rule through tokens = b v, b = sqrt(1 - exp(2 z)):  d_v = d_tokens b;  d_z = d_z(scan) - d_tokens v a^2 / b
+    np.testing.assert_allclose(dv, dt * b.numpy(), rtol=1e-10, atol=1e-12)
+    np.testing.assert_allclose(dz, dz_scan - dt * (values.double() * a * a / b).numpy(), rtol=1e-8, atol=1e-9)
+    np.testing.assert_allclose(di, di_scan, rtol=1e-12)
+    # a = 0.6 exactly-ish (z = log 0.6 rounded to fp32): b = 0.8, so x[t] = 0.6 x[t-1] + 0.8 v[t]
+    T = 25
+    z = np.full((1, 1, T), np.log(0.6), np.float32)
+    v = values[:1, :1, :T].numpy()
+    want = np.zeros(T)
+    s = 0.0
+    a6 = np.exp(np.float64(z[0, 0, 0]))
+    for t in range(T):
+        s = a6 * s + np.sqrt(1.0 - a6 * a6) * float(v[0, 0, t])
+        want[t] = s
+    np.testing.assert_allclose(seqscan.forward_expnorm(z, v)[0, 0], want, rtol=1e-13)
+    assert abs(np.sqrt(1.0 - a6 * a6) - 0.8) < 1e-7
+    # a constant value c from a zero state tends to c b / (1 - a) = c sqrt((1 + a) / (1 - a))
+    out = seqscan.forward_expnorm(np.full((1, 1, 400), np.log(0.6), np.float32), np.full((1, 1, 400), 1.5, np.float32))
+    np.testing.assert_allclose(out[0, 0, -1], 1.5 * np.sqrt((1 + a6) / (1 - a6)), rtol=1e-12)
+    # z = -800 (gate 0): the values themselves; z = 0 (gate 1, scale 0): the initial state stays
+    x = values[:1, :1, :50].numpy()
+    np.testing.assert_allclose(seqscan.forward_expnorm(np.full_like(x, -800.0), x), x, rtol=1e-12, atol=1e-12)
+    np.testing.assert_allclose(seqscan.forward_expnorm(np.zeros_like(x), x, np.full((1, 1), 0.5, np.float32)), 0.5,
+                               rtol=1e-12, atol=1e-12)
+    # unit-variance values keep a unit-variance state (what the scale is for): stationary variance b^2 / (1 - a^2) = 1
+    big = torch.randn(64, 1, 20000, generator=gen)
+    out = seqscan.forward_expnorm(np.full((64, 1, 20000), -0.05, np.float32), big.numpy())
+    assert abs(out[:, :, 2000:].var() - 1.0) < 0.05
