@@ -63,17 +63,17 @@ __device__ __forceinline__ void sigmoid_pair(float v, float& gate, float& comple
 
 // exp(v) and sqrt(1 - exp(2 v)) for v <= 0 (0 for v > 0).  1 - exp(w), w = 2 v, loses
 // its leading digits to cancellation as w approaches 0, where the gates of long
-// memories live; for w > -1/16 it is summed as -w (1 + w/2 (1 + w/3 (1 + w/4 (1 + w/5))))
+// memories live; for w > -1/16 it is summed as -w (1 + w/2 + w^2/6 + w^3/24 + w^4/120)
 // instead (truncation below 2e-9 relative; the difference 1 - a^2 is good to 1e-6 relative
 // below that), so the scale keeps fp32 accuracy for every gate.  v = 0, the
 // out-of-row fill, gives exactly (1, 0).
 __device__ __forceinline__ void exp_norm_pair(float v, float& gate, float& scale) {
     gate = exp_gate(v);
     const float w = v + v;
-    float series = __builtin_fmaf(w, 0.2f, 1.0f);
-    series = __builtin_fmaf(w * 0.25f, series, 1.0f);
-    series = __builtin_fmaf(w * (1.0f / 3.0f), series, 1.0f);
-    series = __builtin_fmaf(w * 0.5f, series, 1.0f);
+    float series = __builtin_fmaf(w, 1.0f / 120.0f, 1.0f / 24.0f);
+    series = __builtin_fmaf(series, w, 1.0f / 6.0f);
+    series = __builtin_fmaf(series, w, 0.5f);
+    series = __builtin_fmaf(series, w, 1.0f);
     const float direct = __builtin_fmaf(-gate, gate, 1.0f);
     const float m = w > -0.0625f ? -w * series : direct;
     scale = __builtin_amdgcn_sqrtf(__builtin_fmaxf(m, 0.0f));
