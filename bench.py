@@ -20,7 +20,12 @@ host cores on a bounded sample of the same workload.
 same buffers with the same read/write mix (tests/native/stream_probe.hip),
 timed after the scan's timed region.
 
-Other workloads: --dtype {fp32,bf16,fp16,c64} --shape B D T.  --sweep FILE runs
+Other workloads: --dtype {fp32,bf16,fp16,c64} --shape B D T; --gate {sigmoid,exp,lerp,
+exp_norm} times the scans whose gate non-linearity (and, for lerp and exp_norm, whose
+token) is formed inside the kernels: the first input then holds gate pre-activations
+(logarithms for exp and exp_norm) of the same gates, the forward kernel moves 3 tensors
+and the backward kernel 5 (sigmoid, exp) or 6 (lerp, exp_norm: it reads the values
+again).  --sweep FILE runs
 the reference's benchmark grid, one JSON line per point into FILE and the same
 points as a Markdown table into FILE.md (the single summary line is still
 printed).  The reference's max-abs-error table is asserted by
@@ -47,8 +52,8 @@ HBM_PEAK_GBPS = 8000.0  # MI355X HBM3E, published peak
 # this script, so the figure is carried over from those runs, not measured in
 # the run that prints it; `traffic_source` in the output says so.
 MEASURED_TRAFFIC_BYTES = {
-    ((8, 1536, 65536), "fp32"): (4721988 * 2 + 6292382) * 1024,
-    ((8, 1536, 65536), "bf16"): (2367186 * 2 + 3146579) * 1024,
+    ((8, 1536, 65536), "fp32"): (4721467 * 2 + 6292215) * 1024,
+    ((8, 1536, 65536), "bf16"): (2367395 * 2 + 3146527) * 1024,
 }
 TRAFFIC_SOURCE = {
     ((8, 1536, 65536), "fp32"): "profiles/scan_f32_8x1536x65536_fwd_bwd.md (rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE); "
@@ -67,6 +72,9 @@ def parse_args():
                     help="untimed warm-up steps (default 5; 100 for workloads below 1 GiB per tensor)")
     ap.add_argument("--dtype", choices=["fp32", "bf16", "fp16", "c64"], default="fp32")
     ap.add_argument("--shape", type=int, nargs=3, default=[8, 1536, 65536], metavar=("B", "D", "T"))
+    ap.add_argument("--gate", choices=["identity", "sigmoid", "exp", "lerp", "exp_norm"], default="identity",
+                    help="gate non-linearity applied inside the kernels (real dtypes; default: finished gates, "
+                         "the reference's operator)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--pmc-calibration", action="store_true",
                     help="for rocprofv3 --pmc runs: 3 plain copies of 1 GiB (torch copy_), then 3 steps "
@@ -77,7 +85,11 @@ def parse_args():
     return ap.parse_args()
 
 
-def make_inputs(shape, dtype_name, device):
+GATE_CODES = {"identity": 0, "sigmoid": 1, "lerp": 2, "exp": 3, "exp_norm": 4}  # ascan_gate of include/ascan.h
+GATES_WITH_VALUES = ("lerp", "exp_norm")
+
+
+def make_inputs(shape, dtype_name, device, gate="identity"):
     import torch
 
     torch.manual_seed(12312323)
@@ -90,12 +102,16 @@ def make_inputs(shape, dtype_name, device):
         return gates, tokens, grad_out
     dt = {"fp32": torch.float32, "bf16": torch.bfloat16, "fp16": torch.float16}[dtype_name]
     gates = (0.999 + 0.001 * torch.rand(*shape, device=device)).half().float()
+    if gate in ("sigmoid", "lerp"):  # the pre-activations of the same gates
+        gates = torch.logit(gates.clamp(max=1.0 - 2.0 ** -20))
+    elif gate in ("exp", "exp_norm"):  # their logarithms (strictly negative for exp_norm)
+        gates = torch.log(gates).clamp(max=-(2.0 ** -20))
     tokens = torch.rand(*shape, device=device)
     grad_out = torch.randn(*shape, device=device)
     return gates.to(dt), tokens.to(dt), grad_out.to(dt)
 
 
-def run_workload(shape, dtype_name, steps, warmup):
+def run_workload(shape, dtype_name, steps, warmup, gate="identity"):
     """Times `steps` forward+backward passes; returns a dict of measurements.
 
     Tensors below 1 GiB are comparable to the 256 MB Infinity Cache, so such
@@ -108,7 +124,24 @@ def run_workload(shape, dtype_name, steps, warmup):
     from accelerated_scan import _abi
 
     device = torch.device("cuda:0")
-    gates, tokens, grad_out = make_inputs(shape, dtype_name, device)
+    gates, tokens, grad_out = make_inputs(shape, dtype_name, device, gate)
+    code = GATE_CODES[gate]
+    bwd_tensors = 6 if gate in GATES_WITH_VALUES else 5
+
+    def forward(g, x, states):
+        if gate == "identity":
+            _abi.forward(g, x, states, False)
+        else:
+            _abi.forward_gated(g, x, states, code)
+
+    def backward(g, x, states, d, d_gates, d_tokens):
+        if gate == "identity":
+            _abi.backward(g, states, d, d_gates, d_tokens)
+        elif gate in GATES_WITH_VALUES:
+            _abi.backward_gated_values(g, x, states, d, d_gates, d_tokens, code)
+        else:
+            _abi.backward_gated(g, states, d, d_gates, d_tokens, code)
+
     elems = tokens.numel()
     esize = tokens.element_size()
     nsets = 1 if elems * esize >= (1 << 30) else 4
@@ -116,18 +149,18 @@ def run_workload(shape, dtype_name, steps, warmup):
     for k in range(nsets):
         g, x, d = (gates, tokens, grad_out) if k == 0 else (gates.clone(), tokens.clone(), grad_out.clone())
         states, d_gates, d_tokens = torch.empty_like(x), torch.empty_like(x), torch.empty_like(x)
-        _abi.forward(g, x, states, False)  # the backward passes read valid states from the first step on
+        forward(g, x, states)  # the backward passes read valid states from the first step on
         sets.append((g, x, d, states, d_gates, d_tokens))
 
     def step(i, events=None):
         g, x, _, states, _, _ = sets[i % nsets]
         if events is not None:
             events[0].record()
-        _abi.forward(g, x, states, False)
+        forward(g, x, states)
         if events is not None:
             events[1].record()
-        g, _, d, states, d_gates, d_tokens = sets[(i + nsets // 2) % nsets]
-        _abi.backward(g, states, d, d_gates, d_tokens)
+        g, x, d, states, d_gates, d_tokens = sets[(i + nsets // 2) % nsets]
+        backward(g, x, states, d, d_gates, d_tokens)
         if events is not None:
             events[2].record()
 
@@ -160,9 +193,10 @@ def run_workload(shape, dtype_name, steps, warmup):
         "ms_per_step": ms_per_step,
         "fwd_ms": fwd_ms,
         "bwd_ms": bwd_ms,
-        "gbps": 8 * elems * esize / (ms_per_step * 1e-3) / 1e9,
+        "bwd_tensors": bwd_tensors,
+        "gbps": (3 + bwd_tensors) * elems * esize / (ms_per_step * 1e-3) / 1e9,
         "fwd_gbps": 3 * elems * esize / (fwd_ms * 1e-3) / 1e9,
-        "bwd_gbps": 5 * elems * esize / (bwd_ms * 1e-3) / 1e9,
+        "bwd_gbps": bwd_tensors * elems * esize / (bwd_ms * 1e-3) / 1e9,
     }
 
 
@@ -405,6 +439,10 @@ def main():
     _abi.load()  # no fallback: fail here if the HIP library is missing
 
     shape = tuple(args.shape)
+    gated = args.gate != "identity"
+    if gated and args.dtype == "c64":
+        print("bench.py: --gate needs a real dtype", file=sys.stderr)
+        return 2
     # Sub-millisecond steps need a longer run: with 5 + 20 steps of 0.4 ms the whole measurement is over in 10 ms,
     # before clocks and caches have settled (measured at (4,1024,8192) complex64: 68.4 % of peak with 5 + 20 steps,
     # 72.2 % with 100 + 200).  The headline's defaults are the driver's: 5 + 20 steps of 4.4 ms.
@@ -420,12 +458,12 @@ def main():
         for _ in range(3):
             dst.copy_(src)
         torch.cuda.synchronize()
-        m = run_workload(shape, args.dtype, 3, 0)
+        m = run_workload(shape, args.dtype, 3, 0, args.gate)
         device_ceiling(shape, args.dtype, m["buffers"], steps=3, warmup=0)  # the probe kernels, for the same counters
         print(json.dumps({"calibration_copy_bytes_read": src.numel() * 4, "calibration_copy_bytes_written":
                           src.numel() * 4, "workload_shape": list(shape), "dtype": args.dtype}))
         return 0
-    m = run_workload(shape, args.dtype, args.steps, args.warmup)
+    m = run_workload(shape, args.dtype, args.steps, args.warmup, args.gate)
     ceiling = device_ceiling(shape, args.dtype, m.pop("buffers"))
 
     if args.sweep:
@@ -433,10 +471,14 @@ def main():
 
     dtype_field = {"fp32": "f32", "bf16": "bf16 storage, f32 arithmetic",
                    "fp16": "f16 storage, f32 arithmetic", "c64": "complex64 (f32 pairs)"}[args.dtype]
-    bwd_bytes = 5 * m["elems"] * m["esize"]
+    bwd_bytes = m["bwd_tensors"] * m["elems"] * m["esize"]
+    gate_text = {"identity": "", "sigmoid": ", gates = sigmoid(stored) inside the kernels",
+                 "exp": ", gates = exp(stored) inside the kernels",
+                 "lerp": ", x[t] = a x[t-1] + (1 - a) v[t] with a = sigmoid(stored) inside the kernels",
+                 "exp_norm": ", x[t] = a x[t-1] + sqrt(1 - a^2) v[t] with a = exp(stored) inside the kernels"}[args.gate]
     result = {
-        "metric": "fwd+bwd achieved HBM GB/s (algorithmic bytes: 3 tensors forward + 5 backward) "
-                  f"at {shape} {args.dtype}",
+        "metric": f"fwd+bwd achieved HBM GB/s (algorithmic bytes: 3 tensors forward + {m['bwd_tensors']} backward) "
+                  f"at {shape} {args.dtype}" + gate_text,
         "value": m["gbps"],
         "unit": "GB/s",
         "n_gpus": 1,
@@ -451,7 +493,9 @@ def main():
         "config": {
             "workload": f"scan forward + fused backward, shape {list(shape)}, {args.dtype}, " + (
                 "gates r*exp(i*theta) with r ~ 0.9+0.1*U(0,1), tokens and grad_out complex N(0,1)"
-                if args.dtype == "c64" else "gates 0.999+0.001*U(0,1), tokens U(0,1), grad_out N(0,1)"),
+                if args.dtype == "c64" else "gates 0.999+0.001*U(0,1), tokens U(0,1), grad_out N(0,1)") + (
+                f"; gate {args.gate}: the first input holds the gates' " + (
+                    "logarithms" if args.gate in ("exp", "exp_norm") else "sigmoid pre-activations") if gated else ""),
             "input_sets": m["input_sets"],
             "steps_with_kernel_events": m["event_steps"],
             "fwd_ms": m["fwd_ms"],
@@ -469,12 +513,12 @@ def main():
             "frac": m["bwd_gbps"] / HBM_PEAK_GBPS,
             "algorithmic_bytes_per_launch": bwd_bytes,
             "avg_launch_ms": m["bwd_ms"],
-            "traffic": MEASURED_TRAFFIC_BYTES.get((shape, args.dtype)),
-            "traffic_source": TRAFFIC_SOURCE.get((shape, args.dtype)),
+            "traffic": None if gated else MEASURED_TRAFFIC_BYTES.get((shape, args.dtype)),
+            "traffic_source": None if gated else TRAFFIC_SOURCE.get((shape, args.dtype)),
             "device_ceiling": ceiling,
         },
     }
-    if not args.no_cpu_baseline:
+    if not args.no_cpu_baseline and not gated:  # the baseline is the reference's operator: finished gates
         result["cpu_baseline"] = cpu_baseline(shape, args.dtype)
     print(json.dumps(result))
     return 0
