@@ -25,7 +25,7 @@ exp_norm} times the scans whose gate non-linearity (and, for lerp and exp_norm, 
 token) is formed inside the kernels: the first input then holds gate pre-activations
 (logarithms for exp and exp_norm) of the same gates, the forward kernel moves 3 tensors
 and the backward kernel 5 (sigmoid, exp) or 6 (lerp, exp_norm: it reads the values
-again).  --sweep FILE runs
+again).  --reverse times the reverse scan and its own backward kernel.  --sweep FILE runs
 the reference's benchmark grid, one JSON line per point into FILE and the same
 points as a Markdown table into FILE.md (the single summary line is still
 printed).  The reference's max-abs-error table is asserted by
@@ -75,6 +75,8 @@ def parse_args():
     ap.add_argument("--gate", choices=["identity", "sigmoid", "exp", "lerp", "exp_norm"], default="identity",
                     help="gate non-linearity applied inside the kernels (real dtypes; default: finished gates, "
                          "the reference's operator)")
+    ap.add_argument("--reverse", action="store_true",
+                    help="time the reverse scan x[t] = gate[t] x[t+1] + token[t] and its own fused backward kernel")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--pmc-calibration", action="store_true",
                     help="for rocprofv3 --pmc runs: 3 plain copies of 1 GiB (torch copy_), then 3 steps "
@@ -111,7 +113,7 @@ def make_inputs(shape, dtype_name, device, gate="identity"):
     return gates.to(dt), tokens.to(dt), grad_out.to(dt)
 
 
-def run_workload(shape, dtype_name, steps, warmup, gate="identity"):
+def run_workload(shape, dtype_name, steps, warmup, gate="identity", reverse=False):
     """Times `steps` forward+backward passes; returns a dict of measurements.
 
     Tensors below 1 GiB are comparable to the 256 MB Infinity Cache, so such
@@ -130,13 +132,13 @@ def run_workload(shape, dtype_name, steps, warmup, gate="identity"):
 
     def forward(g, x, states):
         if gate == "identity":
-            _abi.forward(g, x, states, False)
+            _abi.forward(g, x, states, reverse)
         else:
             _abi.forward_gated(g, x, states, code)
 
     def backward(g, x, states, d, d_gates, d_tokens):
         if gate == "identity":
-            _abi.backward(g, states, d, d_gates, d_tokens)
+            _abi.backward(g, states, d, d_gates, d_tokens, reverse=reverse)
         elif gate in GATES_WITH_VALUES:
             _abi.backward_gated_values(g, x, states, d, d_gates, d_tokens, code)
         else:
@@ -443,6 +445,9 @@ def main():
     if gated and args.dtype == "c64":
         print("bench.py: --gate needs a real dtype", file=sys.stderr)
         return 2
+    if gated and args.reverse:
+        print("bench.py: the gated scans run forward in time only", file=sys.stderr)
+        return 2
     # Sub-millisecond steps need a longer run: with 5 + 20 steps of 0.4 ms the whole measurement is over in 10 ms,
     # before clocks and caches have settled (measured at (4,1024,8192) complex64: 68.4 % of peak with 5 + 20 steps,
     # 72.2 % with 100 + 200).  The headline's defaults are the driver's: 5 + 20 steps of 4.4 ms.
@@ -458,12 +463,12 @@ def main():
         for _ in range(3):
             dst.copy_(src)
         torch.cuda.synchronize()
-        m = run_workload(shape, args.dtype, 3, 0, args.gate)
+        m = run_workload(shape, args.dtype, 3, 0, args.gate, args.reverse)
         device_ceiling(shape, args.dtype, m["buffers"], steps=3, warmup=0)  # the probe kernels, for the same counters
         print(json.dumps({"calibration_copy_bytes_read": src.numel() * 4, "calibration_copy_bytes_written":
                           src.numel() * 4, "workload_shape": list(shape), "dtype": args.dtype}))
         return 0
-    m = run_workload(shape, args.dtype, args.steps, args.warmup, args.gate)
+    m = run_workload(shape, args.dtype, args.steps, args.warmup, args.gate, args.reverse)
     ceiling = device_ceiling(shape, args.dtype, m.pop("buffers"))
 
     if args.sweep:
@@ -478,7 +483,7 @@ def main():
                  "exp_norm": ", x[t] = a x[t-1] + sqrt(1 - a^2) v[t] with a = exp(stored) inside the kernels"}[args.gate]
     result = {
         "metric": f"fwd+bwd achieved HBM GB/s (algorithmic bytes: 3 tensors forward + {m['bwd_tensors']} backward) "
-                  f"at {shape} {args.dtype}" + gate_text,
+                  f"at {shape} {args.dtype}" + gate_text + (", reverse scan and its backward pass" if args.reverse else ""),
         "value": m["gbps"],
         "unit": "GB/s",
         "n_gpus": 1,
@@ -491,7 +496,8 @@ def main():
         "dtype": dtype_field,
         "data": "synthetic",
         "config": {
-            "workload": f"scan forward + fused backward, shape {list(shape)}, {args.dtype}, " + (
+            "workload": ("reverse scan + its fused backward" if args.reverse else "scan forward + fused backward")
+                        + f", shape {list(shape)}, {args.dtype}, " + (
                 "gates r*exp(i*theta) with r ~ 0.9+0.1*U(0,1), tokens and grad_out complex N(0,1)"
                 if args.dtype == "c64" else "gates 0.999+0.001*U(0,1), tokens U(0,1), grad_out N(0,1)") + (
                 f"; gate {args.gate}: the first input holds the gates' " + (
@@ -518,7 +524,7 @@ def main():
             "device_ceiling": ceiling,
         },
     }
-    if not args.no_cpu_baseline and not gated:  # the baseline is the reference's operator: finished gates
+    if not args.no_cpu_baseline and not gated and not args.reverse:  # the baseline is the reference's operator
         result["cpu_baseline"] = cpu_baseline(shape, args.dtype)
     print(json.dumps(result))
     return 0
