@@ -27,8 +27,8 @@ token) is formed inside the kernels: the first input then holds gate pre-activat
 and the backward kernel 5 (sigmoid, exp) or 6 (lerp, exp_norm: it reads the values
 again).  --reverse times the reverse scan and its own backward kernel.  --sweep FILE runs
 the reference's benchmark grid, one JSON line per point into FILE and the same
-points as a Markdown table into FILE.md (the single summary line is still
-printed).  The reference's max-abs-error table is asserted by
+points as a Markdown table into FILE.md and the (8,1536,T) grid as FILE.csv (the
+single summary line is still printed).  The reference's max-abs-error table is asserted by
 tests/test_precision_gpu.py.
 """
 
@@ -345,6 +345,20 @@ def run_sweep(path, steps, warmup):
         rec["train_real_inputs_ms"] = ms
         emit(rec)
     write_sweep_markdown(records, str(path) + ".md", steps, warmup)
+    write_sweep_csv(records, str(path) + ".csv")
+
+
+def write_sweep_csv(records, path):
+    """The (8, 1536, T) grid as CSV, one row per dtype and T (the reference's
+    harness saves one CSV per direction with a SEQUENCE_LENGTH column,
+    tests/bench.py:100-115 of the reference); empty cells were not measured."""
+    columns = ("forward_ms", "reverse_ms", "backward_ms", "train_ms")
+    with open(path, "w") as f:
+        f.write("dtype,SEQUENCE_LENGTH," + ",".join(columns) + "\n")
+        for rec in records:
+            if rec["dtype"] != "c64":
+                f.write(f"{rec['dtype']},{rec['shape'][2]}," + ",".join(
+                    f"{rec[c]:.6f}" if c in rec else "" for c in columns) + "\n")
 
 
 def write_sweep_markdown(records, path, steps, warmup):
