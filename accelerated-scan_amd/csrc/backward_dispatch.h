@@ -112,8 +112,9 @@ int backward_typed(const BackwardBuffers& b, int64_t rows, int64_t T, int act, c
         const int64_t SUBS = (int64_t)backward_blocks_of(act, SplitTuning<Tr>::UB) * 64 * Tr::EPV;
         constexpr int64_t SUBSG = (int64_t)SplitTuning<Tr>::UBG * 64 * Tr::EPV;
         const bool regular = lead == 0 && T % (SUBS * kSplitWaves) == 0;
-        const int64_t ntiles = host_tiles_per_row<Tr>(T, (regular ? SUBS : SUBSG) * kSplitWaves, regular, at);
-        if (want_split(rows, ntiles) && workspace_fits(ws, rows, ntiles)) {
+        const int64_t tile = (regular ? SUBS : SUBSG) * kSplitWaves;
+        const int64_t ntiles = host_tiles_per_row<Tr>(T, tile, regular, at);
+        if (want_split(kSweepClass<Tr>, rows, T * kElem, tile * kElem, ntiles, regular) && workspace_fits(ws, rows, ntiles)) {
             err = with_gate<Tr, REV>(act, [&](auto gate) {
                 constexpr int ACT = decltype(gate)::value;
                 return regular ? launch_backward_split<Tr, REV, true, ACT>(b, rows, T, at.grid, ntiles, ws, stream)

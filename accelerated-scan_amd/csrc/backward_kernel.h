@@ -59,20 +59,18 @@ __global__ void __launch_bounds__(64 * kMaxWavesPerBlock)
     const int64_t ntiles = tiles_per_row(longest, TILE, head);
     __shared__ V slots_all[W == 1 ? 1 : 2 * kSlotsPerBuffer];
     __shared__ S stage_all[PACKED ? W * SUB : 1];
-    // Split rows: the workgroups take tiles by ticket, row by row, until none
+    // Split rows: the workgroups take tiles by ticket, in memory order, until none
     // is left; a workgroup only ever waits for tiles whose owners started before it.
-    __shared__ long long split_mailbox[2];
+    __shared__ int split_mailbox[2];
     __shared__ u32x4_t parked[SPLIT ? NIN * U * 64 : 1];  // wave 0's raw vectors during its walk back
     __shared__ V parked_values[SPLIT ? 4 * U * 64 : 1];  // and its per-lane scan results
-    SplitWalk walk;  // starts at row blockIdx % rows
-    walk.row = SPLIT ? (int64_t)(blockIdx.x % rows) : 0;
-    walk.has_drawn = false;
+    const unsigned long long split_wait_limit = SPLIT ? split->wait_limit : 0ull;  // the longest wait allowed
     for (bool first_visit = true;; first_visit = false) {
     int64_t row;
     int w, slot_base;
     int64_t k_begin = 0, k_end = ntiles;
     if constexpr (SPLIT) {
-        if (!take_split_tile(split, rows, ntiles, walk, row, k_begin, split_mailbox)) break;
+        if (!take_split_tile(split, rows, ntiles, row, k_begin, split_mailbox)) break;
         k_end = k_begin + 1;
         int thread = threadIdx.x;
         asm volatile("" : "+v"(thread));  // nothing derived from the wave index is carried from visit to visit
@@ -281,7 +279,8 @@ __global__ void __launch_bounds__(64 * kMaxWavesPerBlock)
         V c;
         if constexpr (SPLIT) {
             exchange_carries_split<V, W, U>(
-                totA, totX, c, slots, w, lane, split, split_records(split, rows) + row * ntiles, 1, k, vzero<V>(),
+                totA, totX, c, slots, w, lane, split, split_wait_limit, split_records(split) + row * ntiles, k, ntiles,
+                vzero<V>(),
                 [&] {
 #pragma unroll
                     for (int j = 0; j < U; ++j) {

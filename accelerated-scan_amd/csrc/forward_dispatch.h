@@ -99,8 +99,9 @@ int forward_typed(const void* gates, const void* tokens, void* out, const void* 
         const int64_t SUBS = (int64_t)forward_split_blocks_of(act, SplitTuning<Tr>::U) * 64 * Tr::EPV;
         const int64_t SUBSG = (int64_t)forward_split_blocks_of(act, SplitTuning<Tr>::UG) * 64 * Tr::EPV;
         const bool regular = lead == 0 && T % (SUBS * kSplitWaves) == 0;
-        const int64_t ntiles = host_tiles_per_row<Tr>(T, (regular ? SUBS : SUBSG) * kSplitWaves, regular, at);
-        if (want_split(rows, ntiles) && workspace_fits(ws, rows, ntiles)) {
+        const int64_t tile = (regular ? SUBS : SUBSG) * kSplitWaves;
+        const int64_t ntiles = host_tiles_per_row<Tr>(T, tile, regular, at);
+        if (want_split(kSweepClass<Tr>, rows, T * kElem, tile * kElem, ntiles, regular) && workspace_fits(ws, rows, ntiles)) {
             auto go = [&](auto rev, auto reg, auto gate) {
                 return launch_forward_split<Tr, decltype(rev)::value, decltype(reg)::value, decltype(gate)::value>(
                     gates, tokens, out, initial, rows, T, at.grid, ntiles, ws, stream);

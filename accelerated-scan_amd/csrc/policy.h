@@ -166,20 +166,34 @@ inline int launch_status(hipError_t e) {
 }
 
 
-// Split-row policy.  A call is split when its rows alone would leave most
-// compute units without a workgroup and every row has several tiles.  Split
-// tiles are those of the long-row kernels (16 waves): a tile costs one ticket,
-// and tickets of one row are drawn from one address (measured with 4-wave
-// tiles: a single row of 64 Mi elements 1.87 ms, with 16-wave tiles 0.59 ms;
-// 128 rows of 1 Mi elements 0.84 and 0.75 ms).
+// Split-row policy.  With a table from the caller, the tiles of all rows can be
+// swept in memory order by persistent 16-wave workgroups (split.h).  That is the only
+// way to occupy the GPU when there are fewer rows than compute units, and for long
+// rows it is faster than one workgroup walking each row whatever their number --
+// where the tiles are large and mostly full.  Measured at (8,1536,T), forward +
+// backward, % of the 8 TB/s peak, row walk -> sweep: fp32 T = 16384 72 -> 81,
+// 32768 72 -> 82, 49152 65 -> 82, 65536 73 -> 82.5, 65533 (five tiles for four
+// tiles' worth of row) 68 -> 71.5, 24576 (1.5 tiles) 71 -> 75, 20000 (1.2 tiles)
+// 74 -> 71, 8192 (half a tile) 76 -> 72; bf16 T = 32768 72 -> 81, 65536 74 -> 82,
+// but 65533, whose kernels carry masking code and take 32 KiB tiles, 71 -> 62;
+// complex64 (8,768,65536) 71 -> 70 with 64 KiB forward tiles (which spill) and 64
+// with 32 KiB ones.  A tile costs a ticket, a look at the table and three barriers,
+// about 2.4 us in which its compute unit requests nothing, whatever its size.
+// ASCAN_SPLIT_MAX_ROWS (0 = never split) and ASCAN_SPLIT_MIN_ROW_BYTES (split every
+// row at least that long) override the rule, read once.
 constexpr int kSplitWaves = 16;
-constexpr int64_t kSplitMaxRowsDefault = 128;
+constexpr int64_t kSweepMinRowBytes = 64 * 1024;
 
+int64_t env_int64(const char* name, int64_t fallback) {
+    const char* s = getenv(name);
+    return s ? (int64_t)atoll(s) : fallback;
+}
 int64_t split_max_rows() {
-    static const int64_t v = [] {
-        const char* s = getenv("ASCAN_SPLIT_MAX_ROWS");
-        return s ? (int64_t)atoll(s) : kSplitMaxRowsDefault;
-    }();
+    static const int64_t v = env_int64("ASCAN_SPLIT_MAX_ROWS", INT64_MAX);
+    return v;
+}
+int64_t split_forced_min_row_bytes() {
+    static const int64_t v = env_int64("ASCAN_SPLIT_MIN_ROW_BYTES", 0);
     return v;
 }
 
@@ -194,14 +208,44 @@ unsigned long long split_wait_limit() {
     return v;
 }
 
-// With up to 64 rows two tiles per row already pay; up to the limit, four.
-bool want_split(int64_t rows, int64_t ntiles) {
-    return rows <= split_max_rows() && (ntiles >= 4 || (ntiles >= 2 && rows <= 64));
+enum class SweepClass { kF32, kNarrow, kComplex };
+template <class Tr>
+constexpr SweepClass kSweepClass = Tr::kNarrow ? SweepClass::kNarrow
+                                               : (std::is_same<typename Tr::V, float>::value ? SweepClass::kF32
+                                                                                             : SweepClass::kComplex);
+
+// Too few rows to occupy the compute units with one workgroup each: with up to 64
+// rows two tiles per row already pay; up to 128, four.
+bool too_few_rows(int64_t rows, int64_t ntiles) {
+    return (ntiles >= 2 && rows <= 64) || (ntiles >= 4 && rows <= 128);
+}
+
+// `row_bytes`: one row of states; `tile_bytes`, `ntiles`: of the kernel that would run;
+// `regular`: that kernel is the mask-free one.
+bool want_split(SweepClass c, int64_t rows, int64_t row_bytes, int64_t tile_bytes, int64_t ntiles, bool regular) {
+    if (rows > split_max_rows()) return false;
+    if (too_few_rows(rows, ntiles)) return true;
+    if (split_forced_min_row_bytes() > 0) return row_bytes >= split_forced_min_row_bytes();
+    if (row_bytes < kSweepMinRowBytes) return false;
+    if (row_bytes * 10 < ntiles * tile_bytes * 7) return false;  // tiles less than 70 % full
+    switch (c) {
+        case SweepClass::kF32: return true;
+        case SweepClass::kNarrow: return regular;
+        default: return false;
+    }
+}
+
+// Whether some kernel of a call of this shape may want the table (`ntiles_most`: with
+// the smallest tile any kernel uses): what ascan_workspace_bytes goes by.
+bool may_split(bool complex, int64_t rows, int64_t row_bytes, int64_t ntiles_most) {
+    if (rows > split_max_rows()) return false;
+    if (too_few_rows(rows, ntiles_most)) return true;
+    if (split_forced_min_row_bytes() > 0) return row_bytes >= split_forced_min_row_bytes();
+    return !complex && row_bytes >= kSweepMinRowBytes;
 }
 
 size_t split_bytes(int64_t rows, int64_t ntiles) {
-    return sizeof(SplitHeader) + (size_t)rows * sizeof(SplitTicket) +
-           (size_t)rows * (size_t)ntiles * sizeof(SplitRecord);
+    return sizeof(SplitHeader) + sizeof(SplitTicket) + (size_t)rows * (size_t)ntiles * sizeof(SplitRecord);
 }
 
 bool workspace_fits(const Workspace& ws, int64_t rows, int64_t ntiles) {

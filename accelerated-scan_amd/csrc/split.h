@@ -10,27 +10,41 @@ namespace ascan {
 namespace {
 
 // ---------------------------------------------------------------------------
-// Split rows: several workgroups per row, for calls with too few rows to
-// occupy the machine.  A workgroup works on one tile of one row at a time; the
-// state entering the tile comes from the workgroups of the earlier tiles
-// through a small table in global memory (single pass, "decoupled look-back"):
-//   * a workgroup publishes its tile's aggregate (A, X) as soon as it has it;
-//   * it then walks back over the earlier tiles of its row, folding aggregates
-//     until it meets a tile whose inclusive state P is already published;
-//   * it publishes its own inclusive state and finishes the tile.
-// Tiles are handed out by ticket: every row has a counter, and a workgroup
-// takes the next tile of the row it serves with one fetch-add on it.  A tile
-// is therefore only ever waited for by workgroups that started after its
-// owner did: progress never depends on a workgroup that has not been
-// dispatched yet, whatever else is running on the GPU, and the launch size
-// (what an idle GPU holds at once) is a matter of speed only.  One counter per
-// row keeps the fetch-adds of different rows apart (measured: ~11 ns each on
-// one address on an idle GPU, ~60 ns under streaming load; concurrent across
-// addresses).  Each wait is nevertheless bounded by a limit set by the host;
-// a wait that runs out poisons the result with NaN and is counted in the
-// header.  Waiting time is summed from clock differences capped at 10 us
-// each, so a stretch during which the whole kernel was not running does not
-// count.
+// Split rows: the tiles of all rows are handed out in memory order, one tile to
+// one workgroup at a time, and the state entering a tile comes from the
+// workgroups of the row's earlier tiles through a small table in global memory.
+//
+// Order.  There is one ticket counter for the whole launch: ticket n is tile
+// n % ntiles of row n / ntiles, so the resident workgroups together sweep the
+// tensors front to back, each taking the next 16-wave tile whenever it is done
+// with its last.  Measured on MI355X with kernels that only move the bytes
+// (3 reads + 2 writes, 3.2 GB per tensor): one workgroup walking each 256 KiB
+// row 5.56 TB/s (5.1 with rows 192 KiB apart); this sweep, with a wait on the
+// row's earlier tiles before a tile's stores, 6.46 TB/s (6.25).  What the sweep
+// buys is the compact stretch of memory in flight at any one time; what it
+// costs is one look at the table per tile, whose latency (about 3 us under
+// load, same XCD or not) is idle time of one compute unit that the others fill.
+// A ticket is drawn when the workgroup is ready for the tile, never ahead: a
+// tile held back by its owner's previous tile stalls every later tile of the row.
+//
+// Because tickets are taken in order, a tile is only ever waited for by
+// workgroups that started after its owner did: progress never depends on a
+// workgroup that has not been dispatched yet, whatever else is running on the
+// GPU, and the launch size (what an idle GPU holds at once) is a matter of
+// speed only.  Each wait is nevertheless bounded by a limit set by the host; a
+// wait that runs out poisons the result with NaN and is counted in the header.
+// Waiting time is summed from clock differences capped at 10 us each, so a
+// stretch during which the whole kernel was not running does not count.
+//
+// Look-back.  The tiles of a row form windows of 64.  A workgroup publishes its
+// tile's aggregate (A, X) as soon as it has it; the state entering tile k is the
+// state entering k's window folded with the aggregates of the window's tiles
+// before k -- lane i of wave 0 reads tile i of the window, all at once, and the
+// 64 pairs are folded by the wave scan, in one fixed order.  The state entering
+// a window is the inclusive state its predecessor's last tile publishes (the
+// row's start for window 0), so the chain of waits is one hop per 64 tiles, and
+// what a tile receives does not depend on timing: results are reproducible
+// run to run.
 // ---------------------------------------------------------------------------
 struct SplitHeader {
     unsigned long long reserved0;
@@ -40,14 +54,15 @@ struct SplitHeader {
 };
 static_assert(sizeof(SplitHeader) == 64, "header is 64 bytes");
 
-// One ticket counter per row, each on a cache line of its own.
+// The ticket counter of the launch, on a cache line of its own.
 struct alignas(64) SplitTicket {
-    unsigned long long next;  // scan-order index of the next tile to hand out
+    unsigned long long next;  // next tile to hand out: tile next % ntiles of row next / ntiles
     unsigned long long pad[7];
 };
 static_assert(sizeof(SplitTicket) == 64, "ticket line is 64 bytes");
 
 constexpr unsigned long long kWaitStepCap = 1000;  // 10 us in 100 MHz ticks
+constexpr int kSplitWindow = 64;                   // tiles per look-back window: one per lane
 
 // One record per (row, tile).  Every field is a 64-bit word holding an fp32
 // payload in its low half and a tag in its high half (0 = not written yet,
@@ -57,7 +72,7 @@ constexpr unsigned long long kWaitStepCap = 1000;  // 10 us in 100 MHz ticks
 struct alignas(64) SplitRecord {
     unsigned long long a[2];  // aggregate gate product of the tile (re, im)
     unsigned long long x[2];  // aggregate state of the tile from a zero start (re, im)
-    unsigned long long p[2];  // inclusive state at the end of the tile (re, im)
+    unsigned long long p[2];  // inclusive state at the end of the tile (re, im); last tile of a window only
     unsigned long long pad[2];
 };
 static_assert(sizeof(SplitRecord) == 64, "record is 64 bytes");
@@ -103,72 +118,46 @@ __global__ void split_reset_kernel(uint32_t* words, size_t nwords, unsigned long
     if (i < nwords) words[i] = i == 2 ? (uint32_t)wait_limit : (i == 3 ? (uint32_t)(wait_limit >> 32) : 0u);
 }
 
-// Layout of the table: header, one ticket line per row, one record per (row, tile).
-__device__ __forceinline__ SplitTicket* split_tickets(SplitHeader* header) {
+// Layout of the table: header, the ticket line, one record per (row, tile).
+__device__ __forceinline__ SplitTicket* split_ticket(SplitHeader* header) {
     return reinterpret_cast<SplitTicket*>(header + 1);
 }
-__device__ __forceinline__ SplitRecord* split_records(SplitHeader* header, int64_t rows) {
-    return reinterpret_cast<SplitRecord*>(split_tickets(header) + rows);
+__device__ __forceinline__ SplitRecord* split_records(SplitHeader* header) {
+    return reinterpret_cast<SplitRecord*>(split_ticket(header) + 1);
 }
 
-// A workgroup's place in the hand-out of tiles: the row it is taking tiles from
-// and the ticket it has already drawn for its next tile (drawn while the
-// current tile's loads are in flight, so that the fetch-add's latency is off
-// the critical path).  Meaningful in wave 0 only.
-struct SplitWalk {
-    int64_t row;
-    unsigned long long drawn;  // valid when has_drawn
-    bool has_drawn;
-};
-
-__device__ __forceinline__ unsigned long long draw_ticket(SplitTicket* ticket, int lane) {
-    unsigned long long t = 0;
-    if (lane == 0) t = __hip_atomic_fetch_add(&ticket->next, 1ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    return t;  // lane 0 holds the ticket
-}
-__device__ __forceinline__ unsigned long long from_lane0(unsigned long long v) {
-    return ((unsigned long long)(unsigned)__builtin_amdgcn_readfirstlane((int)(v >> 32)) << 32) |
-           (unsigned)__builtin_amdgcn_readfirstlane((int)v);
-}
-
-// Hands the workgroup its next tile.  Workgroup b serves row b % rows -- with
-// fewer rows than workgroups several workgroups share a row and draw its tiles
-// in turn -- and, when that row has no tiles left, the rows b + G, b + 2G, ...
-// (G = workgroups in the launch), so every row is served whatever G is.
-// (Letting idle workgroups look for tiles in other rows was tried: near the end
-// hundreds of them draw from the few counters that still have tiles, and the
-// owners' own draws queue behind them.)  Returns false when the workgroup has
-// nothing left to do.  All threads of the workgroup call it together and get
-// the same answer; `mailbox` is two words of LDS.
-__device__ __forceinline__ bool take_split_tile(SplitHeader* header, int64_t rows, int64_t ntiles, SplitWalk& walk,
-                                                int64_t& row, int64_t& k, long long* mailbox) {
-    if (threadIdx.x < 64) {  // wave 0
-        const int lane = threadIdx.x;
-        SplitTicket* tickets = split_tickets(header);
-        long long got_row = -1, got_k = -1;
-        while (walk.row < rows) {
-            const unsigned long long ticket =
-                from_lane0(walk.has_drawn ? walk.drawn : draw_ticket(&tickets[walk.row], lane));
-            walk.has_drawn = false;
-            if (ticket < (unsigned long long)ntiles) {
-                got_row = walk.row;
-                got_k = (long long)ticket;
-                if (ticket + 1 < (unsigned long long)ntiles) {  // draw the next one now; it is read at the next call
-                    walk.drawn = draw_ticket(&tickets[walk.row], lane);
-                    walk.has_drawn = true;
-                }
-                break;
-            }
-            walk.row += gridDim.x;  // this row is handed out completely
+// Hands the workgroup its next tile, or returns false when none is left: thread 0
+// draws the ticket, all threads of the workgroup call this together and get the
+// same answer through `mailbox` (two words of LDS).  rows * ntiles is below 2^31.
+//
+// The ticket is drawn here, when the workgroup is ready to start on it, so tiles
+// start in ticket order.  (Drawn a tile step ahead, behind the previous tile's
+// loads, the fetch-add costs nothing, but then a tile starts whenever its owner's
+// previous tile is done, and a workgroup held up in its look-back holds up the
+// later tiles of the row it has the next ticket for: measured, a row's earlier
+// tiles were ready 8-9 us after the later ones one time in ten, and the kernel lost
+// a fifth of its speed.)  The draw, the mailbox and the barrier stay together in
+// one straight piece of code, and what comes out of the mailbox is made wave-uniform
+// explicitly, so that the loop around it branches uniformly: a thread-0-only draw
+// at the far end of the loop body was compiled into a loop in which thread 0 left
+// for its draw while the other lanes went on to read the mailbox it had yet to fill.
+__device__ __forceinline__ bool take_split_tile(SplitHeader* header, int64_t rows, int64_t ntiles, int64_t& row,
+                                                int64_t& k, int* mailbox) {
+    if (threadIdx.x == 0) {
+        const unsigned long long ticket = __hip_atomic_fetch_add(&split_ticket(header)->next, 1ull, __ATOMIC_RELAXED,
+                                                                 __HIP_MEMORY_SCOPE_AGENT);
+        int got_row = -1, got_k = -1;
+        if (ticket < (unsigned long long)(rows * ntiles)) {
+            const unsigned n = (unsigned)ticket, per_row = (unsigned)ntiles;
+            got_row = (int)(n / per_row);
+            got_k = (int)(n - (unsigned)got_row * per_row);
         }
-        if (lane == 0) {
-            mailbox[0] = got_row;
-            mailbox[1] = got_k;
-        }
+        mailbox[0] = got_row;
+        mailbox[1] = got_k;
     }
     __syncthreads();
-    const long long got_row = mailbox[0];
-    const long long got_k = mailbox[1];
+    const int got_row = __builtin_amdgcn_readfirstlane(mailbox[0]);
+    const int got_k = __builtin_amdgcn_readfirstlane(mailbox[1]);
     __syncthreads();  // the mailbox may be rewritten by the next call
     if (got_row < 0) return false;
     row = got_row;
@@ -176,117 +165,92 @@ __device__ __forceinline__ bool take_split_tile(SplitHeader* header, int64_t row
     return true;
 }
 
-__device__ __forceinline__ float read_lane_at(float v, int lane) {
-    return i2f(__builtin_amdgcn_readlane(f2i(v), lane));
+// Waits (bounded) until both fields are published and returns them; false when the
+// wait ran out.  The words of both fields are requested together: one round trip.
+// The clock is only read once a look has found nothing.
+template <class V>
+__device__ __forceinline__ bool await_pair(unsigned long long (&fa)[2], unsigned long long (&fx)[2], V& a, V& x,
+                                           unsigned long long limit) {
+    unsigned long long waited = 0, last = 0;
+    for (bool first = true;; first = false) {
+        const bool has_a = peek(fa, a);
+        const bool has_x = peek(fx, x);
+        if (has_a && has_x) return true;
+        const unsigned long long now = __builtin_amdgcn_s_memrealtime();
+        if (!first) waited += now - last < kWaitStepCap ? now - last : kWaitStepCap;
+        last = now;
+        if (waited > limit) return false;
+        __builtin_amdgcn_s_sleep(1);
+    }
 }
-__device__ __forceinline__ cfloat read_lane_at(cfloat v, int lane) {
-    cfloat r;
-    r.re = read_lane_at(v.re, lane);
-    r.im = read_lane_at(v.im, lane);
-    return r;
+template <class V>
+__device__ __forceinline__ bool await_field(unsigned long long (&field)[2], V& v, unsigned long long limit) {
+    unsigned long long waited = 0, last = 0;
+    for (bool first = true;; first = false) {
+        if (peek(field, v)) return true;
+        const unsigned long long now = __builtin_amdgcn_s_memrealtime();
+        if (!first) waited += now - last < kWaitStepCap ? now - last : kWaitStepCap;
+        last = now;
+        if (waited > limit) return false;
+        __builtin_amdgcn_s_sleep(1);
+    }
 }
 
 // State entering scan-order tile k of a row, for wave 0 of the workgroup that
-// owns the tile.  `mine` is that row's first record; records of successive
-// tiles are `stride` apart.  (tileA, tileX) is this tile's aggregate and
-// `row_start` the state entering tile 0.
-//
-// The walk back is done 64 tiles at a time: lane i looks at tile k-1-i, all
-// lanes wait for their record in parallel (one memory round trip instead of one
-// per tile), then the records from the nearest inclusive state forward are
-// folded with lane reads.
+// owns the tile.  `mine` is the row's first record; (tileA, tileX) is this
+// tile's aggregate and `row_start` the state entering tile 0.
 template <class V>
-__device__ __forceinline__ V split_look_back(SplitHeader* header, SplitRecord* mine, int64_t stride, int64_t k,
-                                             V tileA, V tileX, V row_start, int lane) {
-    SplitRecord* rec = mine + k * stride;
-    V carry_in = row_start;  // the state entering tile 0
-    if (k > 0) {
-        if (lane == 0) {
-            publish(rec->a, tileA);
-            publish(rec->x, tileX);
-        }
-        const unsigned long long limit = header->wait_limit;
-        V accA = vone<V>(), accX = vzero<V>();  // aggregate of the tiles nearer than the current window
-        bool done = false;
-        for (int64_t base = k - 1; base >= 0 && !done; base -= 64) {
-            const int64_t q = base - lane;
-            const bool active = q >= 0;
-            // 0 nothing seen, 1 aggregate in (A, X), 2 inclusive state in X
-            int seen = 0;
-            V A = vone<V>(), X = vzero<V>();
-            if (active) {
-                SplitRecord* prev = mine + q * stride;
-                unsigned long long waited = 0, last = __builtin_amdgcn_s_memrealtime();
-                for (;;) {
-                    V P, Aq, Xq;
-                    if (peek(prev->p, P)) {
-                        X = P;
-                        seen = 2;
-                        break;
-                    }
-                    const bool has_a = peek(prev->a, Aq);
-                    const bool has_x = peek(prev->x, Xq);
-                    if (has_a && has_x) {
-                        A = Aq;
-                        X = Xq;
-                        seen = 1;
-                        break;
-                    }
-                    const unsigned long long now = __builtin_amdgcn_s_memrealtime();
-                    waited += now - last < kWaitStepCap ? now - last : kWaitStepCap;
-                    last = now;
-                    if (waited > limit) break;
-                    __builtin_amdgcn_s_sleep(1);
-                }
-            }
-            const int n_active = base + 1 < 64 ? (int)(base + 1) : 64;
-            const unsigned long long inclusive = __ballot(active && seen == 2);
-            const unsigned long long late = __ballot(active && seen == 0);
-            // lanes [0, first) hold aggregates to fold; lane `first`, if active, holds an inclusive state
-            const int first = inclusive ? (int)__builtin_ctzll(inclusive) : n_active;
-            const unsigned long long needed = first >= 63 ? ~0ull : ((2ull << first) - 1ull);
-            if (late & needed) {
-                // a wait ran out: give up on this tile, visibly
-                if (lane == 0) atomicAdd(&header->timeouts, 1u);
-                carry_in = poison(carry_in);
-                done = true;
-            } else {
-                V wA = vone<V>(), wX = vzero<V>();  // aggregate of tiles k-1-(first-1) .. k-1 of this window
-                for (int i = first - 1; i >= 0; --i) {
-                    const V Ai = read_lane_at(A, i);
-                    const V Xi = read_lane_at(X, i);
-                    wX = vfma(wX, Ai, Xi);
-                    wA = vmul(wA, Ai);
-                }
-                // (w) o (acc): the window's tiles come before the nearer ones
-                accX = vfma(wX, accA, accX);
-                accA = vmul(wA, accA);
-                if (first < n_active) {
-                    const V P = read_lane_at(X, first);
-                    carry_in = vfma(accA, P, accX);
-                    done = true;
-                }
-            }
-        }
-        // tile 0 always publishes an inclusive state, so the walk ends there at the latest
+__device__ __forceinline__ V split_look_back(SplitHeader* header, unsigned long long limit, SplitRecord* mine,
+                                             int64_t k, int64_t ntiles, V tileA, V tileX, V row_start, int lane) {
+    SplitRecord* rec = mine + k;
+    const int64_t window = k & ~(int64_t)(kSplitWindow - 1);  // first tile of k's window
+    const int r = (int)(k - window);                          // tiles of the window before k
+    const bool closes_window = r == kSplitWindow - 1;
+    const bool has_successor = k + 1 < ntiles;
+    // the aggregate is read by the later tiles of the window, the inclusive state by the next window
+    if (lane == 0 && has_successor && !closes_window) {
+        publish(rec->a, tileA);
+        publish(rec->x, tileX);
     }
-    if (lane == 0) publish(rec->p, vfma(tileA, carry_in, tileX));
+    V carry_in = row_start;
+    if (k > 0) {
+        V A = vone<V>(), X = vzero<V>();
+        bool late = false;
+        if (lane < r) {
+            SplitRecord* prev = mine + window + lane;
+            late = !await_pair(prev->a, prev->x, A, X, limit);
+        } else if (lane == kSplitWindow - 1 && window > 0) {
+            // the state entering the window; lane 63 never holds an aggregate (r <= 63)
+            late = !await_field((mine + window - 1)->p, X, limit);
+        }
+        if (__ballot(late)) {
+            // a wait ran out: give up on this tile, visibly
+            if (lane == 0) atomicAdd(&header->timeouts, 1u);
+            carry_in = poison(carry_in);
+        } else {
+            const V entering = window > 0 ? read_lane<kSplitWindow - 1>(X) : row_start;
+            if (lane == kSplitWindow - 1) X = vzero<V>();
+            wave_scan_inclusive<false>(A, X);  // lanes past r hold the identity
+            carry_in = vfma(read_lane<63>(A), entering, read_lane<63>(X));
+        }
+    }
+    if (lane == 0 && has_successor && closes_window) publish(rec->p, vfma(tileA, carry_in, tileX));
     return carry_in;
 }
 
 // exchange_carries for a workgroup that owns a single tile of a split row: the
 // tile carry comes from split_look_back instead of the previous loop iteration.
 //
-// Wave 0 walks back over the row's earlier tiles while it holds its sub-tile in
-// registers like every other wave, and the walk needs registers of its own.
-// `set_aside()` / `take_back()` are called by wave 0 only, around the walk: the
-// kernels park their raw vectors in LDS there, which frees those registers for
-// the walk without a trip through scratch memory.
+// Wave 0 looks back while it holds its sub-tile in registers like every other
+// wave, and the look-back needs registers of its own.  `set_aside()` /
+// `take_back()` are called by wave 0 only, around it: the kernels park their raw
+// vectors in LDS there, which frees those registers without a trip through
+// scratch memory.
 template <class V, int W, int U, class SetAside, class TakeBack>
 __device__ __forceinline__ void exchange_carries_split(const V (&totA)[U], const V (&totX)[U], V& c, V* slots,
-                                                       int w, int lane, SplitHeader* header, SplitRecord* mine,
-                                                       int64_t stride, int64_t k, V row_start, SetAside set_aside,
-                                                       TakeBack take_back) {
+                                                       int w, int lane, SplitHeader* header, unsigned long long limit,
+                                                       SplitRecord* mine, int64_t k, int64_t ntiles, V row_start,
+                                                       SetAside set_aside, TakeBack take_back) {
     V TA = totA[0], TX = totX[0];
 #pragma unroll
     for (int j = 1; j < U; ++j) {
@@ -313,7 +277,7 @@ __device__ __forceinline__ void exchange_carries_split(const V (&totA)[U], const
     V* carry_slot = slots + kSlotsPerBuffer;
     if (w == 0) {  // wave-uniform
         set_aside();
-        const V carry_in = split_look_back(header, mine, stride, k, runA, runX, row_start, lane);
+        const V carry_in = split_look_back(header, limit, mine, k, ntiles, runA, runX, row_start, lane);
         if (lane == 0) *carry_slot = carry_in;
         take_back();
     }

@@ -108,15 +108,20 @@ def test_workspace_sizing_and_split_entry_validation():
     lib = _abi.load()
     buf = ctypes.create_string_buffer(256)
     p = ctypes.addressof(buf)
-    # many rows, or short rows: the plain kernels are the right choice
-    assert lib.ascan_workspace_bytes(12288, 65536, 0) == 0
+    # short rows, and many complex rows: the plain kernels are the right choice
+    assert lib.ascan_workspace_bytes(12288, 8192, 0) == 0
     assert lib.ascan_workspace_bytes(4, 4096, 0) == 0
+    assert lib.ascan_workspace_bytes(6144, 65536, 3) == 0
+    # rows of 64 KiB and more in a real dtype are swept in memory order, however many there are
+    assert lib.ascan_workspace_bytes(12288, 65536, 0) == 128 + 12288 * (65536 // 8192 + 1) * 64
+    assert lib.ascan_workspace_bytes(12288, 32768, 1) > 0
     assert lib.ascan_workspace_bytes(4, 1 << 20, 9) == 0  # unknown dtype
     assert lib.ascan_workspace_bytes(-1, 1 << 20, 0) == 0
-    # few long rows: header (64 bytes) + one 64-byte ticket line per row
+    # few long rows: header (64 bytes) + the ticket line (64 bytes)
     # + one 64-byte record per (row, smallest tile)
     nbytes = lib.ascan_workspace_bytes(4, 1 << 20, 0)
-    assert nbytes == 64 + 4 * 64 + 4 * ((1 << 20) // 8192 + 1) * 64
+    assert nbytes == 64 + 64 + 4 * ((1 << 20) // 8192 + 1) * 64
+    assert lib.ascan_workspace_bytes(4, 1 << 20, 3) > 0  # complex rows too, when they are few
     assert lib.ascan_workspace_bytes(4, 1 << 20, 1) < nbytes  # 16-bit tiles hold more elements
     # the split entry points validate like the plain ones, before touching the GPU
     assert lib.ascan_forward_split(p, p, p, 1, 4, 7, 0, None, 0, None) == 3
