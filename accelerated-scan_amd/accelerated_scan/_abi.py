@@ -13,7 +13,7 @@ from pathlib import Path
 
 import torch
 
-ABI_VERSION = 9
+ABI_VERSION = 10
 
 # ascan_gate codes of include/ascan.h
 GATE_IDENTITY, GATE_SIGMOID, GATE_SIGMOID_LERP, GATE_EXP, GATE_EXP_NORM = 0, 1, 2, 3, 4
@@ -61,6 +61,7 @@ _SIGNATURES = {
         [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p,
          ctypes.c_int64, ctypes.c_int64, ctypes.c_int, ctypes.c_int, ctypes.c_void_p],
     ),
+    "ascan_static_workspace_timeouts": (ctypes.c_int, [ctypes.POINTER(ctypes.c_uint), ctypes.c_void_p]),
     "ascan_forward_from": (
         ctypes.c_int,
         [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p,
@@ -207,6 +208,19 @@ def _launch(device: torch.device, fn, *args) -> None:
         check(status)
 
 
+# ASCAN_DEBUG_SPLIT=1: after every call that was given a table, wait for the device and
+# raise if a wait for an earlier tile ran out (such a tile holds NaN in the output).
+_DEBUG_SPLIT = os.environ.get("ASCAN_DEBUG_SPLIT", "0") not in ("", "0")
+
+
+def _after_split(workspace, what: str) -> None:
+    if _DEBUG_SPLIT and workspace is not None:
+        ran_out = workspace_timeouts(workspace)
+        if ran_out:
+            raise RuntimeError(f"accelerated_scan: {ran_out} wait(s) for an earlier tile ran out in {what}; "
+                               "the affected tiles of the output hold NaN")
+
+
 @functools.lru_cache(maxsize=1024)
 def _workspace_bytes(rows: int, seqlen: int, code: int) -> int:
     return (_lib or load()).ascan_workspace_bytes(rows, seqlen, code)
@@ -218,7 +232,9 @@ def _workspace(rows: int, seqlen: int, code: int, device: torch.device):
     nbytes = _workspace_bytes(rows, seqlen, code)
     if nbytes == 0:
         return None
-    return torch.empty(nbytes, dtype=torch.uint8, device=device)
+    # (zeroed under ASCAN_DEBUG_SPLIT: a kernel that decides against the table leaves its header as it was)
+    make = torch.zeros if _DEBUG_SPLIT else torch.empty
+    return make(nbytes, dtype=torch.uint8, device=device)
 
 
 def _check_state(state, like, name: str) -> None:
@@ -266,6 +282,7 @@ def forward(gates, tokens, out, reverse: bool, workspace=None, initial=None) -> 
     else:
         _launch(tokens.device, lib.ascan_forward_split, gates.data_ptr(), tokens.data_ptr(), out.data_ptr(), rows,
                 seqlen, code, 1 if reverse else 0, workspace.data_ptr(), workspace.numel())
+    _after_split(workspace, "forward")
 
 
 def backward(gates, states, grad_out, d_gates, d_tokens, workspace=None, initial=None, d_initial=None,
@@ -296,6 +313,7 @@ def backward(gates, states, grad_out, d_gates, d_tokens, workspace=None, initial
     else:
         _launch(gates.device, lib.ascan_backward_split, gates.data_ptr(), states.data_ptr(), grad_out.data_ptr(),
                 d_gates.data_ptr(), d_tokens.data_ptr(), rows, seqlen, code, workspace.data_ptr(), workspace.numel())
+    _after_split(workspace, "backward")
 
 
 def forward_gated(gate_inputs, tokens, out, gate: int, workspace=None, initial=None) -> None:
@@ -308,6 +326,7 @@ def forward_gated(gate_inputs, tokens, out, gate: int, workspace=None, initial=N
     _launch(tokens.device, lib.ascan_forward_gated, gate_inputs.data_ptr(), tokens.data_ptr(), _ptr(initial),
             out.data_ptr(), rows, seqlen, code, gate, _ptr(workspace),
             workspace.numel() if workspace is not None else 0)
+    _after_split(workspace, "forward_gated")
 
 
 def backward_gated(gate_inputs, states, grad_out, d_gate_inputs, d_tokens, gate: int, workspace=None,
@@ -322,6 +341,7 @@ def backward_gated(gate_inputs, states, grad_out, d_gate_inputs, d_tokens, gate:
     _launch(gate_inputs.device, lib.ascan_backward_gated, gate_inputs.data_ptr(), states.data_ptr(), _ptr(initial),
             grad_out.data_ptr(), d_gate_inputs.data_ptr(), d_tokens.data_ptr(), _ptr(d_initial), rows, seqlen, code,
             gate, _ptr(workspace), workspace.numel() if workspace is not None else 0)
+    _after_split(workspace, "backward_gated")
 
 
 def backward_gated_values(gate_inputs, values, states, grad_out, d_gate_inputs, d_values, gate: int, workspace=None,
@@ -340,6 +360,7 @@ def backward_gated_values(gate_inputs, values, states, grad_out, d_gate_inputs, 
             states.data_ptr(), _ptr(initial), grad_out.data_ptr(), d_gate_inputs.data_ptr(), d_values.data_ptr(),
             _ptr(d_initial), rows, seqlen, code, gate, _ptr(workspace),
             workspace.numel() if workspace is not None else 0)
+    _after_split(workspace, "backward_gated_values")
 
 
 def backward_lerp(gate_inputs, values, states, grad_out, d_gate_inputs, d_values, workspace=None,
@@ -354,6 +375,7 @@ def backward_lerp(gate_inputs, values, states, grad_out, d_gate_inputs, d_values
     _launch(gate_inputs.device, lib.ascan_backward_lerp, gate_inputs.data_ptr(), values.data_ptr(), states.data_ptr(),
             _ptr(initial), grad_out.data_ptr(), d_gate_inputs.data_ptr(), d_values.data_ptr(), _ptr(d_initial), rows,
             seqlen, code, _ptr(workspace), workspace.numel() if workspace is not None else 0)
+    _after_split(workspace, "backward_lerp")
 
 
 def workspace_timeouts(workspace) -> int:

@@ -177,7 +177,8 @@ def exp_norm_scan(log_gates, values, initial=None):
 
     Arguments:
         log_gates (torch.Tensor): shape (B, C, T), contiguous; fp32, bf16 or fp16; logarithms of the
-            gates, strictly negative (at 0 the input scale vanishes and its derivative is unbounded).
+            gates, negative (at 0 the input scale vanishes and its derivative is unbounded; the backward pass
+            takes that derivative as 0 there, so a stored 0 gives finite gradients).
         values (torch.Tensor): shape (B, C, T), contiguous, same dtype.
         initial (torch.Tensor, optional): shape (B, C), the state ``x[-1]`` (zero if absent).
 

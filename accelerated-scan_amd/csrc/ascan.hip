@@ -266,6 +266,21 @@ int ascan_forward_split_static(const void* gates, const void* tokens, void* out,
     return forward_checked(gates, tokens, out, nullptr, rows, seqlen, dtype, reverse, ASCAN_GATE_IDENTITY, ws, stream);
 }
 
+int ascan_static_workspace_timeouts(unsigned int* count, void* stream) {
+    if (count == nullptr) return ASCAN_ERR_NULL_POINTER;
+    void* table = static_workspace();
+    if (table == nullptr) return ASCAN_ERR_LAUNCH;
+    SplitHeader header;
+    hipError_t e = hipStreamSynchronize(static_cast<hipStream_t>(stream));
+    if (e == hipSuccess) e = hipMemcpy(&header, table, sizeof(header), hipMemcpyDeviceToHost);
+    if (e != hipSuccess) {
+        g_last_hip_error = (int)e;
+        return ASCAN_ERR_LAUNCH;
+    }
+    *count = header.timeouts;
+    return ASCAN_OK;
+}
+
 int ascan_backward_split(const void* gates, const void* states, const void* grad_out, void* d_gates,
                          void* d_tokens, int64_t rows, int64_t seqlen, int dtype, void* workspace,
                          size_t workspace_bytes, void* stream) {

@@ -356,8 +356,10 @@ __global__ void __launch_bounds__(64 * kMaxWavesPerBlock)
                     dg[e] = (gr * (before[e] - v[e])) * (a[e] * a_rest[e]);
                 } else if constexpr (ACT == kGateExpNorm) {
                     // token = b v, b = sqrt(1 - a^2):  d_v = g b;  d_z = g (a x[t-1] + v db/dz),  db/dz = -a^2 / b
+                    // (b = 0, a stored logarithm of exactly 0: the unbounded db/dz is taken as 0)
                     dt[e] = gr * a_rest[e];
-                    dg[e] = gr * (a[e] * (before[e] - v[e] * (a[e] * __builtin_amdgcn_rcpf(a_rest[e]))));
+                    const V slope = a_rest[e] == 0.0f ? 0.0f : a[e] * __builtin_amdgcn_rcpf(a_rest[e]);
+                    dg[e] = gr * (a[e] * (before[e] - v[e] * slope));
                 } else {
                     dt[e] = gr;
                     dg[e] = vmul(gr, vconj(before[e]));

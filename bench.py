@@ -27,7 +27,7 @@ token) is formed inside the kernels: the first input then holds gate pre-activat
 and the backward kernel 5 (sigmoid, exp) or 6 (lerp, exp_norm: it reads the values
 again).  --reverse times the reverse scan and its own backward kernel.  --sweep FILE runs
 the reference's benchmark grid, one JSON line per point into FILE and the same
-points as a Markdown table into FILE.md and the (8,1536,T) grid as FILE.csv (the
+points as a Markdown table into FILE.md and the (8,1536,T) grid as FILE.<direction>.csv (the
 single summary line is still printed).  The reference's max-abs-error table is asserted by
 tests/test_precision_gpu.py.
 """
@@ -214,14 +214,20 @@ def load_stream_probe():
     lib.stream_probe_launch.restype = ctypes.c_int
     lib.stream_probe_launch.argtypes = ([ctypes.c_void_p] * 5 + [ctypes.c_int64] * 2 + [ctypes.c_int] * 5
                                         + [ctypes.c_uint, ctypes.c_void_p])
+    lib.stream_probe_sweep.restype = ctypes.c_int
+    lib.stream_probe_sweep.argtypes = ([ctypes.c_void_p] * 5 + [ctypes.c_int64] * 2 + [ctypes.c_int] * 4
+                                       + [ctypes.c_void_p, ctypes.c_size_t, ctypes.c_uint, ctypes.c_void_p])
     return lib
 
 
 def device_ceiling(shape, dtype_name, bufs, steps=12, warmup=4):
     """Streams the workload's own buffers (`bufs`: the buffer sets of run_workload) with kernels that do no arithmetic:
     the backward scan's mix (3 tensors read, 2 written) and the forward scan's
-    (2 read, 1 written), as a linear sweep and as one workgroup walking each
-    row.  Returns GB/s per variant; run outside the scan's timed region."""
+    (2 read, 1 written), as a linear sweep of fresh workgroups, as one workgroup
+    walking each row, and as a sweep in 64 KiB tiles that persistent workgroups take
+    by ticket -- without and with the wait of a scan that passes carries from tile
+    to tile through global memory.  Returns GB/s per variant; run outside the scan's
+    timed region."""
     import torch
 
     probe = load_stream_probe()
@@ -236,7 +242,10 @@ def device_ceiling(shape, dtype_name, bufs, steps=12, warmup=4):
            "what": "kernels without arithmetic on the same buffers, 16-byte nontemporal accesses "
                    "(tests/native/stream_probe.hip): linear = consecutive workgroups move consecutive 16 KiB; "
                    "row_walk = one 1024-thread workgroup per row in 64 KiB tiles with one barrier per tile, "
-                   "the scan kernels' own order"}
+                   "the order of the scan kernels that own whole rows; ticket_sweep = one persistent 1024-thread "
+                   "workgroup per compute unit takes 64 KiB tiles in memory order from a ticket counter, the order of "
+                   "the scan kernels that pass carries through a table; ticket_sweep_carry_wait = the same, each "
+                   "tile storing only after its row's earlier tiles have flagged their loads as landed"}
     for name, reads, writes, pattern in (("3R2W_linear", 3, 2, 0), ("3R2W_row_walk", 3, 2, 2),
                                          ("2R1W_linear", 2, 1, 0), ("2R1W_row_walk", 2, 1, 2)):
         def fn():
@@ -251,6 +260,26 @@ def device_ceiling(shape, dtype_name, bufs, steps=12, warmup=4):
             continue
         ms = time_call(fn, steps, warmup, min_ms=30.0)
         out[name] = (reads + writes) * nbytes / ms / 1e6
+    tile = 64 * 1024
+    if row_bytes % tile == 0 and row_bytes // tile <= 64 and rows * (row_bytes // tile) < 2 ** 31:
+        table = torch.zeros(64 + rows * (row_bytes // tile) * 64, dtype=torch.uint8, device=bufs[0][0].device)
+        grid = torch.cuda.get_device_properties(bufs[0][0].device).multi_processor_count
+        for name, reads, writes, chain in (("3R2W_ticket_sweep", 3, 2, 0), ("3R2W_ticket_sweep_carry_wait", 3, 2, 1),
+                                           ("2R1W_ticket_sweep", 2, 1, 0), ("2R1W_ticket_sweep_carry_wait", 2, 1, 1)):
+            def fn():
+                g, x, d, states, d_gates, d_tokens = bufs[turn[0] % len(bufs)]
+                turn[0] += 1
+                table.zero_()  # the scan's own launches clear their table too
+                rc = probe.stream_probe_sweep(g.data_ptr(), states.data_ptr(), d.data_ptr(), d_gates.data_ptr(),
+                                              d_tokens.data_ptr(), rows, row_bytes, reads, writes, chain, 4,
+                                              table.data_ptr(), table.numel(), grid, stream)
+                if rc != 0:
+                    raise RuntimeError(f"stream probe: status {rc}")
+            ms = time_call(fn, steps, warmup, min_ms=30.0)
+            out[name] = (reads + writes) * nbytes / ms / 1e6
+        torch.cuda.synchronize()
+        if int(table[8:12].view(torch.int32).item()) != 0:
+            raise RuntimeError("stream probe: a wait of the ticket sweep ran out")
     return out
 
 
@@ -324,6 +353,11 @@ def run_sweep(path, steps, warmup):
                     x = tokens.clone().requires_grad_(True)
                     ms = time_call(lambda: torch.autograd.grad(warp_scan(g, x), (g, x), grad_out), steps, warmup, min_ms)
                     rec["train_ms"], rec["train_GBps"] = ms, 8 * nbytes / ms / 1e6
+                    del g, x
+                # forward + backward captured once into a HIP graph and replayed: what a caller reaches who
+                # takes the per-call host cost (Python, autograd, allocation) out of the loop
+                ms = time_call(graphed_step(gates, tokens, grad_out, out, d_gates, d_tokens), steps, warmup, min_ms)
+                rec["train_graph_ms"], rec["train_graph_GBps"] = ms, 8 * nbytes / ms / 1e6
                 emit(rec)
                 del gates, tokens, grad_out, out, d_gates, d_tokens
 
@@ -345,20 +379,54 @@ def run_sweep(path, steps, warmup):
         rec["train_real_inputs_ms"] = ms
         emit(rec)
     write_sweep_markdown(records, str(path) + ".md", steps, warmup)
-    write_sweep_csv(records, str(path) + ".csv")
+    write_sweep_csv(records, str(path))
 
 
-def write_sweep_csv(records, path):
-    """The (8, 1536, T) grid as CSV, one row per dtype and T (the reference's
-    harness saves one CSV per direction with a SEQUENCE_LENGTH column,
-    tests/bench.py:100-115 of the reference); empty cells were not measured."""
-    columns = ("forward_ms", "reverse_ms", "backward_ms", "train_ms")
-    with open(path, "w") as f:
-        f.write("dtype,SEQUENCE_LENGTH," + ",".join(columns) + "\n")
-        for rec in records:
-            if rec["dtype"] != "c64":
-                f.write(f"{rec['dtype']},{rec['shape'][2]}," + ",".join(
-                    f"{rec[c]:.6f}" if c in rec else "" for c in columns) + "\n")
+def graphed_step(gates, tokens, grad_out, out, d_gates, d_tokens):
+    """Captures one forward + backward through the C ABI (outputs and tables allocated
+    beforehand) into a HIP graph; returns the function that replays it."""
+    import torch
+
+    from accelerated_scan import _abi
+
+    rows, seqlen, code = _abi._problem(gates, tokens)
+    nbytes = _abi.load().ascan_workspace_bytes(rows, seqlen, code)
+    tables = [torch.empty(nbytes, dtype=torch.uint8, device=gates.device) if nbytes else None for _ in range(2)]
+
+    def step():
+        _abi.forward(gates, tokens, out, False, workspace=tables[0])
+        _abi.backward(gates, out, grad_out, d_gates, d_tokens, workspace=tables[1])
+
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        step()  # warm-up outside capture
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        step()
+    return graph.replay
+
+
+SWEEP_DIRECTIONS = ("forward", "reverse", "backward", "train", "train_graph")
+
+
+def write_sweep_csv(records, stem):
+    """The (8, 1536, T) grid as CSV, one file per direction (STEM.<direction>.csv) with a
+    SEQUENCE_LENGTH column and one column of milliseconds per dtype, as the reference's
+    harness saves them (tests/bench.py:100-115 of the reference); empty cells were not measured."""
+    dtypes = [dt for dt in ("fp32", "bf16") if any(r["dtype"] == dt for r in records)]
+    lengths = sorted({r["shape"][2] for r in records if r["dtype"] in dtypes})
+    for direction in SWEEP_DIRECTIONS:
+        with open(f"{stem}.{direction}.csv", "w") as f:
+            f.write("SEQUENCE_LENGTH," + ",".join(f"{dt}_ms" for dt in dtypes) + "\n")
+            for T in lengths:
+                cells = []
+                for dt in dtypes:
+                    rec = next((r for r in records if r["dtype"] == dt and r["shape"][2] == T), {})
+                    cells.append(f"{rec[direction + '_ms']:.6f}" if direction + "_ms" in rec else "")
+                f.write(f"{T}," + ",".join(cells) + "\n")
 
 
 def write_sweep_markdown(records, path, steps, warmup):
@@ -383,13 +451,15 @@ def write_sweep_markdown(records, path, steps, warmup):
                 f"least {steps} calls and 40 ms after at least {warmup} calls and 20 ms of warm-up, HIP events; one set of buffers per point, so tensors up to a few hundred MB "
                 "see some Infinity Cache hits). Cells: ms per call (algorithmic TB/s). forward / reverse / backward "
                 "are kernel calls through the C ABI; train = autograd forward + backward of `warp.scan`, "
-                "allocation included.\n")
+                "allocation included; train (graph) = forward + backward through the C ABI captured once into a "
+                "HIP graph and replayed, i.e. without the per-call host cost.\n")
         for dt in ("fp32", "bf16"):
-            f.write(f"\n## {dt}, shape (8, 1536, T)\n\n| T | forward | reverse | backward | train |\n|---|---|---|---|---|\n")
+            f.write(f"\n## {dt}, shape (8, 1536, T)\n\n| T | forward | reverse | backward | train | train (graph) |\n"
+                    "|---|---|---|---|---|---|\n")
             for rec in records:
                 if rec["dtype"] == dt:
                     f.write(f"| {rec['shape'][2]} | {cell(rec, 'forward')} | {cell(rec, 'reverse')} | "
-                            f"{cell(rec, 'backward')} | {cell(rec, 'train')} |\n")
+                            f"{cell(rec, 'backward')} | {cell(rec, 'train')} | {cell(rec, 'train_graph')} |\n")
         for rec in records:
             if rec["dtype"] == "c64":
                 f.write(f"\n## complex64, shape {tuple(rec['shape'])} (tests/bench_complex.py:79-90 of the reference)\n\n"

@@ -49,7 +49,17 @@
  *     blocks, or equal storage offsets) take the vectorised kernels for any
  *     seqlen, at full speed when they also agree modulo 128; buffers at
  *     different offsets inside a 16-byte block take element-wise kernels with
- *     the same arithmetic;
+ *     the same arithmetic.  The vectorised kernels move aligned 16-byte blocks
+ *     only: where a tensor does not begin or end on a 16-byte boundary they READ
+ *     the whole block that straddles its first or last element, i.e. up to 15
+ *     bytes outside the tensor's range (inside the same 16-byte block, so inside
+ *     the same page and allocation granule), and discard them; they never write
+ *     outside the range.  A caller that sub-allocates tensors at odd offsets while
+ *     another stream writes the neighbouring bytes will see those reads in a race
+ *     detector; the results do not depend on them;
+ *   - results are reproducible: the same call on the same data gives the same
+ *     bits, run to run and whatever else the GPU is doing, on every path
+ *     (including rows split over workgroups, see below);
  *   - errors are reported by return code, never by abort or exception.
  */
 #ifndef ASCAN_H_
@@ -62,7 +72,7 @@
 extern "C" {
 #endif
 
-#define ASCAN_ABI_VERSION 9
+#define ASCAN_ABI_VERSION 10
 
 /* Marks the exported entry points (the library is built with hidden visibility). */
 #define ASCAN_API __attribute__((visibility("default")))
@@ -118,8 +128,10 @@ enum ascan_gate {
      * The same gate, and the second input holds values v rather than tokens:
      * token = sqrt(1 - gate^2) * v, i.e. x[t] = a * x[t-1] + sqrt(1 - a^2) * v[t]
      * with a = exp(stored), the update of RG-LRU / Hawk-style layers (the scale
-     * keeps the state's variance at that of the values).  Stored values must be
-     * negative: at 0 the scale is 0 and its derivative unbounded.  Forward:
+     * keeps the state's variance at that of the values).  Stored values should be
+     * negative: at 0 the scale is 0 and its derivative unbounded; the backward
+     * pass takes the derivative of the scale as 0 there (a stored +0 or -0, e.g. a
+     * 16-bit logarithm that underflowed), so gradients stay finite.  Forward:
      * ascan_forward_gated; backward: ascan_backward_gated_values (it needs v).
      * float32, bfloat16, float16.
      */
@@ -150,17 +162,25 @@ ASCAN_API int ascan_backward(const void* gates, const void* states, const void* 
                    void* stream);
 
 /*
- * Split rows.  With few rows (B*D up to about half the number of compute
- * units) and long sequences the plain entry points leave most of the GPU idle:
- * they give each row one workgroup.  The *_split entry points hand the tiles of
- * every row to separate workgroups that pass the running state through a small
- * table in caller-provided device memory (one pass over the data, no extra
- * traffic).  They have no counterpart in the reference, whose kernels give one
- * thread block to each sequence (warp.cuh:279; scalar.py:98; complex.py:174).
+ * Rows split over workgroups, with a table in caller-provided memory.  The
+ * plain entry points give every row to one workgroup that walks it from end
+ * to end.  That leaves most of the GPU idle when there are few rows, and for
+ * long rows it is not the fastest order either: with thousands of rows being
+ * walked side by side the memory system sees as many streams.  Given a
+ * workspace, the *_split entry points (and every entry point below that takes
+ * one) instead hand out the 16-wave tiles of all rows in memory order, one
+ * tile at a time to whichever resident workgroup is free, and pass the running
+ * state from tile to tile through a small table in the workspace: one pass over
+ * the data, no extra traffic.  Measured on MI355X, fp32 (8, 1536, 65536) forward +
+ * backward: 4.40 ms without a workspace, 3.90 ms with one.  They have no
+ * counterpart in the reference, whose kernels give one thread block to each
+ * sequence (warp.cuh:279; scalar.py:98; complex.py:174).
  *
- *   ascan_workspace_bytes  size of the table for a problem, or 0 when splitting
- *                          would not help (then the *_split calls behave exactly
- *                          like the plain ones and ignore the workspace);
+ *   ascan_workspace_bytes  size of the table for a problem, or 0 when no kernel
+ *                          would use one (short rows; many complex64 rows): then
+ *                          the calls behave exactly like the plain ones and
+ *                          ignore the workspace.  Otherwise 128 bytes plus 64
+ *                          bytes per tile, a few MB at most for tensors of GBs;
  *   workspace              device memory, 64-byte aligned, at least that many
  *                          bytes, not shared with another call that may run at
  *                          the same time; contents on entry do not matter (it
@@ -169,15 +189,22 @@ ASCAN_API int ascan_backward(const void* gates, const void* states, const void* 
  *                          has completed.  NULL or a too-small buffer selects
  *                          the plain path.
  *
- * A workgroup waits for the workgroups of earlier tiles.  Tiles are handed out
- * in order by a ticket counter per row, so the owner of a tile that is waited
+ * A workgroup waits for the workgroups of earlier tiles of its row.  Tiles are
+ * handed out in order by one ticket counter, and a workgroup starts on its tile
+ * as soon as it has drawn the ticket, so the owner of a tile that is waited
  * for has always started already: progress does not depend on how much of the
  * GPU the call gets, and concurrent calls (each with its own workspace) are
- * fine.  Every wait is bounded all the same (2 s of running time by default);
- * a wait that runs out writes NaN into the affected tile and is counted: copy
+ * fine.  What a tile receives is the state entering its window of 64 tiles
+ * folded with the aggregates of the window's earlier tiles in one fixed order,
+ * whichever of them were published first: results are the same bits run to run
+ * (they differ from the plain path's by rounding, the association being another).
+ * Every wait is bounded all the same (2 s of running time by default; the
+ * environment variable ASCAN_SPLIT_WAIT_US, read once, sets another limit); a
+ * wait that runs out writes NaN into the affected tile and is counted: copy
  * the first 64 bytes of the workspace to the host after the stream has
  * completed and pass them to ascan_workspace_timeouts (0 = all waits were
- * served).
+ * served).  NaN in whole tiles of an output whose inputs are finite means that
+ * a wait ran out.
  */
 ASCAN_API size_t ascan_workspace_bytes(int64_t rows, int64_t seqlen, int dtype);
 
@@ -208,13 +235,24 @@ ASCAN_API unsigned int ascan_workspace_timeouts(const void* workspace_header_cop
  *   - all calls on one GPU share that GPU's array (it is cleared by a small
  *     kernel on `stream` at the start of each call): two calls that may run at
  *     the same time on one GPU -- different streams, or graph branches -- race
- *     on it.  Use ascan_forward_split with separate workspaces for those.
+ *     on it.  Use ascan_forward_split with separate workspaces for those;
+ *   - the first use on a GPU looks the array's address up (hipGetSymbolAddress,
+ *     which loads the library's code object on that GPU): make it outside any
+ *     stream capture -- a first call of ascan_static_workspace_timeouts does.
+ *
+ * ascan_static_workspace_timeouts waits for `stream` and stores in *count the
+ * number of waits that ran out in the last ascan_forward_split_static call on the
+ * current GPU that used the table (see ascan_workspace_timeouts; whatever the
+ * array holds before the first such call counts as 0 only if it is zero, which
+ * it is at load time).  Not for use under capture.
  */
 #define ASCAN_STATIC_WORKSPACE_BYTES (4 * 1024 * 1024)
 
 ASCAN_API int ascan_forward_split_static(const void* gates, const void* tokens, void* out,
                                int64_t rows, int64_t seqlen, int dtype, int reverse,
                                void* stream);
+
+ASCAN_API int ascan_static_workspace_timeouts(unsigned int* count, void* stream);
 
 /*
  * Scans that start from a given state, for callers that process a long
@@ -329,7 +367,9 @@ ASCAN_API int ascan_backward_lerp(const void* gate_inputs, const void* values, c
  *
  * in one fused reverse-time pass (4 tensors read, 2 written).  1 - a^2 is
  * evaluated without cancellation for gates close to 1 (a series in
- * 2 * gate_inputs above -0.25).  Any other gate: ASCAN_ERR_BAD_ACTIVATION.
+ * 2 * gate_inputs where that is above -1/16); where b is exactly 0
+ * (gate_inputs = 0) the term values * a^2 / b is taken as 0.  Any other gate:
+ * ASCAN_ERR_BAD_ACTIVATION.
  * No counterpart in the reference.
  */
 ASCAN_API int ascan_backward_gated_values(const void* gate_inputs, const void* values, const void* states,

@@ -16,7 +16,15 @@
 //   pattern 4  row walk by `row_step` persistent workgroups: workgroup b walks
 //              rows b, b + row_step, ... (fewer rows in flight than compute units
 //              when row_step is below their number).
-// `blocks_per_wave` in {1, 2, 4, 8} sets the tile of patterns 1-3: that many KiB
+//   pattern 5  ticket sweep (stream_probe_sweep): persistent 1024-thread workgroups
+//              take tiles in memory order from one ticket counter, so that the
+//              stretch of memory in flight stays compact however long the rows are;
+//   pattern 6  ticket sweep in which a tile may store only after the earlier tiles
+//              of its row have announced that their loads have landed -- one
+//              64-byte record per tile, lane i of wave 0 reads record n-1-i with
+//              device-scope loads -- i.e. with the dependency (and the idle round
+//              trip) of a scan whose tiles pass carries through global memory.
+// `blocks_per_wave` in {1, 2, 4, 8} sets the tile of patterns 1-3 and 5-6: that many KiB
 // per wave, 16 times as much per workgroup (the scan kernels: 4, 64 KiB tiles).
 // `row_step` > 1 (patterns 1, 2) hands consecutive workgroups rows that far apart.
 // `lds_bytes` of dynamic LDS are requested per workgroup (nothing uses them):
@@ -90,6 +98,75 @@ __global__ void __launch_bounds__(kThreads) stream_probe_rows(Tensors t, int64_t
     }
 }
 
+// Patterns 5 and 6.  table: [0] the ticket counter, then one 64-byte record per tile from
+// byte 64 on; cleared by the caller before every launch.  Every wait is bounded; waits that
+// ran out are counted in table word 1.
+template <int NR, int NW, bool CHAIN, int BPW>
+__global__ void __launch_bounds__(kThreads) stream_probe_tickets(Tensors t, int64_t total_tiles, int tiles_per_row,
+                                                                unsigned long long* table) {
+    __shared__ long long mailbox;
+    __shared__ unsigned int carry_word;
+    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    constexpr int64_t kTileVec = tile_bytes(BPW) / 16;
+    unsigned long long* flags = table + 8;
+    for (;;) {
+        if (threadIdx.x == 0) {
+            const long long n = (long long)__hip_atomic_fetch_add(table, 1ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            mailbox = n < total_tiles ? n : -1;
+        }
+        __syncthreads();
+        const long long tile = __builtin_amdgcn_readfirstlane((int)mailbox);
+        __syncthreads();
+        if (tile < 0) break;
+        const int64_t base = tile * kTileVec + (int64_t)wave * (64 * BPW) + lane;
+        u32x4_t s[BPW];
+#pragma unroll
+        for (int j = 0; j < BPW; ++j) {
+            s[j] = u32x4_t{1u, 2u, 3u, 4u};
+#pragma unroll
+            for (int r = 0; r < NR; ++r) s[j] += __builtin_nontemporal_load(t.in[r] + base + j * 64);
+        }
+        unsigned int c = 0;
+        if constexpr (CHAIN) {
+            __syncthreads();  // everybody's loads have landed (the sums above consumed them)
+            if (wave == 0) {
+                if (lane == 0) {
+                    __hip_atomic_store(flags + tile * 8, (unsigned long long)(tile + 1), __ATOMIC_RELAXED,
+                                       __HIP_MEMORY_SCOPE_AGENT);
+                }
+                const int k = (int)(tile % tiles_per_row);
+                unsigned int got = 0;
+                if (lane < k) {
+                    const unsigned long long want = (unsigned long long)(tile - lane);  // record tile-1-lane holds tile-lane
+                    for (unsigned spins = 0;; ++spins) {
+                        const unsigned long long v = __hip_atomic_load(flags + (tile - 1 - lane) * 8, __ATOMIC_RELAXED,
+                                                                       __HIP_MEMORY_SCOPE_AGENT);
+                        if (v == want) {
+                            got = (unsigned int)v;
+                            break;
+                        }
+                        if (spins > 4000000u) {
+                            atomicAdd(reinterpret_cast<unsigned int*>(table + 1), 1u);
+                            break;
+                        }
+                        __builtin_amdgcn_s_sleep(1);
+                    }
+                }
+                for (int o = 32; o > 0; o >>= 1) got += __shfl_xor(got, o);
+                if (lane == 0) carry_word = got;
+            }
+            __syncthreads();
+            c = carry_word;
+        }
+#pragma unroll
+        for (int j = 0; j < BPW; ++j) {
+#pragma unroll
+            for (int w = 0; w < NW; ++w) __builtin_nontemporal_store(s[j] + (unsigned)w + c, t.out[w] + base + j * 64);
+            if constexpr (NW == 0) keep(s[j], t.out[0] + base + j * 64);
+        }
+    }
+}
+
 template <class K>
 hipError_t allow_lds(K kernel, unsigned lds_bytes) {
     if (lds_bytes <= 64u * 1024u) return hipSuccess;
@@ -138,7 +215,53 @@ hipError_t launch(const Tensors& t, int64_t rows, int64_t row_bytes, int pattern
     }
 }
 
+template <int NR, int NW>
+hipError_t launch_tickets(const Tensors& t, int64_t total_tiles, int tiles_per_row, bool chain, int bpw,
+                          unsigned long long* table, unsigned grid, hipStream_t stream) {
+    auto go = [&](auto kernel) {
+        hipLaunchKernelGGL(kernel, dim3(grid), dim3(kThreads), 0, stream, t, total_tiles, tiles_per_row, table);
+        return hipGetLastError();
+    };
+    if (bpw == 2) return chain ? go(stream_probe_tickets<NR, NW, true, 2>) : go(stream_probe_tickets<NR, NW, false, 2>);
+    return chain ? go(stream_probe_tickets<NR, NW, true, 4>) : go(stream_probe_tickets<NR, NW, false, 4>);
+}
+
 }  // namespace
+
+// Patterns 5 (chain = 0) and 6 (chain = 1): `grid` persistent workgroups sweep rows x row_bytes
+// bytes of every tensor in tiles of 16 * blocks_per_wave KiB (blocks_per_wave in {2, 4}).  `table`
+// holds 64 bytes plus 64 bytes per tile and must be zero when the launch starts.  Returns 0, -1
+// for arguments the kernels do not cover, or a hipError_t.
+extern "C" __attribute__((visibility("default"))) int stream_probe_sweep(
+    const void* in0, const void* in1, const void* in2, void* out0, void* out1, int64_t rows, int64_t row_bytes,
+    int reads, int writes, int chain, int blocks_per_wave, void* table, size_t table_bytes, unsigned grid,
+    void* stream) {
+    if (rows <= 0 || row_bytes <= 0 || grid == 0 || (blocks_per_wave != 2 && blocks_per_wave != 4)) return -1;
+    const int64_t tile = tile_bytes(blocks_per_wave);
+    if (row_bytes % tile != 0 || row_bytes / tile > 64) return -1;
+    const int64_t total_tiles = rows * (row_bytes / tile);
+    if (total_tiles > 2147483647LL || !table || reinterpret_cast<uintptr_t>(table) % 64 ||
+        table_bytes < 64 + (size_t)total_tiles * 64) {
+        return -1;
+    }
+    const void* ins[3] = {in0, in1, in2};
+    void* outs[2] = {out0, out1};
+    for (int r = 0; r < reads; ++r)
+        if (r >= 3 || !ins[r] || reinterpret_cast<uintptr_t>(ins[r]) % 16) return -1;
+    for (int w = 0; w < (writes > 0 ? writes : 1); ++w)
+        if (w >= 2 || !outs[w] || reinterpret_cast<uintptr_t>(outs[w]) % 16) return -1;
+    Tensors t;
+    for (int r = 0; r < 3; ++r) t.in[r] = static_cast<const u32x4_t*>(ins[r]);
+    for (int w = 0; w < 2; ++w) t.out[w] = static_cast<u32x4_t*>(outs[w]);
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    auto* words = static_cast<unsigned long long*>(table);
+    const int per_row = (int)(row_bytes / tile);
+    switch (reads * 10 + writes) {
+        case 32: return (int)launch_tickets<3, 2>(t, total_tiles, per_row, chain != 0, blocks_per_wave, words, grid, s);
+        case 21: return (int)launch_tickets<2, 1>(t, total_tiles, per_row, chain != 0, blocks_per_wave, words, grid, s);
+        default: return -1;
+    }
+}
 
 // Returns 0, -1 for arguments the kernels do not cover, or a hipError_t.
 extern "C" __attribute__((visibility("default"))) int stream_probe_launch(

@@ -160,6 +160,32 @@ def test_long_memory_and_short_memory_fp32():
     _run_and_compare(16, 5000, torch.float32, seed=3, what="short memory", with_initial=True, logit_mean=3.0)
 
 
+@pytest.mark.parametrize("dtype", DTYPES, ids=IDS)
+def test_log_gates_at_and_next_to_zero_give_finite_gradients(dtype):
+    """A stored logarithm of +0 or -0 (a 16-bit logarithm that underflowed, a layer that clamps at 0)
+    makes the input scale exactly 0, where its derivative is unbounded: the backward kernel takes that
+    derivative as 0, so all gradients stay finite; at the smallest negative values of the storage type
+    the scale is tiny but positive and the gradients are large and finite."""
+    from accelerated_scan import gated
+
+    tiny = torch.finfo(dtype).tiny
+    smallest = tiny * torch.finfo(dtype).eps  # the smallest subnormal
+    T = 96
+    z = torch.full((1, 3, T), -0.01, dtype=dtype)
+    z[0, 0, 5], z[0, 0, 17], z[0, 0, 40], z[0, 0, 41] = 0.0, -0.0, -smallest, -tiny
+    z[0, 1, :] = -0.0
+    z[0, 2, ::2] = -smallest
+    v = torch.randn(1, 3, T, generator=torch.Generator().manual_seed(5)).to(dtype)
+    zd, vd = z.to(DEVICE).requires_grad_(), v.to(DEVICE).requires_grad_()
+    out = gated.exp_norm_scan(zd, vd)
+    (out.float().sum() * 1e-3).backward()  # (a small loss scale: next to zero the slope is in the thousands, and fp16 ends at 65504)
+    assert torch.isfinite(out).all()
+    assert torch.isfinite(zd.grad).all() and torch.isfinite(vd.grad).all()
+    # a gate of exactly 1 lets no value in and passes the state on
+    assert torch.equal(out[0, 1], torch.zeros_like(out[0, 1]))
+    assert vd.grad[0, 1].abs().max().item() == 0.0
+
+
 def test_unit_variance_values_keep_a_unit_variance_state():
     """What the scale is for: with independent unit-variance values the stationary variance of the state is
     b^2 / (1 - a^2) = 1 for every decay."""

@@ -1005,6 +1005,29 @@ assert (timeouts == 0) == (nans == 0)
     done = subprocess.run([sys.executable, "-c", code], env=env, capture_output=True, text=True, timeout=110)
     assert done.returncode == 0, done.stdout + done.stderr
     assert "timeouts" in done.stdout
+    # ASCAN_DEBUG_SPLIT=1 turns a wait that ran out into an exception of the Python binding
+    # (with the limit at zero some wait of this shape practically always runs out; the check
+    # accepts a run in which none did)
+    debug = r"""
+import sys
+sys.path[:0] = [%r, %r]
+import torch
+from accelerated_scan import _abi
+rows, T = 4, 1 << 22
+g = torch.rand(1, rows, T, device="cuda")
+x = torch.rand(1, rows, T, device="cuda")
+out = torch.empty_like(x)
+try:
+    _abi.forward(g, x, out, False)
+    print("no wait ran out; rows_with_nan", int(torch.isnan(out).any(dim=-1).sum()))
+except RuntimeError as e:
+    assert "ran out" in str(e), e
+    print("raised:", e)
+""" % (str(ROOT), str(ROOT / "accelerated-scan_amd"))
+    done = subprocess.run([sys.executable, "-c", debug], env=dict(env, ASCAN_DEBUG_SPLIT="1"), capture_output=True,
+                          text=True, timeout=110)
+    assert done.returncode == 0, done.stdout + done.stderr
+    assert "raised:" in done.stdout or "rows_with_nan 0" in done.stdout, done.stdout
 
 
 # ---------------------------------------------------------------------------

@@ -4,10 +4,10 @@ the raw C ABI and compared with ascan_forward_split (caller-provided workspace)
 and with the fp64 recurrence, on two calls in a row, the second one smaller, so
 that the second call meets the first call's leftovers in the shared array.
 
-The look-back of a split row folds its earlier tiles in an order that depends on
-which of them have published their states yet, so two split runs agree to fp32
-rounding, not bit for bit: the bar is the fp32 one of the other GPU tests,
-2e-5 relative to the largest magnitude.
+A tile of a split row receives the state entering its window of 64 tiles folded
+with the aggregates of the window's earlier tiles in one fixed order, so the two
+entry points agree bit for bit; against the fp64 recurrence the bar is the fp32
+one of the other GPU tests, 2e-5 relative to the largest magnitude.
 """
 
 import ctypes
@@ -51,14 +51,16 @@ def _run_both(lib, gates, tokens, code, reverse):
     torch.cuda.synchronize()
     free_after = torch.cuda.mem_get_info()[0]
     assert _abi.workspace_timeouts(workspace) == 0
+    ran_out = ctypes.c_uint(99)
+    _abi.check(lib.ascan_static_workspace_timeouts(ctypes.byref(ran_out), stream))
+    assert ran_out.value == 0, "a wait of the call on the static table ran out"
     return got, want, free_before - free_after
 
 
 def _check(got, want, gates, tokens, reverse, tol):
     truth = seqscan.forward(gates.float().numpy(), tokens.float().numpy(), reverse=reverse)
     scale = max(1.0, float(np.abs(truth).max()))
-    np.testing.assert_allclose(got.float().cpu().numpy(), want.float().cpu().numpy(), rtol=tol, atol=tol * scale,
-                               err_msg="static table against caller-provided workspace")
+    assert torch.equal(got, want), "static table against caller-provided workspace"
     np.testing.assert_allclose(got.float().cpu().numpy(), truth, rtol=tol, atol=tol * scale,
                                err_msg="static table against the fp64 recurrence")
 
@@ -103,3 +105,51 @@ def test_static_table_limit_and_unsplit_shapes():
     assert lib.ascan_forward_split_static(None, x.data_ptr(), out.data_ptr(), 4, 256, 0, 0, stream) == 1
     assert lib.ascan_forward_split_static(g.data_ptr(), x.data_ptr(), out.data_ptr(), 4, 256, 9, 0, stream) == 3
     assert lib.ascan_forward_split_static(g.data_ptr(), x.data_ptr(), g.data_ptr(), 4, 256, 0, 0, stream) == 7
+
+
+def test_static_table_under_graph_capture():
+    """After one eager call (which looks the array's address up), the entry point is
+    captured into a HIP graph and replayed on new inputs; every replay must equal
+    ascan_forward_split on the same inputs."""
+    from accelerated_scan import _abi
+
+    lib = _abi.load()
+    rows, T = 3, 300000
+    nbytes = lib.ascan_workspace_bytes(rows, T, 0)
+    assert 0 < nbytes <= 4 * 1024 * 1024
+    gen = torch.Generator().manual_seed(7)
+    g = torch.empty(rows, T, device=DEVICE)
+    x = torch.empty(rows, T, device=DEVICE)
+    got, want = torch.empty_like(g), torch.empty_like(g)
+    workspace = torch.empty(nbytes, dtype=torch.uint8, device=DEVICE)
+
+    def refill():
+        g.copy_(0.9 + 0.1 * torch.rand(rows, T, generator=gen))
+        x.copy_(torch.randn(rows, T, generator=gen))
+
+    def run_static():
+        stream = torch.cuda.current_stream().cuda_stream
+        _abi.check(lib.ascan_forward_split_static(g.data_ptr(), x.data_ptr(), got.data_ptr(), rows, T, 0, 0, stream))
+
+    refill()
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        run_static()  # outside capture: the first use on this GPU
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        run_static()
+    for _ in range(3):
+        refill()
+        got.fill_(float("nan"))
+        graph.replay()
+        torch.cuda.synchronize()
+        _abi.check(lib.ascan_forward_split(g.data_ptr(), x.data_ptr(), want.data_ptr(), rows, T, 0, 0,
+                                           workspace.data_ptr(), nbytes, torch.cuda.current_stream().cuda_stream))
+        torch.cuda.synchronize()
+        assert torch.equal(got, want)
+        ran_out = ctypes.c_uint(99)
+        _abi.check(lib.ascan_static_workspace_timeouts(ctypes.byref(ran_out), None))
+        assert ran_out.value == 0
