@@ -73,8 +73,7 @@ int backward_typed(const BackwardBuffers& b, int64_t rows, int64_t T, int act, c
                    hipStream_t stream) {
     constexpr int64_t kElem = (int64_t)sizeof(typename Tr::S);
     const int64_t SUB = (int64_t)backward_blocks_of(act, Tuning<Tr>::UB) * 64 * Tr::EPV;  // regular kernels
-    constexpr int64_t SUBG = (int64_t)Tuning<Tr>::UBG * 64 * Tr::EPV;                     // kernels with masking code
-    static_assert(Tuning<Tr>::UBG <= 2 && SplitTuning<Tr>::UBG <= 2, "the interpolating gate assumes 2 KiB per wave here");
+    const int64_t SUBG = (int64_t)backward_blocks_of(act, Tuning<Tr>::UBG) * 64 * Tr::EPV;  // kernels with masking code
     const void* const state_like[] = {b.gates, b.states, b.grad_out, b.d_gates, b.values ? b.values : b.gates};
     const Lead at = find_lead<Tr>(state_like, b.d_tokens);
     const bool same_lead = at.same;
@@ -110,11 +109,11 @@ int backward_typed(const BackwardBuffers& b, int64_t rows, int64_t T, int act, c
     }
     if (same_lead && ws.ptr != nullptr) {
         const int64_t SUBS = (int64_t)backward_blocks_of(act, SplitTuning<Tr>::UB) * 64 * Tr::EPV;
-        constexpr int64_t SUBSG = (int64_t)SplitTuning<Tr>::UBG * 64 * Tr::EPV;
+        const int64_t SUBSG = (int64_t)backward_blocks_of(act, SplitTuning<Tr>::UBG) * 64 * Tr::EPV;
         const bool regular = lead == 0 && T % (SUBS * kSplitWaves) == 0;
         const int64_t tile = (regular ? SUBS : SUBSG) * kSplitWaves;
         const int64_t ntiles = host_tiles_per_row<Tr>(T, tile, regular, at);
-        if (want_split(kSweepClass<Tr>, rows, T * kElem, tile * kElem, ntiles, regular) && workspace_fits(ws, rows, ntiles)) {
+        if (want_split(kSweepClass<Tr>, rows, T * kElem, tile * kElem, ntiles, regular, act, false) && workspace_fits(ws, rows, ntiles)) {
             err = with_gate<Tr, REV>(act, [&](auto gate) {
                 constexpr int ACT = decltype(gate)::value;
                 return regular ? launch_backward_split<Tr, REV, true, ACT>(b, rows, T, at.grid, ntiles, ws, stream)

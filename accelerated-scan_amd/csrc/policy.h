@@ -39,6 +39,7 @@ template <> struct Tuning<TraitsC64RealTokens> : Tuning<TraitsC64> {};
 template <class Tr> struct SplitTuning {
     static constexpr int U = Tuning<Tr>::U, UG = Tuning<Tr>::UG, UB = Tuning<Tr>::UB, UBG = Tuning<Tr>::UBG;
 };
+template <> struct SplitTuning<TraitsF32> { static constexpr int U = 4, UG = 4, UB = 4, UBG = 2; };
 template <> struct SplitTuning<TraitsC64> { static constexpr int U = 2, UG = 2, UB = 2, UBG = 2; };
 template <> struct SplitTuning<TraitsC64RealTokens> : SplitTuning<TraitsC64> {};
 
@@ -173,9 +174,10 @@ inline int launch_status(hipError_t e) {
 // where the tiles are large and mostly full.  Measured at (8,1536,T), forward +
 // backward, % of the 8 TB/s peak, row walk -> sweep: fp32 T = 16384 72 -> 81,
 // 32768 72 -> 82, 49152 65 -> 82, 65536 73 -> 82.5, 65533 (five tiles for four
-// tiles' worth of row) 68 -> 71.5, 24576 (1.5 tiles) 71 -> 75, 20000 (1.2 tiles)
-// 74 -> 71, 8192 (half a tile) 76 -> 72; bf16 T = 32768 72 -> 81, 65536 74 -> 82,
-// but 65533, whose kernels carry masking code and take 32 KiB tiles, 71 -> 62;
+// tiles' worth of row) 68 -> 75, 24576 (1.5 tiles) 71 -> 79, 30000 and 40000 -> 78,
+// but 20000 (1.2 tiles) 76 -> 75, 17000 74 -> 68, 8192 (half a tile) 75 -> 70;
+// bf16 T = 32768 72 -> 81, 65536 74 -> 82, but 65533 and 40000, whose kernels carry
+// masking code and take 32 KiB tiles, 70 -> 63 and 72 -> 64;
 // complex64 (8,768,65536) 71 -> 70 with 64 KiB forward tiles (which spill) and 64
 // with 32 KiB ones.  A tile costs a ticket, a look at the table and three barriers,
 // about 2.4 us in which its compute unit requests nothing, whatever its size.
@@ -221,16 +223,26 @@ bool too_few_rows(int64_t rows, int64_t ntiles) {
 }
 
 // `row_bytes`: one row of states; `tile_bytes`, `ntiles`: of the kernel that would run;
-// `regular`: that kernel is the mask-free one.
-bool want_split(SweepClass c, int64_t rows, int64_t row_bytes, int64_t tile_bytes, int64_t ntiles, bool regular) {
+// `regular`: that kernel is the mask-free one; `act`: its gate.  A compute unit holds one
+// swept workgroup, so what a tile costs in arithmetic is not hidden behind another
+// workgroup's loads: the 16-bit kernels that evaluate a sigmoid (or the normalised
+// exponential gate's scale) for eight elements per vector lose when swept (bf16
+// (8,1536,65536), % of peak, whole rows -> swept: sigmoid 70 -> 67, interpolating gate
+// 72 -> 64, normalised exponential 71 -> 58; the plain exponential 73 -> 75 and the fp32
+// kernels of all gates 72 -> 78-81), and so does a forward kernel with 32 KiB tiles (the
+// normalised exponential gate's, fp32: 6.0 -> 5.3 TB/s) -- the backward kernels move five
+// or six tensors per tile and do well with 32 KiB of each.
+bool want_split(SweepClass c, int64_t rows, int64_t row_bytes, int64_t tile_bytes, int64_t ntiles, bool regular, int act,
+                bool forward) {
     if (rows > split_max_rows()) return false;
     if (too_few_rows(rows, ntiles)) return true;
     if (split_forced_min_row_bytes() > 0) return row_bytes >= split_forced_min_row_bytes();
     if (row_bytes < kSweepMinRowBytes) return false;
     if (row_bytes * 10 < ntiles * tile_bytes * 7) return false;  // tiles less than 70 % full
+    if (forward && tile_bytes < kSweepMinRowBytes) return false;
     switch (c) {
         case SweepClass::kF32: return true;
-        case SweepClass::kNarrow: return regular;
+        case SweepClass::kNarrow: return regular && (act == kGateIdentity || act == kGateExp);
         default: return false;
     }
 }

@@ -232,5 +232,5 @@ def test_wheel_carries_library_and_header(tmp_path):
     assert wheel.name.startswith("accelerated_scan-") and wheel.name.endswith("-py3-none-linux_x86_64.whl")
     names = {n.split("accelerated_scan/", 1)[1] for n in zipfile.ZipFile(wheel).namelist() if "accelerated_scan/" in n}
     assert {"libascan.so", "include/ascan.h", "__init__.py", "_abi.py", "_ops.py", "warp.py", "scalar.py",
-            "complex.py", "stateful.py"} <= names
+            "complex.py", "stateful.py", "gated.py", "ref.py"} <= names
     assert not (src / "accelerated_scan" / "include").exists()  # the header copy is temporary
