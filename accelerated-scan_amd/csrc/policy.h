@@ -260,9 +260,11 @@ size_t split_bytes(int64_t rows, int64_t ntiles) {
     return sizeof(SplitHeader) + sizeof(SplitTicket) + (size_t)rows * (size_t)ntiles * sizeof(SplitRecord);
 }
 
+// The table is usable for this launch: aligned, large enough, and the tickets fit the
+// 32 bits the kernels turn into (row, tile).
 bool workspace_fits(const Workspace& ws, int64_t rows, int64_t ntiles) {
     return ws.ptr != nullptr && (reinterpret_cast<uintptr_t>(ws.ptr) % alignof(SplitRecord)) == 0 &&
-           ws.bytes >= split_bytes(rows, ntiles);
+           rows <= 2147483647LL / ntiles && ws.bytes >= split_bytes(rows, ntiles);
 }
 
 hipError_t reset_split_table(const Workspace& ws, int64_t rows, int64_t ntiles, hipStream_t stream) {
