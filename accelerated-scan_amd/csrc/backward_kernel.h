@@ -178,6 +178,25 @@ __global__ void __launch_bounds__(64 * kMaxWavesPerBlock)
             }
         }
 
+        // (split rows: the same, and the wave still takes its part in the hand-over between tiles)
+        if constexpr (!FULL && SPLIT) {
+            if (!touches) {  // wave-uniform
+                V totA[U], totX[U];
+#pragma unroll
+                for (int j = 0; j < U; ++j) {
+                    totA[j] = vone<V>();
+                    totX[j] = vzero<V>();
+                }
+                V c;
+                exchange_carries_split<V, W, U>(
+                    totA, totX, c, slots, w, lane, split, split_wait_limit, split_records(split) + row * ntiles, k, ntiles,
+                    vzero<V>(), [] {}, [] {});
+                // the gradient scan passes through an empty sub-tile unchanged
+                if (d_initial != nullptr && k == ntiles - 1 && w == W - 1) store_start_gradient(c);  // wave-uniform
+                return;
+            }
+        }
+
         u32x4_t araw[U], draw[U], xraw[U], vraw[LERP ? U : 1];
         if (touches) {
 #pragma unroll

@@ -34,12 +34,16 @@ template <> struct Tuning<TraitsC64> { static constexpr int U = 4, UG = 4, UB = 
 template <> struct Tuning<TraitsC64RealTokens> : Tuning<TraitsC64> {};
 
 // The same four for split rows (forward regular / general, backward regular /
-// general).  The split kernels also hold the ticket walk and the look-back in
-// registers, so some of them take smaller tiles than their plain counterparts.
+// general).  A swept tile has a fixed cost (ticket, look-back, barriers), so the real
+// dtypes take 4 KiB per wave in every swept kernel, the ones with masking code included
+// (which fit their registers: wave 0 parks its vectors in LDS during the look-back, and a
+// sub-tile that holds nothing of the row is skipped); the complex kernels keep 2 KiB.
 template <class Tr> struct SplitTuning {
     static constexpr int U = Tuning<Tr>::U, UG = Tuning<Tr>::UG, UB = Tuning<Tr>::UB, UBG = Tuning<Tr>::UBG;
 };
-template <> struct SplitTuning<TraitsF32> { static constexpr int U = 4, UG = 4, UB = 4, UBG = 2; };
+template <> struct SplitTuning<TraitsF32> { static constexpr int U = 4, UG = 4, UB = 4, UBG = 4; };
+template <> struct SplitTuning<TraitsBF16> { static constexpr int U = 4, UG = 4, UB = 4, UBG = 4; };
+template <> struct SplitTuning<TraitsF16> { static constexpr int U = 4, UG = 4, UB = 4, UBG = 4; };
 template <> struct SplitTuning<TraitsC64> { static constexpr int U = 2, UG = 2, UB = 2, UBG = 2; };
 template <> struct SplitTuning<TraitsC64RealTokens> : SplitTuning<TraitsC64> {};
 
@@ -171,16 +175,17 @@ inline int launch_status(hipError_t e) {
 // swept in memory order by persistent 16-wave workgroups (split.h).  That is the only
 // way to occupy the GPU when there are fewer rows than compute units, and for long
 // rows it is faster than one workgroup walking each row whatever their number --
-// where the tiles are large and mostly full.  Measured at (8,1536,T), forward +
+// where the tiles are large and not mostly empty.  Measured at (8,1536,T), forward +
 // backward, % of the 8 TB/s peak, row walk -> sweep: fp32 T = 16384 72 -> 81,
-// 32768 72 -> 82, 49152 65 -> 82, 65536 73 -> 82.5, 65533 (five tiles for four
-// tiles' worth of row) 68 -> 75, 24576 (1.5 tiles) 71 -> 79, 30000 and 40000 -> 78,
-// but 20000 (1.2 tiles) 76 -> 75, 17000 74 -> 68, 8192 (half a tile) 75 -> 70;
-// bf16 T = 32768 72 -> 81, 65536 74 -> 82, but 65533 and 40000, whose kernels carry
-// masking code and take 32 KiB tiles, 70 -> 63 and 72 -> 64;
-// complex64 (8,768,65536) 71 -> 70 with 64 KiB forward tiles (which spill) and 64
-// with 32 KiB ones.  A tile costs a ticket, a look at the table and three barriers,
-// about 2.4 us in which its compute unit requests nothing, whatever its size.
+// 32768 72 -> 82, 49152 65 -> 82, 65536 73 -> 82.5, and with rows of any start and
+// length 65533 68 -> 81, 100000 -> 82, 50001 -> 82, 33000 / 36000 70 -> 80, 20000 /
+// 22000 74 -> 78, 17000 (tiles 52 % full) 74 -> 75; not 8192 (half a tile) 75 -> 70.
+// bf16 T = 32768 72 -> 81, 65536 74 -> 82, 49152 73 -> 78, 100000 / 131071 69 -> 74 /
+// 75, 45000 (tiles 69 % full) 71 -> 72, but 40000 (61 %) 72 -> 70 and 35000 (53 %)
+// 70 -> 61.  complex64 (8,768,65536) 71 -> 70 with 64 KiB forward tiles (which spill)
+// and 64 with 32 KiB ones.  A tile costs a ticket, a look at the table and three
+// barriers, about 2.4 us in which its compute unit requests nothing, whatever its
+// size: all swept kernels of the real dtypes take 64 KiB tiles (4 KiB per wave).
 // ASCAN_SPLIT_MAX_ROWS (0 = never split) and ASCAN_SPLIT_MIN_ROW_BYTES (split every
 // row at least that long) override the rule, read once.
 constexpr int kSplitWaves = 16;
@@ -238,11 +243,14 @@ bool want_split(SweepClass c, int64_t rows, int64_t row_bytes, int64_t tile_byte
     if (too_few_rows(rows, ntiles)) return true;
     if (split_forced_min_row_bytes() > 0) return row_bytes >= split_forced_min_row_bytes();
     if (row_bytes < kSweepMinRowBytes) return false;
-    if (row_bytes * 10 < ntiles * tile_bytes * 7) return false;  // tiles less than 70 % full
+    // a row that leaves its tiles mostly empty: the remainder tile costs little (it is the first of its
+    // row in scan order and its empty sub-tiles are skipped), but not nothing
+    const int64_t least_full_percent = c == SweepClass::kF32 ? 55 : 66;
+    if (row_bytes * 100 < ntiles * tile_bytes * least_full_percent) return false;
     if (forward && tile_bytes < kSweepMinRowBytes) return false;
     switch (c) {
         case SweepClass::kF32: return true;
-        case SweepClass::kNarrow: return regular && (act == kGateIdentity || act == kGateExp);
+        case SweepClass::kNarrow: return tile_bytes >= kSweepMinRowBytes && (act == kGateIdentity || act == kGateExp);
         default: return false;
     }
 }
