@@ -179,7 +179,8 @@ inline int launch_status(hipError_t e) {
 // backward, % of the 8 TB/s peak, row walk -> sweep: fp32 T = 16384 72 -> 81,
 // 32768 72 -> 82, 49152 65 -> 82, 65536 73 -> 82.5, and with rows of any start and
 // length 65533 68 -> 81, 100000 -> 82, 50001 -> 82, 33000 / 36000 70 -> 80, 20000 /
-// 22000 74 -> 78, 17000 (tiles 52 % full) 74 -> 75; not 8192 (half a tile) 75 -> 70.
+// 22000 74 -> 78, 17000 (tiles 52 % full) 74 -> 75; a row of half a tile (8192)
+// 75 -> 72, but its backward pass alone gains (want_split).
 // bf16 T = 32768 72 -> 81, 65536 74 -> 82, 49152 73 -> 78, 100000 / 131071 69 -> 74 /
 // 75, 45000 (tiles 69 % full) 71 -> 72, but 40000 (61 %) 72 -> 70 and 35000 (53 %)
 // 70 -> 61.  complex64 (8,768,65536) 71 -> 70 with 64 KiB forward tiles (which spill)
@@ -189,7 +190,7 @@ inline int launch_status(hipError_t e) {
 // ASCAN_SPLIT_MAX_ROWS (0 = never split) and ASCAN_SPLIT_MIN_ROW_BYTES (split every
 // row at least that long) override the rule, read once.
 constexpr int kSplitWaves = 16;
-constexpr int64_t kSweepMinRowBytes = 64 * 1024;
+constexpr int64_t kSweepTileBytes = 64 * 1024;  // of one tensor, 16 waves x 4 KiB
 
 int64_t env_int64(const char* name, int64_t fallback) {
     const char* s = getenv(name);
@@ -228,7 +229,7 @@ bool too_few_rows(int64_t rows, int64_t ntiles) {
 }
 
 // `row_bytes`: one row of states; `tile_bytes`, `ntiles`: of the kernel that would run;
-// `regular`: that kernel is the mask-free one; `act`: its gate.  A compute unit holds one
+// `act`: its gate; `forward`: the forward kernel (3 tensors per tile) or the backward one (5 or 6).  A compute unit holds one
 // swept workgroup, so what a tile costs in arithmetic is not hidden behind another
 // workgroup's loads: the 16-bit kernels that evaluate a sigmoid (or the normalised
 // exponential gate's scale) for eight elements per vector lose when swept (bf16
@@ -237,20 +238,24 @@ bool too_few_rows(int64_t rows, int64_t ntiles) {
 // kernels of all gates 72 -> 78-81), and so does a forward kernel with 32 KiB tiles (the
 // normalised exponential gate's, fp32: 6.0 -> 5.3 TB/s) -- the backward kernels move five
 // or six tensors per tile and do well with 32 KiB of each.
-bool want_split(SweepClass c, int64_t rows, int64_t row_bytes, int64_t tile_bytes, int64_t ntiles, bool regular, int act,
-                bool forward) {
+bool want_split(SweepClass c, int64_t rows, int64_t row_bytes, int64_t tile_bytes, int64_t ntiles, int act, bool forward) {
     if (rows > split_max_rows()) return false;
     if (too_few_rows(rows, ntiles)) return true;
     if (split_forced_min_row_bytes() > 0) return row_bytes >= split_forced_min_row_bytes();
-    if (row_bytes < kSweepMinRowBytes) return false;
-    // a row that leaves its tiles mostly empty: the remainder tile costs little (it is the first of its
-    // row in scan order and its empty sub-tiles are skipped), but not nothing
-    const int64_t least_full_percent = c == SweepClass::kF32 ? 55 : 66;
-    if (row_bytes * 100 < ntiles * tile_bytes * least_full_percent) return false;
-    if (forward && tile_bytes < kSweepMinRowBytes) return false;
+    if (forward && tile_bytes < kSweepTileBytes) return false;
+    if (tile_bytes < kSweepTileBytes && row_bytes < kSweepTileBytes) return false;
+    // How full the row's tiles are.  The remainder tile costs little (it is the first of its row in scan
+    // order and its empty sub-tiles are skipped) but not nothing, and a row shorter than a tile leaves
+    // part of its only tile's workgroup idle.  Measured, fp32 (8,1536,T), TB/s whole rows -> swept:
+    // forward T = 8192 6.1 -> 5.0, 12000 6.1 -> 5.8, 14000 6.1 -> 6.2, 17000 5.9 -> 5.6, 20000 5.9 -> 6.2;
+    // backward (320 KiB per full tile rather than 192) 8192 6.0 -> 6.2, 10000 6.1 -> 6.3, 12000 6.0 -> 6.4,
+    // 17000 5.9 -> 6.3; bf16 35000 (53 %) 70 -> 61 % of peak, 40000 (61 %) 72 -> 70, 45000 (69 %) 71 -> 72,
+    // 24000 and 16384 (one tile, 73 and 50 % full) 71 -> 69 and 78 -> 63.
+    const int64_t percent_full = row_bytes * 100 / (ntiles * tile_bytes);
     switch (c) {
-        case SweepClass::kF32: return true;
-        case SweepClass::kNarrow: return tile_bytes >= kSweepMinRowBytes && (act == kGateIdentity || act == kGateExp);
+        case SweepClass::kF32: return percent_full >= (forward ? (ntiles == 1 ? 80 : 55) : 50);
+        case SweepClass::kNarrow:
+            return row_bytes >= kSweepTileBytes && percent_full >= 66 && (act == kGateIdentity || act == kGateExp);
         default: return false;
     }
 }
@@ -261,7 +266,7 @@ bool may_split(bool complex, int64_t rows, int64_t row_bytes, int64_t ntiles_mos
     if (rows > split_max_rows()) return false;
     if (too_few_rows(rows, ntiles_most)) return true;
     if (split_forced_min_row_bytes() > 0) return row_bytes >= split_forced_min_row_bytes();
-    return !complex && row_bytes >= kSweepMinRowBytes;
+    return !complex && row_bytes >= kSweepTileBytes / 2;
 }
 
 size_t split_bytes(int64_t rows, int64_t ntiles) {
