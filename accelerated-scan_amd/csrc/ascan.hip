@@ -241,8 +241,9 @@ size_t ascan_workspace_bytes(int64_t rows, int64_t seqlen, int dtype) {
     // rows are addressed from the 128-byte boundary below their first element at most
     const int64_t head = 128 / (int64_t)es - 1;
     const int64_t ntiles = (seqlen + head + tile - 1) / tile;
-    const bool complex = dtype == ASCAN_C64 || dtype == ASCAN_C64_REAL_TOKENS;
-    if (!may_split(complex, rows, seqlen * (int64_t)es, ntiles) || rows > 2147483647LL / ntiles) return 0;
+    const SweepClass c = dtype == ASCAN_F32 ? SweepClass::kF32
+                         : (dtype == ASCAN_BF16 || dtype == ASCAN_F16 ? SweepClass::kNarrow : SweepClass::kComplex);
+    if (!may_split(c, rows, seqlen * (int64_t)es, ntiles) || rows > 2147483647LL / ntiles) return 0;
     return split_bytes(rows, ntiles);
 }
 

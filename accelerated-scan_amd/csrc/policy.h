@@ -262,11 +262,15 @@ bool want_split(SweepClass c, int64_t rows, int64_t row_bytes, int64_t tile_byte
 
 // Whether some kernel of a call of this shape may want the table (`ntiles_most`: with
 // the smallest tile any kernel uses): what ascan_workspace_bytes goes by.
-bool may_split(bool complex, int64_t rows, int64_t row_bytes, int64_t ntiles_most) {
+bool may_split(SweepClass c, int64_t rows, int64_t row_bytes, int64_t ntiles_most) {
     if (rows > split_max_rows()) return false;
     if (too_few_rows(rows, ntiles_most)) return true;
     if (split_forced_min_row_bytes() > 0) return row_bytes >= split_forced_min_row_bytes();
-    return !complex && row_bytes >= kSweepTileBytes / 2;
+    switch (c) {
+        case SweepClass::kF32: return row_bytes >= kSweepTileBytes / 2;
+        case SweepClass::kNarrow: return row_bytes >= kSweepTileBytes;
+        default: return false;
+    }
 }
 
 size_t split_bytes(int64_t rows, int64_t ntiles) {

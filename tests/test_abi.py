@@ -109,11 +109,14 @@ def test_workspace_sizing_and_split_entry_validation():
     buf = ctypes.create_string_buffer(256)
     p = ctypes.addressof(buf)
     # short rows, and many complex rows: the plain kernels are the right choice
-    assert lib.ascan_workspace_bytes(12288, 8192, 0) == 0
+    assert lib.ascan_workspace_bytes(12288, 4096, 0) == 0
+    assert lib.ascan_workspace_bytes(12288, 16384, 1) == 0
     assert lib.ascan_workspace_bytes(4, 4096, 0) == 0
     assert lib.ascan_workspace_bytes(6144, 65536, 3) == 0
-    # rows of 64 KiB and more in a real dtype are swept in memory order, however many there are
+    # long rows in a real dtype are swept in memory order, however many there are (fp32 from 32 KiB on:
+    # the backward kernel gains from half-full 64 KiB tiles; 16-bit from 64 KiB on)
     assert lib.ascan_workspace_bytes(12288, 65536, 0) == 128 + 12288 * (65536 // 8192 + 1) * 64
+    assert lib.ascan_workspace_bytes(12288, 8192, 0) > 0
     assert lib.ascan_workspace_bytes(12288, 32768, 1) > 0
     assert lib.ascan_workspace_bytes(4, 1 << 20, 9) == 0  # unknown dtype
     assert lib.ascan_workspace_bytes(-1, 1 << 20, 0) == 0
