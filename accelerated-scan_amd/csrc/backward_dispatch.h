@@ -29,30 +29,32 @@ hipError_t launch_backward(const BackwardBuffers& b, int64_t rows, int64_t T, in
     constexpr int U = backward_blocks<ACT>(REGULAR ? Tuning<Tr>::UB : Tuning<Tr>::UBG);
     const unsigned blocks = (unsigned)((rows + rows_per_block - 1) / rows_per_block);
     const unsigned threads = 64u * W * rows_per_block;
-    return launch(scan_backward_kernel<Tr, W, U, REV, ALIGNED, REGULAR, false, ACT, false>, blocks, threads, stream,
+    return launch(scan_backward_kernel<Tr, W, U, REV, ALIGNED, REGULAR, kWholeRows, ACT, false>, blocks, threads, stream,
                   static_cast<const S*>(b.gates), static_cast<const S*>(b.states), static_cast<const S*>(b.grad_out),
                   static_cast<S*>(b.d_gates), static_cast<TokS*>(b.d_tokens), rows, T,
                   static_cast<SplitHeader*>(nullptr), static_cast<const S*>(b.initial), static_cast<S*>(b.d_initial),
                   grid, 0, static_cast<const S*>(b.values));
 }
 
-template <class Tr, bool REV, bool REGULAR, int ACT>
+// MODE = kSweep: `ntiles` tiles per row; kSweepRows: `rows_per_tile` rows per tile (the table is the ticket alone).
+template <class Tr, bool REV, bool REGULAR, int ACT, int MODE>
 hipError_t launch_backward_split(const BackwardBuffers& b, int64_t rows, int64_t T, int grid, int64_t ntiles,
-                                 const Workspace& ws, hipStream_t stream) {
+                                 int rows_per_tile, const Workspace& ws, hipStream_t stream) {
     using S = typename Tr::S;
     using TokS = typename Tr::TokS;
     constexpr int U = backward_blocks<ACT>(REGULAR ? SplitTuning<Tr>::UB : SplitTuning<Tr>::UBG);
-    auto kernel = scan_backward_kernel<Tr, kSplitWaves, U, REV, true, REGULAR, true, ACT, false>;
-    const unsigned resident = resident_workgroups(kernel, 64 * kSplitWaves);
+    auto kernel = scan_backward_kernel<Tr, kSplitWaves, U, REV, true, REGULAR, MODE, ACT, false>;
+    const unsigned resident = resident_workgroups(kernel, 64 * kSplitWaves, MODE == kSweepRows ? 1 : kMaxWavesPerBlock);
     if (resident == 0) return hipErrorInvalidConfiguration;
-    const hipError_t e = reset_split_table(ws, rows, ntiles, stream);
+    const bool whole_rows = MODE == kSweepRows;
+    const hipError_t e = reset_split_table(ws, whole_rows ? 0 : rows, ntiles, stream);
     if (e != hipSuccess) return e;
-    const int64_t tiles = rows * ntiles;
+    const int64_t tiles = whole_rows ? (rows + rows_per_tile - 1) / rows_per_tile : rows * ntiles;
     return launch(kernel, (unsigned)(tiles < resident ? tiles : resident), 64u * kSplitWaves, stream,
                   static_cast<const S*>(b.gates), static_cast<const S*>(b.states), static_cast<const S*>(b.grad_out),
                   static_cast<S*>(b.d_gates), static_cast<TokS*>(b.d_tokens), rows, T,
                   static_cast<SplitHeader*>(ws.ptr), static_cast<const S*>(b.initial), static_cast<S*>(b.d_initial),
-                  grid, 0, static_cast<const S*>(b.values));
+                  grid, rows_per_tile, static_cast<const S*>(b.values));
 }
 
 template <class Tr, bool REV, int PW, bool ALIGNED, int ACT>
@@ -61,7 +63,7 @@ hipError_t launch_backward_packed(const BackwardBuffers& b, int64_t rows, int64_
     using S = typename Tr::S;
     using TokS = typename Tr::TokS;
     const unsigned blocks = (unsigned)((rows + group - 1) / group);
-    return launch(scan_backward_kernel<Tr, PW, Tuning<Tr>::UBG, REV, ALIGNED, false, false, ACT, true>, blocks,
+    return launch(scan_backward_kernel<Tr, PW, Tuning<Tr>::UBG, REV, ALIGNED, false, kWholeRows, ACT, true>, blocks,
                   64u * PW, stream, static_cast<const S*>(b.gates), static_cast<const S*>(b.states),
                   static_cast<const S*>(b.grad_out), static_cast<S*>(b.d_gates), static_cast<TokS*>(b.d_tokens), rows,
                   T, static_cast<SplitHeader*>(nullptr), static_cast<const S*>(b.initial),
@@ -110,14 +112,25 @@ int backward_typed(const BackwardBuffers& b, int64_t rows, int64_t T, int act, c
     if (same_lead && ws.ptr != nullptr) {
         const int64_t SUBS = (int64_t)backward_blocks_of(act, SplitTuning<Tr>::UB) * 64 * Tr::EPV;
         const int64_t SUBSG = (int64_t)backward_blocks_of(act, SplitTuning<Tr>::UBG) * 64 * Tr::EPV;
+        if constexpr (kSweepClass<Tr> != SweepClass::kComplex) {
+            // rows of half a tile: two whole rows per swept tile
+            const int per_tile = lead == 0 ? sweep_rows_per_tile(kSweepClass<Tr>, rows, T, kElem, SUBS, act) : 0;
+            if (per_tile != 0 && workspace_fits(ws, 0, 1)) {
+                err = with_gate<Tr, REV>(act, [&](auto gate) {
+                    return launch_backward_split<Tr, REV, true, decltype(gate)::value, kSweepRows>(b, rows, T, at.grid, 1,
+                                                                                                 per_tile, ws, stream);
+                });
+                return launch_status(err);
+            }
+        }
         const bool regular = lead == 0 && T % (SUBS * kSplitWaves) == 0;
         const int64_t tile = (regular ? SUBS : SUBSG) * kSplitWaves;
         const int64_t ntiles = host_tiles_per_row<Tr>(T, tile, regular, at);
         if (want_split(kSweepClass<Tr>, rows, T * kElem, tile * kElem, ntiles, act, false) && workspace_fits(ws, rows, ntiles)) {
             err = with_gate<Tr, REV>(act, [&](auto gate) {
                 constexpr int ACT = decltype(gate)::value;
-                return regular ? launch_backward_split<Tr, REV, true, ACT>(b, rows, T, at.grid, ntiles, ws, stream)
-                               : launch_backward_split<Tr, REV, false, ACT>(b, rows, T, at.grid, ntiles, ws, stream);
+                return regular ? launch_backward_split<Tr, REV, true, ACT, kSweep>(b, rows, T, at.grid, ntiles, 0, ws, stream)
+                               : launch_backward_split<Tr, REV, false, ACT, kSweep>(b, rows, T, at.grid, ntiles, 0, ws, stream);
             });
             return launch_status(err);
         }

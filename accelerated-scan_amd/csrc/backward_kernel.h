@@ -29,7 +29,8 @@ namespace {
 // normalised exponential gate (x[t] = a x[t-1] + b v[t], a = exp(z), b = sqrt(1 - a^2))
 // d_v[t] = g[t] b[t] and d_z[t] = g[t] (a[t] x[t-1] - v[t] a[t]^2 / b[t]).
 // ---------------------------------------------------------------------------
-template <class Tr, int W, int U, bool REV, bool ALIGNED, bool REGULAR, bool SPLIT, int ACT, bool PACKED>
+// SPLIT: kWholeRows, kSweep or kSweepRows (split.h); with kSweepRows `group` is the number of rows a tile holds.
+template <class Tr, int W, int U, bool REV, bool ALIGNED, bool REGULAR, int SPLIT, int ACT, bool PACKED>
 __global__ void __launch_bounds__(64 * kMaxWavesPerBlock)
     scan_backward_kernel(const typename Tr::S* __restrict__ gates, const typename Tr::S* __restrict__ states,
                          const typename Tr::S* __restrict__ grad_out, typename Tr::S* __restrict__ d_gates,
@@ -43,6 +44,7 @@ __global__ void __launch_bounds__(64 * kMaxWavesPerBlock)
     constexpr int64_t TILE = SUB * W;
     static_assert(!PACKED || (!SPLIT && !REGULAR), "packed rows use the general kernels, one group per workgroup");
     static_assert(REV || ACT == kGateIdentity, "the gated scans run forward in time only");
+    constexpr bool ROWS = SPLIT == kSweepRows;
     constexpr bool LERP = kGateTakesValues<ACT>;  // `values` is a fourth input
     // index, inside a vector, of the element the gradient scan reaches first / last
     constexpr int E_FIRST = REV ? Tr::EPV - 1 : 0;
@@ -56,7 +58,10 @@ __global__ void __launch_bounds__(64 * kMaxWavesPerBlock)
     const int64_t longest = PACKED ? (int64_t)group * T : T;
     // rows start at the same misalignment when their length is a multiple of the grid spacing
     const int head = REGULAR ? 0 : (ALIGNED ? (longest % G == 0 ? row_lead<Tr>(gates, G) : G - 1) : 0);
-    const int64_t ntiles = tiles_per_row(longest, TILE, head);
+    const int64_t ntiles = tiles_per_row(longest, TILE, head);  // 1 when a tile holds several rows
+    // Several rows per tile: a row takes as many waves as it has sub-tiles, the tile as many rows as fit.
+    const int row_waves = ROWS ? (int)tiles_per_row(longest, SUB, head) : W;
+    const int64_t units = ROWS ? (rows + group - 1) / group : rows;  // what the tickets count: rows, or tiles of rows
     __shared__ V slots_all[W == 1 ? 1 : 2 * kSlotsPerBuffer];
     __shared__ S stage_all[PACKED ? W * SUB : 1];
     // Split rows: the workgroups take tiles by ticket, in memory order, until none
@@ -64,13 +69,13 @@ __global__ void __launch_bounds__(64 * kMaxWavesPerBlock)
     __shared__ int split_mailbox[2];
     __shared__ u32x4_t parked[SPLIT ? NIN * U * 64 : 1];  // wave 0's raw vectors during its walk back
     __shared__ V parked_values[SPLIT ? 4 * U * 64 : 1];  // and its per-lane scan results
-    const unsigned long long split_wait_limit = SPLIT ? split->wait_limit : 0ull;  // the longest wait allowed
+    const unsigned long long split_wait_limit = SPLIT == kSweep ? split->wait_limit : 0ull;  // the longest wait allowed
     for (bool first_visit = true;; first_visit = false) {
     int64_t row;
     int w, slot_base;
     int64_t k_begin = 0, k_end = ntiles;
     if constexpr (SPLIT) {
-        if (!take_split_tile(split, rows, ntiles, row, k_begin, split_mailbox)) break;
+        if (!take_split_tile(split, units, ntiles, row, k_begin, split_mailbox)) break;
         k_end = k_begin + 1;
         int thread = threadIdx.x;
         asm volatile("" : "+v"(thread));  // nothing derived from the wave index is carried from visit to visit
@@ -86,6 +91,18 @@ __global__ void __launch_bounds__(64 * kMaxWavesPerBlock)
         if (!locate_wave<W>(rows, ntiles, row, w, slot_base)) return;  // wave-uniform
     }
     V* slots = slots_all + (W == 1 ? 0 : slot_base);
+    // Several rows per tile: `row` so far is the tile; this wave's row and its place among the row's waves.
+    const int wave_in_tile = w;
+    if constexpr (ROWS) {
+        const int wave = __builtin_amdgcn_readfirstlane(w);
+        const int row_in_tile = wave / row_waves;
+        row = row * group + row_in_tile;
+        w = wave - row_in_tile * row_waves;
+        if (row_in_tile >= group || row >= rows) {  // wave-uniform: no row for this wave
+            exchange_carries_rows_idle();
+            continue;
+        }
+    }
 
     int64_t lo = (ALIGNED && !REGULAR) ? row_lead<Tr>(gates + row * T, G) : 0;
     // A row rarely fills its last tile.  Swept by ticket, the tile that holds the remainder should be
@@ -94,7 +111,7 @@ __global__ void __launch_bounds__(64 * kMaxWavesPerBlock)
     // fp32 (8,1536,65533), five tiles per row: forward 1.72 ms with the remainder last, 1.50 ms first).
     // A scan that runs down the addresses has it first as things are; one that runs up is addressed
     // from further below instead, so that its last tile ends on the grid boundary above the row.
-    if constexpr (SPLIT && !REV && ALIGNED && !REGULAR) lo += ntiles * TILE - (lo + len + G - 1) / G * G;
+    if constexpr (SPLIT == kSweep && !REV && ALIGNED && !REGULAR) lo += ntiles * TILE - (lo + len + G - 1) / G * G;
     const int64_t hi = lo + len;
     const S* __restrict__ arow = gates + row * T - lo;
     const S* __restrict__ xrow = states + row * T - lo;
@@ -127,7 +144,19 @@ __global__ void __launch_bounds__(64 * kMaxWavesPerBlock)
     // Position of this wave's sub-tile in tile step k of the gradient scan.
     auto sub_tile_base = [&](int64_t k) {
         const int64_t tile = REV ? ntiles - 1 - k : k;
-        return tile * TILE + (int64_t)(REV ? W - 1 - w : w) * SUB;
+        return tile * TILE + (int64_t)(REV ? row_waves - 1 - w : w) * SUB;
+    };
+    // Swept tiles: the gradient entering this wave's sub-tile, from the totals of the tile's waves and, for
+    // a row of several tiles, from the row's earlier tiles (wave 0 sets its vectors aside meanwhile).
+    auto hand_over = [&](const V (&totA)[U], const V (&totX)[U], V& c, int64_t k, int lane, auto set_aside,
+                         auto take_back) {
+        if constexpr (ROWS) {
+            exchange_carries_rows<V, W, U>(totA, totX, c, slots, wave_in_tile, lane, wave_in_tile - w, vzero<V>());
+        } else {
+            exchange_carries_split<V, W, U>(totA, totX, c, slots, w, lane, split, split_wait_limit,
+                                            split_records(split) + row * ntiles, k, ntiles, vzero<V>(), set_aside,
+                                            take_back);
+        }
     };
     // One tile step of this wave; FULL as in the forward kernel.
     auto tile_step = [&](int64_t k, auto full_tag) {
@@ -188,11 +217,9 @@ __global__ void __launch_bounds__(64 * kMaxWavesPerBlock)
                     totX[j] = vzero<V>();
                 }
                 V c;
-                exchange_carries_split<V, W, U>(
-                    totA, totX, c, slots, w, lane, split, split_wait_limit, split_records(split) + row * ntiles, k, ntiles,
-                    vzero<V>(), [] {}, [] {});
+                hand_over(totA, totX, c, k, lane, [] {}, [] {});
                 // the gradient scan passes through an empty sub-tile unchanged
-                if (d_initial != nullptr && k == ntiles - 1 && w == W - 1) store_start_gradient(c);  // wave-uniform
+                if (d_initial != nullptr && k == ntiles - 1 && w == row_waves - 1) store_start_gradient(c);  // wave-uniform
                 return;
             }
         }
@@ -304,9 +331,8 @@ __global__ void __launch_bounds__(64 * kMaxWavesPerBlock)
 
         V c;
         if constexpr (SPLIT) {
-            exchange_carries_split<V, W, U>(
-                totA, totX, c, slots, w, lane, split, split_wait_limit, split_records(split) + row * ntiles, k, ntiles,
-                vzero<V>(),
+            hand_over(
+                totA, totX, c, k, lane,
                 [&] {
 #pragma unroll
                     for (int j = 0; j < U; ++j) {
@@ -410,7 +436,7 @@ __global__ void __launch_bounds__(64 * kMaxWavesPerBlock)
         // A split row's last tile step ends where the differentiated scan started: after
         // pass 2, c is g at the last position this wave's sub-tile holds in the gradient scan.
         if constexpr (SPLIT) {
-            if (d_initial != nullptr && k == ntiles - 1 && w == W - 1) store_start_gradient(c);  // wave-uniform
+            if (d_initial != nullptr && k == ntiles - 1 && w == row_waves - 1) store_start_gradient(c);  // wave-uniform
         }
     };
 

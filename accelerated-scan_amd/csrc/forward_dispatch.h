@@ -16,26 +16,29 @@ hipError_t launch_forward(const void* gates, const void* tokens, void* out, cons
     constexpr int U = REGULAR ? Tuning<Tr>::U : Tuning<Tr>::UG;
     const unsigned blocks = (unsigned)((rows + rows_per_block - 1) / rows_per_block);
     const unsigned threads = 64u * W * rows_per_block;
-    return launch(scan_forward_kernel<Tr, W, U, REV, ALIGNED, REGULAR, false, ACT, false>, blocks, threads, stream,
+    return launch(scan_forward_kernel<Tr, W, U, REV, ALIGNED, REGULAR, kWholeRows, ACT, false>, blocks, threads, stream,
                   static_cast<const S*>(gates), static_cast<const TokS*>(tokens), static_cast<S*>(out), rows, T,
                   static_cast<SplitHeader*>(nullptr), static_cast<const S*>(initial), grid, 0);
 }
 
-template <class Tr, bool REV, bool REGULAR, int ACT>
+// MODE = kSweep: `ntiles` tiles per row; kSweepRows: `rows_per_tile` rows per tile (the table is the ticket alone).
+template <class Tr, bool REV, bool REGULAR, int ACT, int MODE>
 hipError_t launch_forward_split(const void* gates, const void* tokens, void* out, const void* initial, int64_t rows,
-                                int64_t T, int grid, int64_t ntiles, const Workspace& ws, hipStream_t stream) {
+                                int64_t T, int grid, int64_t ntiles, int rows_per_tile, const Workspace& ws,
+                                hipStream_t stream) {
     using S = typename Tr::S;
     using TokS = typename Tr::TokS;
     constexpr int U = forward_split_blocks<ACT>(REGULAR ? SplitTuning<Tr>::U : SplitTuning<Tr>::UG);
-    auto kernel = scan_forward_kernel<Tr, kSplitWaves, U, REV, true, REGULAR, true, ACT, false>;
-    const unsigned resident = resident_workgroups(kernel, 64 * kSplitWaves);
+    auto kernel = scan_forward_kernel<Tr, kSplitWaves, U, REV, true, REGULAR, MODE, ACT, false>;
+    const unsigned resident = resident_workgroups(kernel, 64 * kSplitWaves, MODE == kSweepRows ? 1 : kMaxWavesPerBlock);
     if (resident == 0) return hipErrorInvalidConfiguration;
-    const hipError_t e = reset_split_table(ws, rows, ntiles, stream);
+    const bool whole_rows = MODE == kSweepRows;
+    const hipError_t e = reset_split_table(ws, whole_rows ? 0 : rows, ntiles, stream);
     if (e != hipSuccess) return e;
-    const int64_t tiles = rows * ntiles;
+    const int64_t tiles = whole_rows ? (rows + rows_per_tile - 1) / rows_per_tile : rows * ntiles;
     return launch(kernel, (unsigned)(tiles < resident ? tiles : resident), 64u * kSplitWaves, stream,
                   static_cast<const S*>(gates), static_cast<const TokS*>(tokens), static_cast<S*>(out), rows, T,
-                  static_cast<SplitHeader*>(ws.ptr), static_cast<const S*>(initial), grid, 0);
+                  static_cast<SplitHeader*>(ws.ptr), static_cast<const S*>(initial), grid, rows_per_tile);
 }
 
 template <class Tr, bool REV, bool ALIGNED, int ACT>
@@ -44,7 +47,7 @@ hipError_t launch_forward_packed(const void* gates, const void* tokens, void* ou
     using S = typename Tr::S;
     using TokS = typename Tr::TokS;
     const unsigned blocks = (unsigned)((rows + group - 1) / group);
-    return launch(scan_forward_kernel<Tr, kPackedWaves, Tuning<Tr>::UG, REV, ALIGNED, false, false, ACT, true>, blocks,
+    return launch(scan_forward_kernel<Tr, kPackedWaves, Tuning<Tr>::UG, REV, ALIGNED, false, kWholeRows, ACT, true>, blocks,
                   64u * kPackedWaves, stream, static_cast<const S*>(gates), static_cast<const TokS*>(tokens),
                   static_cast<S*>(out), rows, T, static_cast<SplitHeader*>(nullptr), static_cast<const S*>(initial),
                   grid, group);
@@ -98,13 +101,26 @@ int forward_typed(const void* gates, const void* tokens, void* out, const void* 
     if (same_lead && ws.ptr != nullptr) {
         const int64_t SUBS = (int64_t)forward_split_blocks_of(act, SplitTuning<Tr>::U) * 64 * Tr::EPV;
         const int64_t SUBSG = (int64_t)forward_split_blocks_of(act, SplitTuning<Tr>::UG) * 64 * Tr::EPV;
+        if constexpr (kSweepClass<Tr> != SweepClass::kComplex) {
+            // rows of half a tile: two whole rows per swept tile
+            const int per_tile = lead == 0 ? sweep_rows_per_tile(kSweepClass<Tr>, rows, T, kElem, SUBS, act) : 0;
+            if (per_tile != 0 && workspace_fits(ws, 0, 1)) {
+                auto go = [&](auto rev, auto, auto gate) {
+                    return launch_forward_split<Tr, decltype(rev)::value, true, decltype(gate)::value, kSweepRows>(
+                        gates, tokens, out, initial, rows, T, at.grid, 1, per_tile, ws, stream);
+                };
+                err = dispatch_forward<Tr>(act, reverse, true, go);
+                return launch_status(err);
+            }
+        }
         const bool regular = lead == 0 && T % (SUBS * kSplitWaves) == 0;
         const int64_t tile = (regular ? SUBS : SUBSG) * kSplitWaves;
         const int64_t ntiles = host_tiles_per_row<Tr>(T, tile, regular, at);
         if (want_split(kSweepClass<Tr>, rows, T * kElem, tile * kElem, ntiles, act, true) && workspace_fits(ws, rows, ntiles)) {
             auto go = [&](auto rev, auto reg, auto gate) {
-                return launch_forward_split<Tr, decltype(rev)::value, decltype(reg)::value, decltype(gate)::value>(
-                    gates, tokens, out, initial, rows, T, at.grid, ntiles, ws, stream);
+                return launch_forward_split<Tr, decltype(rev)::value, decltype(reg)::value, decltype(gate)::value,
+                                            kSweep>(gates, tokens, out, initial, rows, T, at.grid, ntiles, 0, ws,
+                                                    stream);
             };
             err = dispatch_forward<Tr>(act, reverse, regular, go);
             return launch_status(err);

@@ -20,7 +20,8 @@ namespace {
 // rows of a workgroup are adjacent in memory, so with W*R = 16 one tile step
 // of the workgroup covers one contiguous span of 16 sub-tiles.
 // ---------------------------------------------------------------------------
-template <class Tr, int W, int U, bool REV, bool ALIGNED, bool REGULAR, bool SPLIT, int ACT, bool PACKED>
+// SPLIT: kWholeRows, kSweep or kSweepRows (split.h); with kSweepRows `group` is the number of rows a tile holds.
+template <class Tr, int W, int U, bool REV, bool ALIGNED, bool REGULAR, int SPLIT, int ACT, bool PACKED>
 __global__ void __launch_bounds__(64 * kMaxWavesPerBlock)
     scan_forward_kernel(const typename Tr::S* __restrict__ gates, const typename Tr::TokS* __restrict__ tokens,
                         typename Tr::S* __restrict__ out, int64_t rows, int64_t T, SplitHeader* split,
@@ -31,6 +32,7 @@ __global__ void __launch_bounds__(64 * kMaxWavesPerBlock)
     constexpr int64_t SUB = (int64_t)U * 64 * EPV;
     constexpr int64_t TILE = SUB * W;
     static_assert(!PACKED || (!SPLIT && !REGULAR), "packed rows use the general kernels, one group per workgroup");
+    constexpr bool ROWS = SPLIT == kSweepRows;
 
     // Packed rows: this workgroup scans rows [first_row, first_row + nrows) as one row of `len` elements.
     const int64_t first_row = PACKED ? (int64_t)blockIdx.x * group : 0;
@@ -38,20 +40,23 @@ __global__ void __launch_bounds__(64 * kMaxWavesPerBlock)
     const int64_t longest = PACKED ? (int64_t)group * T : T;
     // rows start at the same misalignment when their length is a multiple of the grid spacing
     const int head = REGULAR ? 0 : (ALIGNED ? (longest % G == 0 ? row_lead<Tr>(gates, G) : G - 1) : 0);
-    const int64_t ntiles = tiles_per_row(longest, TILE, head);
+    const int64_t ntiles = tiles_per_row(longest, TILE, head);  // 1 when a tile holds several rows
+    // Several rows per tile: a row takes as many waves as it has sub-tiles, the tile as many rows as fit.
+    const int row_waves = ROWS ? (int)tiles_per_row(longest, SUB, head) : W;
+    const int64_t units = ROWS ? (rows + group - 1) / group : rows;  // what the tickets count: rows, or tiles of rows
     __shared__ V slots_all[W == 1 ? 1 : 2 * kSlotsPerBuffer];
     __shared__ S stage_all[PACKED ? W * SUB : 1];
     // Split rows: the workgroups take tiles by ticket, in memory order, until none
     // is left; a workgroup only ever waits for tiles whose owners started before it.
     __shared__ int split_mailbox[2];
     __shared__ u32x4_t parked[SPLIT ? 2 * U * 64 : 1];  // wave 0's raw vectors during its walk back
-    const unsigned long long split_wait_limit = SPLIT ? split->wait_limit : 0ull;  // the longest wait allowed
+    const unsigned long long split_wait_limit = SPLIT == kSweep ? split->wait_limit : 0ull;  // the longest wait allowed
     for (bool first_visit = true;; first_visit = false) {
     int64_t row;
     int w, slot_base;
     int64_t k_begin = 0, k_end = ntiles;
     if constexpr (SPLIT) {
-        if (!take_split_tile(split, rows, ntiles, row, k_begin, split_mailbox)) break;
+        if (!take_split_tile(split, units, ntiles, row, k_begin, split_mailbox)) break;
         k_end = k_begin + 1;
         int thread = threadIdx.x;
         asm volatile("" : "+v"(thread));  // nothing derived from the wave index is carried from visit to visit
@@ -67,6 +72,18 @@ __global__ void __launch_bounds__(64 * kMaxWavesPerBlock)
         if (!locate_wave<W>(rows, ntiles, row, w, slot_base)) return;  // wave-uniform
     }
     V* slots = slots_all + (W == 1 ? 0 : slot_base);
+    // Several rows per tile: `row` so far is the tile; this wave's row and its place among the row's waves.
+    const int wave_in_tile = w;
+    if constexpr (ROWS) {
+        const int wave = __builtin_amdgcn_readfirstlane(w);
+        const int row_in_tile = wave / row_waves;
+        row = row * group + row_in_tile;
+        w = wave - row_in_tile * row_waves;
+        if (row_in_tile >= group || row >= rows) {  // wave-uniform: no row for this wave
+            exchange_carries_rows_idle();
+            continue;
+        }
+    }
 
     int64_t lo = (ALIGNED && !REGULAR) ? row_lead<Tr>(gates + row * T, G) : 0;
     // A row rarely fills its last tile.  Swept by ticket, the tile that holds the remainder should be
@@ -75,7 +92,7 @@ __global__ void __launch_bounds__(64 * kMaxWavesPerBlock)
     // fp32 (8,1536,65533), five tiles per row: forward 1.72 ms with the remainder last, 1.50 ms first).
     // A scan that runs down the addresses has it first as things are; one that runs up is addressed
     // from further below instead, so that its last tile ends on the grid boundary above the row.
-    if constexpr (SPLIT && !REV && ALIGNED && !REGULAR) lo += ntiles * TILE - (lo + len + G - 1) / G * G;
+    if constexpr (SPLIT == kSweep && !REV && ALIGNED && !REGULAR) lo += ntiles * TILE - (lo + len + G - 1) / G * G;
     const int64_t hi = lo + len;
     const S* __restrict__ grow = gates + row * T - lo;
     const typename Tr::TokS* __restrict__ trow = tokens + row * T - lo;
@@ -90,7 +107,19 @@ __global__ void __launch_bounds__(64 * kMaxWavesPerBlock)
     // Position of this wave's sub-tile in tile step k.
     auto sub_tile_base = [&](int64_t k) {
         const int64_t tile = REV ? (ntiles - 1 - k) : k;
-        return tile * TILE + (int64_t)(REV ? (W - 1 - w) : w) * SUB;
+        return tile * TILE + (int64_t)(REV ? (row_waves - 1 - w) : w) * SUB;
+    };
+    // Swept tiles: the state entering this wave's sub-tile, from the totals of the tile's waves and, for
+    // a row of several tiles, from the row's earlier tiles (wave 0 sets its vectors aside meanwhile).
+    auto hand_over = [&](const V (&totA)[U], const V (&totX)[U], V& c, int64_t k, int lane, auto set_aside,
+                         auto take_back) {
+        if constexpr (ROWS) {
+            exchange_carries_rows<V, W, U>(totA, totX, c, slots, wave_in_tile, lane, wave_in_tile - w, row_start);
+        } else {
+            exchange_carries_split<V, W, U>(totA, totX, c, slots, w, lane, split, split_wait_limit,
+                                            split_records(split) + row * ntiles, k, ntiles, row_start, set_aside,
+                                            take_back);
+        }
     };
     // One tile step of this wave.  FULL (a compile-time flag) says that the
     // wave's sub-tile lies entirely inside the row: that copy of the body has no
@@ -145,9 +174,7 @@ __global__ void __launch_bounds__(64 * kMaxWavesPerBlock)
                     totX[j] = vzero<V>();
                 }
                 V c;
-                exchange_carries_split<V, W, U>(
-                    totA, totX, c, slots, w, lane, split, split_wait_limit, split_records(split) + row * ntiles, k, ntiles,
-                    row_start, [] {}, [] {});
+                hand_over(totA, totX, c, k, lane, [] {}, [] {});
                 return;
             }
         }
@@ -213,9 +240,8 @@ __global__ void __launch_bounds__(64 * kMaxWavesPerBlock)
 
         V c;
         if constexpr (SPLIT) {
-            exchange_carries_split<V, W, U>(
-                totA, totX, c, slots, w, lane, split, split_wait_limit, split_records(split) + row * ntiles, k, ntiles,
-                row_start,
+            hand_over(
+                totA, totX, c, k, lane,
                 [&] {
 #pragma unroll
                     for (int j = 0; j < U; ++j) {

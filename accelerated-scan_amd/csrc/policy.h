@@ -217,6 +217,13 @@ unsigned long long split_wait_limit() {
 }
 
 enum class SweepClass { kF32, kNarrow, kComplex };
+
+// ASCAN_SWEEP_ROWS (sweep_rows_per_tile below), read once; -1 when unset.
+int sweep_rows_mode() {
+    static const int v = getenv("ASCAN_SWEEP_ROWS") ? env_int("ASCAN_SWEEP_ROWS") : -1;
+    return v;
+}
+constexpr int64_t kSweepRowsMinBytes = 256ll << 20;  // of one tensor
 template <class Tr>
 constexpr SweepClass kSweepClass = Tr::kNarrow ? SweepClass::kNarrow
                                                : (std::is_same<typename Tr::V, float>::value ? SweepClass::kF32
@@ -268,9 +275,38 @@ bool may_split(SweepClass c, int64_t rows, int64_t row_bytes, int64_t ntiles_mos
     if (split_forced_min_row_bytes() > 0) return row_bytes >= split_forced_min_row_bytes();
     switch (c) {
         case SweepClass::kF32: return row_bytes >= kSweepTileBytes / 2;
-        case SweepClass::kNarrow: return row_bytes >= kSweepTileBytes;
+        case SweepClass::kNarrow:
+            return row_bytes >= kSweepTileBytes ||
+                   (row_bytes == kSweepTileBytes / 2 && rows * row_bytes >= kSweepRowsMinBytes);  // two rows per tile
         default: return false;
     }
+}
+
+// Rows of exactly half a swept tile, starting on the grid: two whole rows per tile of a
+// kSweepRows launch, each on eight waves (returns the rows per tile, or 0).  `sub`: the
+// elements per wave of the mask-free kernel that would run.  The tiles are full and no
+// tile waits for another, so the sweep runs as for rows of one full tile -- but a launch
+// costs the table's reset and the filling of 256 persistent workgroups, which shorter
+// rows (several per tile work just as well) and small tensors do not earn back.
+// Measured, forward + backward, % of peak, whole rows -> swept: fp32 (B,1536,8192) B = 16
+// 77.7 -> 81.6, 8 77.2 -> 79.8, 4 76.8 -> 77.0, 2 73.8 -> 71.6; (8,1536,4096) 79.8 -> 76.7,
+// (8,1536,2048) 78.3 -> 71.6; bf16 (8,1536,16384) 77.2 -> 79.1, (4,1536,16384) 77.9 -> 75.5;
+// fp16 (8,1536,16384) 76.4 -> 79.9.  With a gate, ms forward + backward at those shapes:
+// fp32 sigmoid 0.541 -> 0.510, exp 0.535 -> 0.509, bf16 sigmoid 0.525 -> 0.627, exp
+// 0.514 -> 0.558 (a compute unit holds one swept workgroup and does not hide the 16-bit
+// kernels' gate arithmetic behind another's loads).  Rows that leave sub-tiles partly
+// empty lose (fp32 T = 6000 77.3 -> 75.2, bf16 12000 73.9 -> 63.3), and so do tiles handed
+// out by workgroup index instead of by ticket (70 %).
+// ASCAN_SWEEP_ROWS = 0 / 1 (never / whenever rows divide a tile) overrides the rule.
+int sweep_rows_per_tile(SweepClass c, int64_t rows, int64_t T, int64_t elem_bytes, int64_t sub, int act) {
+    if (c == SweepClass::kComplex || T % sub != 0 || rows > split_max_rows() || sweep_rows_mode() == 0) return 0;
+    const int64_t row_waves = T / sub;
+    if (row_waves * 2 > kSplitWaves || kSplitWaves % row_waves != 0) return 0;
+    const int per_tile = (int)(kSplitWaves / row_waves);
+    if (sweep_rows_mode() == 1) return per_tile;
+    if (per_tile != 2 || rows * T * elem_bytes < kSweepRowsMinBytes) return 0;
+    if (c != SweepClass::kF32 && act != kGateIdentity) return 0;
+    return per_tile;
 }
 
 size_t split_bytes(int64_t rows, int64_t ntiles) {
@@ -292,9 +328,13 @@ hipError_t reset_split_table(const Workspace& ws, int64_t rows, int64_t ntiles, 
 }
 
 // Number of workgroups of `kernel` (of `threads` threads, no dynamic LDS) the
-// current device holds at one time.  Queried once per kernel and device.
+// current device holds at one time, `most_per_cu` per compute unit at most (the same
+// at every call for one kernel).  Queried once per kernel and device.
+// The swept kernels that hold several rows per tile need no registers for a look-back
+// and would fit twice, but run one workgroup per compute unit like the others: measured,
+// fp32 (8,1536,8192) forward 6.3 TB/s with one, 5.9 with two.
 template <class K>
-unsigned resident_workgroups(K kernel, int threads) {
+unsigned resident_workgroups(K kernel, int threads, int most_per_cu) {
     int device = 0;
     if (hipGetDevice(&device) != hipSuccess) return 0;
     constexpr int kMaxDevices = 64;
@@ -308,17 +348,21 @@ unsigned resident_workgroups(K kernel, int threads) {
             per_cu <= 0 || cus <= 0) {
             return 0;
         }
+        if (per_cu > most_per_cu) per_cu = most_per_cu;
         known = (unsigned)per_cu * (unsigned)cus;
         cache[device].store(known, std::memory_order_relaxed);
     }
     return known;
 }
 
-// Tiles per row as the kernels count them (tiles_per_row on the device).
+// Tiles per row as the kernels count them (tiles_per_row on the device), and the
+// distance from the grid boundary they address rows from to a row's first element, at most.
+inline int host_head(int64_t T, bool regular, const Lead& at) {
+    return regular ? 0 : (T % at.grid == 0 ? at.lead : at.grid - 1);
+}
 template <class Tr>
 int64_t host_tiles_per_row(int64_t T, int64_t tile, bool regular, const Lead& at) {
-    const int head = regular ? 0 : (T % at.grid == 0 ? at.lead : at.grid - 1);
-    return (T + head + tile - 1) / tile;
+    return (T + host_head(T, regular, at) + tile - 1) / tile;
 }
 
 // Packed-row policy.  Rows shorter than kPackedMaxRowBytes (of states) are

@@ -61,6 +61,11 @@ struct alignas(64) SplitTicket {
 };
 static_assert(sizeof(SplitTicket) == 64, "ticket line is 64 bytes");
 
+// How a kernel's workgroups come by their work (template argument SPLIT of the scan kernels).
+constexpr int kWholeRows = 0;  // a workgroup owns its rows from start to end
+constexpr int kSweep = 1;      // tiles of all rows by ticket, in memory order; a row's tiles hand their state on
+constexpr int kSweepRows = 2;  // the same for rows of at most half a tile: a tile holds several whole rows
+
 constexpr unsigned long long kWaitStepCap = 1000;  // 10 us in 100 MHz ticks
 constexpr int kSplitWindow = 64;                   // tiles per look-back window: one per lane
 
@@ -284,6 +289,44 @@ __device__ __forceinline__ void exchange_carries_split(const V (&totA)[U], const
     __syncthreads();
     c = vfma(mineA, *carry_slot, mineX);
 }
+
+// The same for a swept tile that holds several whole rows (kSweepRows): the waves
+// [first, first + waves of a row) scan one row, so a wave's prefix runs over the
+// waves of its own row only and starts from that row's own state.  No tile depends
+// on another, so there is no look at the table: one barrier, and the slots are safe
+// to rewrite after the barriers of the next ticket draw.
+template <class V, int W, int U>
+__device__ __forceinline__ void exchange_carries_rows(const V (&totA)[U], const V (&totX)[U], V& c, V* slots, int w,
+                                                      int lane, int first, V row_start) {
+    V TA = totA[0], TX = totX[0];
+#pragma unroll
+    for (int j = 1; j < U; ++j) {
+        TX = vfma(TX, totA[j], totX[j]);
+        TA = vmul(TA, totA[j]);
+    }
+    if (lane == 0) {
+        slots[2 * w] = TA;
+        slots[2 * w + 1] = TX;
+    }
+    __syncthreads();
+    V runA = vone<V>(), runX = vzero<V>();
+    V mineA = runA, mineX = runX;
+#pragma unroll
+    for (int i = 0; i < W; ++i) {
+        const V Ai = slots[2 * i];
+        const V Xi = slots[2 * i + 1];
+        runA = vselect(i == first, vone<V>(), runA);
+        runX = vselect(i == first, vzero<V>(), runX);
+        mineA = vselect(i == w, runA, mineA);
+        mineX = vselect(i == w, runX, mineX);
+        runX = vfma(runX, Ai, Xi);
+        runA = vmul(runA, Ai);
+    }
+    c = vfma(mineA, row_start, mineX);
+}
+// A wave of such a tile that has no row (the tile's waves are not a multiple of a
+// row's, or the rows ran out) keeps the barrier company.
+__device__ __forceinline__ void exchange_carries_rows_idle() { __syncthreads(); }
 
 }  // namespace
 }  // namespace ascan

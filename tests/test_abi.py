@@ -110,7 +110,8 @@ def test_workspace_sizing_and_split_entry_validation():
     p = ctypes.addressof(buf)
     # short rows, and many complex rows: the plain kernels are the right choice
     assert lib.ascan_workspace_bytes(12288, 4096, 0) == 0
-    assert lib.ascan_workspace_bytes(12288, 16384, 1) == 0
+    assert lib.ascan_workspace_bytes(4096, 16384, 1) == 0
+    assert lib.ascan_workspace_bytes(12288, 12288, 1) == 0
     assert lib.ascan_workspace_bytes(4, 4096, 0) == 0
     assert lib.ascan_workspace_bytes(6144, 65536, 3) == 0
     # long rows in a real dtype are swept in memory order, however many there are (fp32 from 32 KiB on:
@@ -118,6 +119,9 @@ def test_workspace_sizing_and_split_entry_validation():
     assert lib.ascan_workspace_bytes(12288, 65536, 0) == 128 + 12288 * (65536 // 8192 + 1) * 64
     assert lib.ascan_workspace_bytes(12288, 8192, 0) > 0
     assert lib.ascan_workspace_bytes(12288, 32768, 1) > 0
+    # 16-bit rows of exactly half a tile, two to a swept tile, once the tensors reach 256 MiB
+    assert lib.ascan_workspace_bytes(12288, 16384, 1) > 0
+    assert lib.ascan_workspace_bytes(12288, 16384, 2) > 0
     assert lib.ascan_workspace_bytes(4, 1 << 20, 9) == 0  # unknown dtype
     assert lib.ascan_workspace_bytes(-1, 1 << 20, 0) == 0
     # few long rows: header (64 bytes) + the ticket line (64 bytes)

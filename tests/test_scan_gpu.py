@@ -878,6 +878,73 @@ def test_sweep_of_many_long_rows(dtype, rows, T):
     _compare_with_truth(gates, tokens, grad_out, out, rev, dg, dx, dtype, what="sweep", reverse_grads=(rdg, rdx))
 
 
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.float16], ids=["fp32", "bf16", "fp16"])
+def test_rows_of_half_a_tile_share_swept_tiles(dtype):
+    """Rows of exactly 32 KiB, enough of them for 256 MiB per tensor: with a table the library
+    sweeps them two to a 64 KiB tile, eight waves each (an odd number of rows, so the last tile
+    holds one).  Every result is compared with that of the plain entry points, which take no
+    table and give each row a workgroup of its own, and a sample of rows -- the first and last
+    tiles among them -- with the fp64 loops.  Both scan directions, initial states included."""
+    from accelerated_scan import _abi
+
+    lib = _abi.load()
+    code = _abi.dtype_code(dtype, dtype)
+    T = (1 << 15) // torch.empty(0, dtype=dtype).element_size()
+    rows = (256 << 20) // (1 << 15) + 1
+    nbytes = lib.ascan_workspace_bytes(rows, T, code)
+    assert nbytes > 0, "rows of this length are meant to be swept"
+    gen = torch.Generator(device=DEVICE).manual_seed(rows)
+    g = torch.rand(rows, T, generator=gen, device=DEVICE).to(dtype)
+    x, d = (torch.randn(rows, T, generator=gen, device=DEVICE).to(dtype) for _ in range(2))
+    start = torch.randn(rows, generator=gen, device=DEVICE).to(dtype)
+    sample = torch.tensor([0, 1, 2, 3, rows // 2, rows - 3, rows - 2, rows - 1], device=DEVICE)
+    tol = _tolerance(dtype)
+    for reverse in (False, True):
+        swept, plain = ([torch.empty_like(g) for _ in range(3)] + [torch.empty_like(start)] for _ in range(2))
+        tables = [torch.ones(nbytes, dtype=torch.uint8, device=DEVICE) for _ in range(2)]  # garbage: the library clears it
+        _abi.forward(g, x, swept[0], reverse, workspace=tables[0], initial=start)
+        _abi.backward(g, swept[0], d, swept[1], swept[2], workspace=tables[1], initial=start, d_initial=swept[3],
+                      reverse=reverse)
+        none = torch.empty(0, dtype=torch.uint8, device=DEVICE)  # a table of no bytes: whole rows per workgroup
+        _abi.forward(g, x, plain[0], reverse, workspace=none, initial=start)
+        _abi.backward(g, swept[0], d, plain[1], plain[2], workspace=none, initial=start, d_initial=plain[3],
+                      reverse=reverse)
+        torch.cuda.synchronize()
+        assert [_abi.workspace_timeouts(t) for t in tables] == [0, 0]
+        # the swept launches drew tickets for tiles of two rows
+        cus = torch.cuda.get_device_properties(0).multi_processor_count
+        for table in tables:
+            drawn = int.from_bytes(bytes(table[64:72].cpu().tolist()), "little")
+            assert drawn == (rows + 1) // 2 + cus, drawn
+        for name, a, b in zip(("out", "d_gates", "d_tokens", "d_initial"), swept, plain):
+            scale = max(1.0, float(b.float().abs().max()))
+            torch.testing.assert_close(a.float(), b.float(), rtol=tol["rtol"], atol=tol["atol"] * scale,
+                                       msg=lambda m: f"{name} reverse={reverse} {dtype}: {m}")
+        gs, xs, ds_, ss, outs = (t[sample].cpu() for t in (g, x, d, start, swept[0]))
+        t_out = seqscan.forward_from(_np32(gs), _np32(xs), _np32(ss), reverse=reverse)
+        t_dg, t_dx, t_di = seqscan.backward_from(_np32(gs), _np32(outs), _np32(ss), _np32(ds_), reverse=reverse)
+        for name, got, want in (("out", swept[0], t_out), ("d_gates", swept[1], t_dg), ("d_tokens", swept[2], t_dx),
+                                ("d_initial", swept[3], t_di)):
+            scale = max(1.0, float(np.abs(want).max()))
+            np.testing.assert_allclose(_np32(got[sample].cpu()), want, rtol=tol["rtol"], atol=tol["atol"] * scale,
+                                       err_msg=f"{name} reverse={reverse} {dtype}")
+
+
+def test_rows_sharing_swept_tiles_small_shapes():
+    """2, 4, 8 and 16 rows per swept tile, tiles whose last rows are missing, initial states, both
+    directions and the gated kernels, at small sizes against the fp64 loops: in a child process,
+    because the switch that makes the library sweep such rows whatever their number
+    (ASCAN_SWEEP_ROWS=1) is read once per process."""
+    import os
+    import subprocess
+    import sys
+
+    done = subprocess.run([sys.executable, str(ROOT / "tests" / "sweep_rows_child.py")],
+                          env=dict(os.environ, ASCAN_SWEEP_ROWS="1"), capture_output=True, text=True, timeout=110)
+    assert done.returncode == 0, done.stdout[-2000:] + done.stderr[-4000:]
+    assert "checked 84" in done.stdout, done.stdout
+
+
 @pytest.mark.parametrize("rows,T", [(3, 1 << 20), (600, 1 << 16), (1, 1 << 23)], ids=["few", "many", "one"])
 def test_split_rows_are_reproducible(rows, T):
     """Twenty runs of one split shape give the same bits: a tile's carry is the state
