@@ -84,8 +84,16 @@ int backward_typed(const BackwardBuffers& b, int64_t rows, int64_t T, int act, c
     // narrower plan for a mostly empty last tile whatever the dtype: fp32 (8,1536,9000) backward 4.9 -> 5.5 TB/s
     const bool trim = kTrimPlan<Tr> || gate_takes_values(act);
     Plan plan = choose_plan(T, SUB, kElem, trim);
-    const Access access = choose_access(same_lead, lead, T, SUB * plan.waves_per_row);
+    Access access = choose_access(same_lead, lead, T, SUB * plan.waves_per_row);
     if (access != Access::kRegular) plan = choose_plan(T, SUBG, kElem, trim);
+    // fp32 rows of exactly 4 KiB: two waves of 2 KiB per row (the kernel with masking code, whose tile steps
+    // inside a row are mask-free as well) instead of one wave of 4 KiB -- measured, (8,1536,1024) 5.7 -> 6.06 TB/s,
+    // (32,1536,1024) 6.22 -> 6.26, (2,1536,1024) 5.03 -> 4.95
+    if (kSweepClass<Tr> == SweepClass::kF32 && access == Access::kRegular && T == SUB && SUBG * 2 == SUB &&
+        forced_plan().waves_per_row == 0 && forced_plan().rows_per_block == 0) {
+        access = Access::kVector;
+        plan = Plan{2, 2};
+    }
     const int R = plan.rows_per_block;
     hipError_t err = hipSuccess;
     // 16-bit rows of 512 bytes and more, vectorised flavour, plenty of them: groups of the wider workgroup

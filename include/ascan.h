@@ -172,7 +172,10 @@ ASCAN_API int ascan_backward(const void* gates, const void* states, const void* 
  * tile at a time to whichever resident workgroup is free, and pass the running
  * state from tile to tile through a small table in the workspace: one pass over
  * the data, no extra traffic.  Measured on MI355X, fp32 (8, 1536, 65536) forward +
- * backward: 4.40 ms without a workspace, 3.90 ms with one.  They have no
+ * backward: 4.40 ms without a workspace, 3.90 ms with one.  (Rows of exactly half
+ * a tile -- 32 KiB, starting on a 128-byte boundary -- are swept as well once the
+ * tensors reach 256 MiB, two whole rows to a tile; the table then serves for the
+ * ticket only.)  They have no
  * counterpart in the reference, whose kernels give one thread block to each
  * sequence (warp.cuh:279; scalar.py:98; complex.py:174).
  *
