@@ -298,7 +298,9 @@ bool may_split(SweepClass c, int64_t rows, int64_t row_bytes, int64_t ntiles_mos
 // 0.514 -> 0.558 (a compute unit holds one swept workgroup and does not hide the 16-bit
 // kernels' gate arithmetic behind another's loads).  Rows that leave sub-tiles partly
 // empty lose (fp32 T = 6000 77.3 -> 75.2, bf16 12000 73.9 -> 63.3), and so do tiles handed
-// out by workgroup index instead of by ticket (70 %).
+// out by workgroup index instead of by ticket (70 %) and tickets drawn a tile ahead, behind
+// the loads (77.5 % at T = 8192: no tile waits for another here, but the stretch of memory
+// in flight is twice as long).
 // ASCAN_SWEEP_ROWS = 0 / 1 (never / whenever rows divide a tile) overrides the rule.
 int sweep_rows_per_tile(SweepClass c, int64_t rows, int64_t T, int64_t elem_bytes, int64_t sub, int act) {
     if (c == SweepClass::kComplex || T % sub != 0 || rows > split_max_rows() || sweep_rows_mode() == 0) return 0;
