@@ -50,6 +50,19 @@ __global__ void __launch_bounds__(64 * kMaxWavesPerBlock)
     constexpr int E_FIRST = REV ? Tr::EPV - 1 : 0;
     constexpr int E_LAST = REV ? 0 : Tr::EPV - 1;
     constexpr int NIN = LERP ? 4 : 3;
+    // The states are needed by pass 2 only.  Requested after pass 1, they travel while the tile looks
+    // at the table (about 3 us under load, in which nothing else of this compute unit's is in flight),
+    // and the compiler schedules the state loads that way, or halfway through pass 1, in most swept
+    // instantiations by itself.  In the fp32 kernel for reverse scans with rows of any start and length
+    // it put all twelve loads up front, and that kernel was the slower of two mirror images: measured at
+    // (8,1536,T), compiler's order -> states held back, T = 65533 2.53 -> 2.44 ms, 50001 2.01 -> 1.90,
+    // 20000 0.885 -> 0.787 (its mirror image for forward scans: 2.45 -> 2.43, 1.89 -> 1.89, 0.783 ->
+    // 0.787, and T = 12000 0.467 -> 0.455).  Held back everywhere, the kernels that own whole rows lose
+    // (nothing to wait for after pass 1: bf16 (8,1536,12000) backward 0.26 -> 0.31 ms) and so do the
+    // swept 16-bit ones (wave 0 sets its vectors aside before it looks and then waits for them: bf16
+    // (8,1536,65533) 1.37 -> 1.48 ms), so the switch is for the fp32 kernels with masking code.
+    constexpr bool STATES_LATE = SPLIT == kSweep && !REGULAR && ACT == kGateIdentity && !Tr::kNarrow &&
+                                 std::is_same<V, float>::value;
 
     const int lane = threadIdx.x & 63;
     // Packed rows: this workgroup scans rows [first_row, first_row + nrows) as one row of `len` elements.
@@ -231,7 +244,11 @@ __global__ void __launch_bounds__(64 * kMaxWavesPerBlock)
                 const int off = vec_offset<U, EPV, REV>(j, lane);
                 araw[j] = load_raw<Tr, ALIGNED, FULL>(asub, off, win, identity_gate<ACT, V>());
                 draw[j] = load_raw<Tr, ALIGNED, FULL>(dsub, off, win, vzero<V>());
-                xraw[j] = load_raw<Tr, ALIGNED, FULL>(xsub, off, win, x_start);
+                if constexpr (STATES_LATE) {
+                    xraw[j] = fill_raw<Tr>(x_start);  // stands in until the load below
+                } else {
+                    xraw[j] = load_raw<Tr, ALIGNED, FULL>(xsub, off, win, x_start);
+                }
                 if constexpr (LERP) vraw[j] = load_raw<Tr, ALIGNED, FULL>(vsub, off, win, vzero<V>());
             }
         } else {
@@ -329,6 +346,17 @@ __global__ void __launch_bounds__(64 * kMaxWavesPerBlock)
             exX[j] = shift_up1(X, vzero<V>());
         }
 
+        if constexpr (STATES_LATE) {
+            // the offset waits for pass 1's last total, so the loads cannot be moved ahead of it
+            const int late = zero_after(totX[U - 1]);
+            if (touches) {
+#pragma unroll
+                for (int j = 0; j < U; ++j) {
+                    xraw[j] = load_raw<Tr, ALIGNED, FULL>(xsub, vec_offset<U, EPV, REV>(j, lane) + late, win, x_start);
+                }
+            }
+        }
+
         V c;
         if constexpr (SPLIT) {
             hand_over(
@@ -377,6 +405,15 @@ __global__ void __launch_bounds__(64 * kMaxWavesPerBlock)
             Tr::unpack(draw[j], d);
             Tr::unpack(xraw[j], x);
             if constexpr (LERP) Tr::unpack(vraw[j], v);
+            if constexpr (STATES_LATE) {  // pass 1 saw stand-ins
+                V lo_edge = x_edge;
+                if (j < U - 1) {
+                    V below[EPV];
+                    Tr::unpack(xraw[j < U - 1 ? j + 1 : j], below);
+                    lo_edge = read_lane<0>(below[E_FIRST]);
+                }
+                x_prev[j] = shift_down1(x[E_FIRST], lo_edge);
+            }
             V gr = carry_in<PACKED>(exA[j], c, exX[j]);  // g entering this lane's vector
             c = carry_in<PACKED>(totA[j], c, totX[j]);
             const int off = vec_offset<U, EPV, REV>(j, lane);

@@ -17,6 +17,15 @@ struct cfloat {
     float re, im;
 };
 
+// An integer zero that the compiler cannot produce before `v` exists: added to the offset of a load, it
+// keeps the load behind the arithmetic that yields `v`.
+__device__ __forceinline__ int zero_after(float v) {
+    int z = 0;
+    asm volatile("" : "+v"(z) : "v"(v));
+    return z;
+}
+__device__ __forceinline__ int zero_after(cfloat v) { return zero_after(v.re); }
+
 __device__ __forceinline__ float vmul(float a, float b) { return a * b; }
 __device__ __forceinline__ float vfma(float a, float b, float c) { return __builtin_fmaf(a, b, c); }
 __device__ __forceinline__ float vconj(float a) { return a; }
