@@ -60,9 +60,13 @@ __global__ void __launch_bounds__(64 * kMaxWavesPerBlock)
     // 0.787, and T = 12000 0.467 -> 0.455).  Held back everywhere, the kernels that own whole rows lose
     // (nothing to wait for after pass 1: bf16 (8,1536,12000) backward 0.26 -> 0.31 ms) and so do the
     // swept 16-bit ones (wave 0 sets its vectors aside before it looks and then waits for them: bf16
-    // (8,1536,65533) 1.37 -> 1.48 ms), so the switch is for the fp32 kernels with masking code.
-    constexpr bool STATES_LATE = SPLIT == kSweep && !REGULAR && ACT == kGateIdentity && !Tr::kNarrow &&
-                                 std::is_same<V, float>::value;
+    // (8,1536,65533) 1.37 -> 1.48 ms), so the switch is for the fp32 kernels with masking code -- and
+    // for the mask-free fp32 kernels of the gates with values, which hold the values back as well (two
+    // of their four inputs, 2 KiB of each per wave: (8,1536,65536) interpolating gate 3.11 -> 2.90 ms,
+    // normalised exponential gate 3.23 -> 3.07; their copies with masking code lose, (8,1536,20000)
+    // 0.93 -> 1.00 ms, and so do the sigmoid and exponential gates' kernels, 2.46 -> 2.52).
+    constexpr bool STATES_LATE = SPLIT == kSweep && ((!REGULAR && ACT == kGateIdentity) || (REGULAR && LERP)) &&
+                                 !Tr::kNarrow && std::is_same<V, float>::value;
 
     const int lane = threadIdx.x & 63;
     // Packed rows: this workgroup scans rows [first_row, first_row + nrows) as one row of `len` elements.
@@ -249,7 +253,11 @@ __global__ void __launch_bounds__(64 * kMaxWavesPerBlock)
                 } else {
                     xraw[j] = load_raw<Tr, ALIGNED, FULL>(xsub, off, win, x_start);
                 }
-                if constexpr (LERP) vraw[j] = load_raw<Tr, ALIGNED, FULL>(vsub, off, win, vzero<V>());
+                if constexpr (LERP && STATES_LATE) {
+                    vraw[j] = fill_raw<Tr>(vzero<V>());
+                } else if constexpr (LERP) {
+                    vraw[j] = load_raw<Tr, ALIGNED, FULL>(vsub, off, win, vzero<V>());
+                }
             }
         } else {
 #pragma unroll
@@ -353,6 +361,9 @@ __global__ void __launch_bounds__(64 * kMaxWavesPerBlock)
 #pragma unroll
                 for (int j = 0; j < U; ++j) {
                     xraw[j] = load_raw<Tr, ALIGNED, FULL>(xsub, vec_offset<U, EPV, REV>(j, lane) + late, win, x_start);
+                    if constexpr (LERP) {
+                        vraw[j] = load_raw<Tr, ALIGNED, FULL>(vsub, vec_offset<U, EPV, REV>(j, lane) + late, win, vzero<V>());
+                    }
                 }
             }
         }
