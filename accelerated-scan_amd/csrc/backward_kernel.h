@@ -50,23 +50,29 @@ __global__ void __launch_bounds__(64 * kMaxWavesPerBlock)
     constexpr int E_FIRST = REV ? Tr::EPV - 1 : 0;
     constexpr int E_LAST = REV ? 0 : Tr::EPV - 1;
     constexpr int NIN = LERP ? 4 : 3;
-    // The states are needed by pass 2 only.  Requested after pass 1, they travel while the tile looks
-    // at the table (about 3 us under load, in which nothing else of this compute unit's is in flight),
-    // and the compiler schedules the state loads that way, or halfway through pass 1, in most swept
-    // instantiations by itself.  In the fp32 kernel for reverse scans with rows of any start and length
-    // it put all twelve loads up front, and that kernel was the slower of two mirror images: measured at
-    // (8,1536,T), compiler's order -> states held back, T = 65533 2.53 -> 2.44 ms, 50001 2.01 -> 1.90,
-    // 20000 0.885 -> 0.787 (its mirror image for forward scans: 2.45 -> 2.43, 1.89 -> 1.89, 0.783 ->
-    // 0.787, and T = 12000 0.467 -> 0.455).  Held back everywhere, the kernels that own whole rows lose
-    // (nothing to wait for after pass 1: bf16 (8,1536,12000) backward 0.26 -> 0.31 ms) and so do the
-    // swept 16-bit ones (wave 0 sets its vectors aside before it looks and then waits for them: bf16
-    // (8,1536,65533) 1.37 -> 1.48 ms), so the switch is for the fp32 kernels with masking code -- and
-    // for the mask-free fp32 kernels of the gates with values, which hold the values back as well (two
-    // of their four inputs, 2 KiB of each per wave: (8,1536,65536) interpolating gate 3.11 -> 2.90 ms,
-    // normalised exponential gate 3.23 -> 3.07; their copies with masking code lose, (8,1536,20000)
-    // 0.93 -> 1.00 ms, and so do the sigmoid and exponential gates' kernels, 2.46 -> 2.52).
-    constexpr bool STATES_LATE = SPLIT == kSweep && ((!REGULAR && ACT == kGateIdentity) || (REGULAR && LERP)) &&
-                                 !Tr::kNarrow && std::is_same<V, float>::value;
+    // The states (and the values of a gate with values) are needed by pass 2 only.  Requested after pass 1,
+    // they travel while the tile looks at the table -- about 3 us under load in which nothing else of this
+    // compute unit's is in flight -- and wave 0, which does the looking, leaves them in flight into their
+    // registers instead of setting them aside with the rest.  The compiler orders the loads that way, or
+    // halfway through pass 1, in most swept instantiations by itself; where it does not, holding them back
+    // by hand pays, and where it does, the hand-made order is the worse one.  Measured, backward kernel,
+    // ms, compiler's order -> states held back, (8,1536,T) unless said otherwise:
+    //   fp32, rows of any start and length: reverse scans (all twelve loads were up front, and the kernel
+    //   trailed its mirror image by 3.4 %) T = 65533 2.53 -> 2.44, 50001 2.01 -> 1.90, 20000 0.885 -> 0.785;
+    //   forward scans 2.45 -> 2.43, 1.89 -> 1.89, 0.783 -> 0.787, 12000 0.467 -> 0.456;
+    //   fp32 mask-free, gates with values (half of a tile's reads): interpolating gate 3.11 -> 2.89,
+    //   normalised exponential gate 3.23 -> 2.93; with masking code 50001 2.42 -> 2.34 but 20000 0.93 -> 1.00;
+    //   fp32 mask-free, identity 2.437 -> 2.448, sigmoid and exponential gate 2.46 -> 2.53;
+    //   bf16 / fp16 mask-free: identity 1.240 -> 1.239, exponential gate 1.31 -> 1.25 (fp16 the same);
+    //   with masking code T = 65533 1.38 -> 1.43;
+    //   complex64 (1,16,524288) 0.081 -> 0.075, (1,16,500001) 0.087 -> 0.085, (1,3,4000000) 0.118 -> 0.112.
+    // So the switch is on for the classes that gain.  The kernels that own whole rows never hold loads
+    // back: nothing to wait for follows pass 1 (bf16 (8,1536,12000) 0.26 -> 0.31 ms when they did).
+    constexpr bool kReal32 = !Tr::kNarrow && std::is_same<V, float>::value;
+    constexpr bool STATES_LATE =
+        SPLIT == kSweep && (kReal32       ? (!REGULAR && ACT == kGateIdentity) || (REGULAR && LERP)
+                            : Tr::kNarrow ? REGULAR && ACT == kGateExp
+                                          : true);
 
     const int lane = threadIdx.x & 63;
     // Packed rows: this workgroup scans rows [first_row, first_row + nrows) as one row of `len` elements.
@@ -377,8 +383,10 @@ __global__ void __launch_bounds__(64 * kMaxWavesPerBlock)
                     for (int j = 0; j < U; ++j) {
                         parked[(NIN * j) * 64 + lane] = araw[j];
                         parked[(NIN * j + 1) * 64 + lane] = draw[j];
-                        parked[(NIN * j + 2) * 64 + lane] = xraw[j];
-                        if constexpr (LERP) parked[(NIN * j + 3) * 64 + lane] = vraw[j];
+                        if constexpr (!STATES_LATE) {  // late loads stay in flight into their registers
+                            parked[(NIN * j + 2) * 64 + lane] = xraw[j];
+                            if constexpr (LERP) parked[(NIN * j + 3) * 64 + lane] = vraw[j];
+                        }
                         parked_values[(4 * j) * 64 + lane] = a_next[j];
                         parked_values[(4 * j + 1) * 64 + lane] = x_prev[j];
                         parked_values[(4 * j + 2) * 64 + lane] = exA[j];
@@ -390,8 +398,10 @@ __global__ void __launch_bounds__(64 * kMaxWavesPerBlock)
                     for (int j = 0; j < U; ++j) {
                         araw[j] = parked[(NIN * j) * 64 + lane];
                         draw[j] = parked[(NIN * j + 1) * 64 + lane];
-                        xraw[j] = parked[(NIN * j + 2) * 64 + lane];
-                        if constexpr (LERP) vraw[j] = parked[(NIN * j + 3) * 64 + lane];
+                        if constexpr (!STATES_LATE) {
+                            xraw[j] = parked[(NIN * j + 2) * 64 + lane];
+                            if constexpr (LERP) vraw[j] = parked[(NIN * j + 3) * 64 + lane];
+                        }
                         a_next[j] = parked_values[(4 * j) * 64 + lane];
                         x_prev[j] = parked_values[(4 * j + 1) * 64 + lane];
                         exA[j] = parked_values[(4 * j + 2) * 64 + lane];
