@@ -134,7 +134,7 @@ int backward_typed(const BackwardBuffers& b, int64_t rows, int64_t T, int act, c
         const bool regular = lead == 0 && T % (SUBS * kSplitWaves) == 0;
         const int64_t tile = (regular ? SUBS : SUBSG) * kSplitWaves;
         const int64_t ntiles = host_tiles_per_row<Tr>(T, tile, regular, at);
-        if (want_split(kSweepClass<Tr>, rows, T * kElem, tile * kElem, ntiles, act, false) && workspace_fits(ws, rows, ntiles)) {
+        if (want_split(kSweepClass<Tr>, rows, T * kElem, tile * kElem, ntiles, act, false, regular) && workspace_fits(ws, rows, ntiles)) {
             err = with_gate<Tr, REV>(act, [&](auto gate) {
                 constexpr int ACT = decltype(gate)::value;
                 return regular ? launch_backward_split<Tr, REV, true, ACT, kSweep>(b, rows, T, at.grid, ntiles, 0, ws, stream)

@@ -63,15 +63,16 @@ __global__ void __launch_bounds__(64 * kMaxWavesPerBlock)
     //   fp32 mask-free, gates with values (half of a tile's reads): interpolating gate 3.11 -> 2.89,
     //   normalised exponential gate 3.23 -> 2.93; with masking code 50001 2.42 -> 2.34 but 20000 0.93 -> 1.00;
     //   fp32 mask-free, identity 2.437 -> 2.448, sigmoid and exponential gate 2.46 -> 2.53;
-    //   bf16 / fp16 mask-free: identity 1.240 -> 1.239, exponential gate 1.31 -> 1.25 (fp16 the same);
-    //   with masking code T = 65533 1.38 -> 1.43;
+    //   bf16 / fp16 mask-free: identity 1.240 -> 1.239, exponential gate 1.31 -> 1.25 (fp16 the same), and
+    //   the sigmoid and the interpolating gate, which lost when swept before, now gain on whole rows per
+    //   workgroup (1.46 -> 1.33, 1.73 -> 1.59); with masking code T = 65533 identity 1.38 -> 1.43;
     //   complex64 (1,16,524288) 0.081 -> 0.075, (1,16,500001) 0.087 -> 0.085, (1,3,4000000) 0.118 -> 0.112.
     // So the switch is on for the classes that gain.  The kernels that own whole rows never hold loads
     // back: nothing to wait for follows pass 1 (bf16 (8,1536,12000) 0.26 -> 0.31 ms when they did).
     constexpr bool kReal32 = !Tr::kNarrow && std::is_same<V, float>::value;
     constexpr bool STATES_LATE =
         SPLIT == kSweep && (kReal32       ? (!REGULAR && ACT == kGateIdentity) || (REGULAR && LERP)
-                            : Tr::kNarrow ? REGULAR && ACT == kGateExp
+                            : Tr::kNarrow ? REGULAR && ACT != kGateIdentity
                                           : true);
 
     const int lane = threadIdx.x & 63;

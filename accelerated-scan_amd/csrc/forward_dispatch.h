@@ -116,7 +116,7 @@ int forward_typed(const void* gates, const void* tokens, void* out, const void* 
         const bool regular = lead == 0 && T % (SUBS * kSplitWaves) == 0;
         const int64_t tile = (regular ? SUBS : SUBSG) * kSplitWaves;
         const int64_t ntiles = host_tiles_per_row<Tr>(T, tile, regular, at);
-        if (want_split(kSweepClass<Tr>, rows, T * kElem, tile * kElem, ntiles, act, true) && workspace_fits(ws, rows, ntiles)) {
+        if (want_split(kSweepClass<Tr>, rows, T * kElem, tile * kElem, ntiles, act, true, regular) && workspace_fits(ws, rows, ntiles)) {
             auto go = [&](auto rev, auto reg, auto gate) {
                 return launch_forward_split<Tr, decltype(rev)::value, decltype(reg)::value, decltype(gate)::value,
                                             kSweep>(gates, tokens, out, initial, rows, T, at.grid, ntiles, 0, ws,

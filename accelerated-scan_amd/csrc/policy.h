@@ -238,16 +238,23 @@ bool too_few_rows(int64_t rows, int64_t ntiles) {
 }
 
 // `row_bytes`: one row of states; `tile_bytes`, `ntiles`: of the kernel that would run;
-// `act`: its gate; `forward`: the forward kernel (3 tensors per tile) or the backward one (5 or 6).  A compute unit holds one
-// swept workgroup, so what a tile costs in arithmetic is not hidden behind another
-// workgroup's loads: the 16-bit kernels that evaluate a sigmoid (or the normalised
+// `act`: its gate; `forward`: the forward kernel (3 tensors per tile) or the backward one
+// (5 or 6); `mask_free`: the kernel for rows of whole tiles on the grid.  A compute unit
+// holds one swept workgroup, so what a tile costs in arithmetic is not hidden behind another
+// workgroup's loads: the 16-bit forward kernels that evaluate a sigmoid (or the normalised
 // exponential gate's scale) for eight elements per vector lose when swept (bf16
-// (8,1536,65536), % of peak, whole rows -> swept: sigmoid 70 -> 67, interpolating gate
-// 72 -> 64, normalised exponential 71 -> 58; the plain exponential 73 -> 75 and the fp32
-// kernels of all gates 72 -> 78-81), and so does a forward kernel with 32 KiB tiles (the
-// normalised exponential gate's, fp32: 6.0 -> 5.3 TB/s) -- the backward kernels move five
-// or six tensors per tile and do well with 32 KiB of each.
-bool want_split(SweepClass c, int64_t rows, int64_t row_bytes, int64_t tile_bytes, int64_t ntiles, int act, bool forward) {
+// (8,1536,65536), ms, whole rows -> swept: sigmoid 0.79 -> 0.92, interpolating gate 0.80 ->
+// 0.97, normalised exponential 0.81 -> 1.20; the plain exponential gains, and so do the fp32
+// kernels of all gates, 72 -> 78-82 % of peak), and so does a forward kernel with 32 KiB
+// tiles (the normalised exponential gate's, fp32: 6.0 -> 5.3 TB/s).  The backward kernels
+// move five or six tensors per tile, do well with 32 KiB of each, and request the states
+// behind pass 1 so that they travel while the tile looks at the table; swept, the mask-free
+// 16-bit ones of the sigmoid and the interpolating gate gain (bf16 (8,1536,65536) backward
+// 1.46 -> 1.33 and 1.73 -> 1.59 ms, T = 32768 0.79 -> 0.71 and 0.93 -> 0.79, fp16 alike; the
+// normalised exponential gate's 1.72 -> 1.72), their copies with masking code do not
+// (T = 65533: sigmoid 1.53 -> 1.63, interpolating gate 1.92 -> 1.86).
+bool want_split(SweepClass c, int64_t rows, int64_t row_bytes, int64_t tile_bytes, int64_t ntiles, int act, bool forward,
+                bool mask_free) {
     if (rows > split_max_rows()) return false;
     if (too_few_rows(rows, ntiles)) return true;
     if (split_forced_min_row_bytes() > 0) return row_bytes >= split_forced_min_row_bytes();
@@ -264,7 +271,9 @@ bool want_split(SweepClass c, int64_t rows, int64_t row_bytes, int64_t tile_byte
     switch (c) {
         case SweepClass::kF32: return percent_full >= (forward ? (ntiles == 1 ? 80 : 55) : 50);
         case SweepClass::kNarrow:
-            return row_bytes >= kSweepTileBytes && percent_full >= 66 && (act == kGateIdentity || act == kGateExp);
+            return row_bytes >= kSweepTileBytes && percent_full >= 66 &&
+                   (act == kGateIdentity || act == kGateExp ||
+                    (!forward && mask_free && (act == kGateSigmoid || act == kGateSigmoidLerp)));
         default: return false;
     }
 }
