@@ -231,6 +231,17 @@ constexpr SweepClass kSweepClass = Tr::kNarrow ? SweepClass::kNarrow
                                                : (std::is_same<typename Tr::V, float>::value ? SweepClass::kF32
                                                                                              : SweepClass::kComplex);
 
+// complex64: many rows.  The forward kernel loses when swept whatever the shape (32 KiB tiles, twice
+// the arithmetic per byte: (8,768,65536) 1.65 -> 2.05 ms).  The mask-free backward kernel, which
+// requests the states behind pass 1, gains on rows of 64 to 512 KiB when there are more than two per
+// compute unit: (8,768,65536) 2.89 -> 2.73 ms, (8,768,32768) 1.41 -> 1.31, (4,1024,8192) 0.235 -> 0.219,
+// (1,2048,32768) 0.476 -> 0.444, (1,512,32768) 0.129 -> 0.123; rows of 1 MiB are level ((1,1024,131072)
+// 0.955 -> 0.966), 256 rows lose (0.124 -> 0.130) and so does the kernel with masking code
+// ((8,768,65533) 2.94 -> 3.18).
+bool complex_rows_swept(int64_t rows, int64_t row_bytes) {
+    return rows >= 512 && row_bytes >= kSweepTileBytes && row_bytes <= 8 * kSweepTileBytes;
+}
+
 // Too few rows to occupy the compute units with one workgroup each: with up to 64
 // rows two tiles per row already pay; up to 128, four.
 bool too_few_rows(int64_t rows, int64_t ntiles) {
@@ -274,7 +285,7 @@ bool want_split(SweepClass c, int64_t rows, int64_t row_bytes, int64_t tile_byte
             return row_bytes >= kSweepTileBytes && percent_full >= 66 &&
                    (act == kGateIdentity || act == kGateExp ||
                     (!forward && mask_free && (act == kGateSigmoid || act == kGateSigmoidLerp)));
-        default: return false;
+        default: return !forward && mask_free && complex_rows_swept(rows, row_bytes);
     }
 }
 
@@ -289,7 +300,7 @@ bool may_split(SweepClass c, int64_t rows, int64_t row_bytes, int64_t ntiles_mos
         case SweepClass::kNarrow:
             return row_bytes >= kSweepTileBytes ||
                    (row_bytes == kSweepTileBytes / 2 && rows * row_bytes >= kSweepRowsMinBytes);  // two rows per tile
-        default: return false;
+        default: return complex_rows_swept(rows, row_bytes);
     }
 }
 
