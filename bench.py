@@ -353,6 +353,11 @@ def run_sweep(path, steps, warmup):
                     x = tokens.clone().requires_grad_(True)
                     ms = time_call(lambda: torch.autograd.grad(warp_scan(g, x), (g, x), grad_out), steps, warmup, min_ms)
                     rec["train_ms"], rec["train_GBps"] = ms, 8 * nbytes / ms / 1e6
+                    if T <= 2048:  # where the host cost shows: the same with the process on one core
+                        with one_core():
+                            ms = time_call(lambda: torch.autograd.grad(warp_scan(g, x), (g, x), grad_out), steps, warmup,
+                                           min_ms)
+                        rec["train_one_core_ms"], rec["train_one_core_GBps"] = ms, 8 * nbytes / ms / 1e6
                     del g, x
                 # forward + backward captured once into a HIP graph and replayed: what a caller reaches who
                 # takes the per-call host cost (Python, autograd, allocation) out of the loop
@@ -382,6 +387,33 @@ def run_sweep(path, steps, warmup):
     write_sweep_csv(records, str(path))
 
 
+class one_core:
+    """Pins every thread of this process to one of its cores for the duration.  A decode-sized
+    autograd step is a hand-over between the calling thread and autograd's backward thread (and the
+    HIP runtime's own threads); on these virtual hosts a wake-up across cores costs tens of
+    microseconds in some processes and not in others, and a process confined to one core
+    (`taskset -c N python ...` does the same from outside) never pays it."""
+
+    def __enter__(self):
+        self.allowed = os.sched_getaffinity(0)
+        self.threads = [int(t) for t in os.listdir("/proc/self/task")]
+        core = {sorted(self.allowed)[0]}
+        for t in self.threads:
+            try:
+                os.sched_setaffinity(t, core)
+            except OSError:
+                pass  # a thread that ended meanwhile
+        return self
+
+    def __exit__(self, *exc):
+        for t in self.threads:
+            try:
+                os.sched_setaffinity(t, self.allowed)
+            except OSError:
+                pass
+        return False
+
+
 def graphed_step(gates, tokens, grad_out, out, d_gates, d_tokens):
     """Captures one forward + backward through the C ABI (outputs and tables allocated
     beforehand) into a HIP graph; returns the function that replays it."""
@@ -409,7 +441,7 @@ def graphed_step(gates, tokens, grad_out, out, d_gates, d_tokens):
     return graph.replay
 
 
-SWEEP_DIRECTIONS = ("forward", "reverse", "backward", "train", "train_graph")
+SWEEP_DIRECTIONS = ("forward", "reverse", "backward", "train", "train_one_core", "train_graph")
 
 
 def write_sweep_csv(records, stem):
@@ -451,15 +483,19 @@ def write_sweep_markdown(records, path, steps, warmup):
                 f"least {steps} calls and 40 ms after at least {warmup} calls and 20 ms of warm-up, HIP events; one set of buffers per point, so tensors up to a few hundred MB "
                 "see some Infinity Cache hits). Cells: ms per call (algorithmic TB/s). forward / reverse / backward "
                 "are kernel calls through the C ABI; train = autograd forward + backward of `warp.scan`, "
-                "allocation included; train (graph) = forward + backward through the C ABI captured once into a "
-                "HIP graph and replayed, i.e. without the per-call host cost.\n")
+                "allocation included; train (one core) = the same with every thread of the process pinned to one core "
+                "(T <= 2048, where the host cost shows: on these virtual hosts the hand-over between the calling thread "
+                "and autograd's backward thread costs tens of microseconds across cores in some processes, none on one "
+                "core; `taskset -c N` from outside does the same); train (graph) = forward + backward through the C ABI "
+                "captured once into a HIP graph and replayed, i.e. without the per-call host cost.\n")
         for dt in ("fp32", "bf16"):
-            f.write(f"\n## {dt}, shape (8, 1536, T)\n\n| T | forward | reverse | backward | train | train (graph) |\n"
-                    "|---|---|---|---|---|---|\n")
+            f.write(f"\n## {dt}, shape (8, 1536, T)\n\n| T | forward | reverse | backward | train | train (one core) | "
+                    "train (graph) |\n|---|---|---|---|---|---|---|\n")
             for rec in records:
                 if rec["dtype"] == dt:
                     f.write(f"| {rec['shape'][2]} | {cell(rec, 'forward')} | {cell(rec, 'reverse')} | "
-                            f"{cell(rec, 'backward')} | {cell(rec, 'train')} | {cell(rec, 'train_graph')} |\n")
+                            f"{cell(rec, 'backward')} | {cell(rec, 'train')} | {cell(rec, 'train_one_core')} | "
+                            f"{cell(rec, 'train_graph')} |\n")
         for rec in records:
             if rec["dtype"] == "c64":
                 f.write(f"\n## complex64, shape {tuple(rec['shape'])} (tests/bench_complex.py:79-90 of the reference)\n\n"
