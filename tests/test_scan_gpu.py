@@ -878,6 +878,36 @@ def test_sweep_of_many_long_rows(dtype, rows, T):
     _compare_with_truth(gates, tokens, grad_out, out, rev, dg, dx, dtype, what="sweep", reverse_grads=(rdg, rdx))
 
 
+@pytest.mark.parametrize("dtype", [torch.complex64, C64_REAL_TOKENS], ids=["c64", "c64-real-tokens"])
+@pytest.mark.parametrize("rows,T", [(600, 8192), (513, 32768), (700, 12288)])
+def test_sweep_of_many_complex_rows(dtype, rows, T):
+    """Complex rows of 64 to 512 KiB, 512 of them and more: the forward kernel keeps one workgroup per
+    row, the mask-free backward kernel is swept by ticket (32 KiB tiles, states requested after its
+    first pass).  Both scan directions against the fp64 loops; no wait may have run out."""
+    from accelerated_scan import _abi
+
+    lib = _abi.load()
+    code = _abi.dtype_code(torch.complex64, torch.float32 if dtype == C64_REAL_TOKENS else torch.complex64)
+    nbytes = lib.ascan_workspace_bytes(rows, T, code)
+    assert nbytes > 0, "the backward kernel of this shape is meant to be swept"
+    gates, tokens, grad_out = _truth_inputs(rows, T, dtype, seed=rows + T)
+    g, x, d = (t.to(DEVICE).reshape(1, rows, T) for t in (gates, tokens, grad_out))
+    out, rev, dg = (torch.empty_like(g) for _ in range(3))
+    dx = torch.empty_like(x)
+    spaces = [torch.ones(nbytes, dtype=torch.uint8, device=DEVICE) for _ in range(2)]  # garbage: cleared by the call
+    _abi.forward(g, x, out, False)
+    _abi.forward(g, x, rev, True)
+    _abi.backward(g, out, d, dg, dx, workspace=spaces[0])
+    rdg, rdx = torch.empty_like(g), torch.empty_like(x)
+    _abi.backward(g, rev, d, rdg, rdx, workspace=spaces[1], reverse=True)
+    torch.cuda.synchronize()
+    assert [_abi.workspace_timeouts(w) for w in spaces] == [0, 0]
+    for table in spaces:  # the backward launches drew a ticket per 32 KiB tile and one per workgroup at the end
+        drawn = int.from_bytes(bytes(table[64:72].cpu().tolist()), "little")
+        assert drawn >= rows * (T // 4096), drawn
+    _compare_with_truth(gates, tokens, grad_out, out, rev, dg, dx, dtype, what="complex sweep", reverse_grads=(rdg, rdx))
+
+
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.float16], ids=["fp32", "bf16", "fp16"])
 def test_rows_of_half_a_tile_share_swept_tiles(dtype):
     """Rows of exactly 32 KiB, enough of them for 256 MiB per tensor: with a table the library
