@@ -232,7 +232,9 @@ int ascan_backward(const void* gates, const void* states, const void* grad_out, 
                             ASCAN_GATE_IDENTITY, false, Workspace{nullptr, 0}, stream);
 }
 
-size_t ascan_workspace_bytes(int64_t rows, int64_t seqlen, int dtype) {
+namespace {
+// Size of the table for a call (`forward_only`: for the identity gate's forward kernel alone).
+size_t table_bytes(int64_t rows, int64_t seqlen, int dtype, bool forward_only) {
     const size_t es = element_size(dtype);
     if (es == 0 || rows <= 0 || seqlen <= 0 || !shape_ok(rows, seqlen)) return 0;
     // the smallest split tile any kernel uses for this dtype: 2 blocks of 64 vectors per wave
@@ -243,9 +245,15 @@ size_t ascan_workspace_bytes(int64_t rows, int64_t seqlen, int dtype) {
     const int64_t ntiles = (seqlen + head + tile - 1) / tile;
     const SweepClass c = dtype == ASCAN_F32 ? SweepClass::kF32
                          : (dtype == ASCAN_BF16 || dtype == ASCAN_F16 ? SweepClass::kNarrow : SweepClass::kComplex);
-    if (!may_split(c, rows, seqlen * (int64_t)es, ntiles) || rows > 2147483647LL / ntiles) return 0;
-    return split_bytes(rows, ntiles);
+    if (may_split(c, rows, seqlen * (int64_t)es, ntiles, forward_only) && rows <= 2147483647LL / ntiles) {
+        return split_bytes(rows, ntiles);
+    }
+    if (forward_only && forward_needs_ticket_only(c, rows, seqlen * (int64_t)es)) return split_bytes(0, 1);
+    return 0;
 }
+}  // namespace
+
+size_t ascan_workspace_bytes(int64_t rows, int64_t seqlen, int dtype) { return table_bytes(rows, seqlen, dtype, false); }
 
 int ascan_forward_split(const void* gates, const void* tokens, void* out, int64_t rows, int64_t seqlen, int dtype,
                         int reverse, void* workspace, size_t workspace_bytes, void* stream) {
@@ -255,7 +263,8 @@ int ascan_forward_split(const void* gates, const void* tokens, void* out, int64_
 
 int ascan_forward_split_static(const void* gates, const void* tokens, void* out, int64_t rows, int64_t seqlen,
                                int dtype, int reverse, void* stream) {
-    const size_t needed = ascan_workspace_bytes(rows, seqlen, dtype);
+    // what this call's one kernel may use: less than ascan_workspace_bytes where only a backward kernel is swept
+    const size_t needed = table_bytes(rows, seqlen, dtype, true);
     if (needed > (size_t)ASCAN_STATIC_WORKSPACE_BYTES) return ASCAN_ERR_TOO_LARGE;
     Workspace ws{nullptr, 0};
     // needed == 0: rows that are not split (or arguments the checks below refuse) use no table

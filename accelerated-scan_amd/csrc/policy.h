@@ -289,19 +289,25 @@ bool want_split(SweepClass c, int64_t rows, int64_t row_bytes, int64_t tile_byte
     }
 }
 
-// Whether some kernel of a call of this shape may want the table (`ntiles_most`: with
-// the smallest tile any kernel uses): what ascan_workspace_bytes goes by.
-bool may_split(SweepClass c, int64_t rows, int64_t row_bytes, int64_t ntiles_most) {
+// Whether some kernel of a call of this shape may want the table with its records (`ntiles_most`:
+// with the smallest tile any kernel uses): what ascan_workspace_bytes goes by.  `forward_only`: the
+// identity gate's forward kernel alone (the entry point with the table in the library's own array).
+bool may_split(SweepClass c, int64_t rows, int64_t row_bytes, int64_t ntiles_most, bool forward_only) {
     if (rows > split_max_rows()) return false;
     if (too_few_rows(rows, ntiles_most)) return true;
     if (split_forced_min_row_bytes() > 0) return row_bytes >= split_forced_min_row_bytes();
+    const bool half_tile_rows = row_bytes == kSweepTileBytes / 2 && rows * row_bytes >= kSweepRowsMinBytes;
     switch (c) {
-        case SweepClass::kF32: return row_bytes >= kSweepTileBytes / 2;
-        case SweepClass::kNarrow:
-            return row_bytes >= kSweepTileBytes ||
-                   (row_bytes == kSweepTileBytes / 2 && rows * row_bytes >= kSweepRowsMinBytes);  // two rows per tile
-        default: return complex_rows_swept(rows, row_bytes);
+        case SweepClass::kF32:  // a backward kernel takes half-full tiles, a forward kernel does not
+            return forward_only ? row_bytes > kSweepTileBytes / 2 : row_bytes >= kSweepTileBytes / 2;
+        case SweepClass::kNarrow: return row_bytes >= kSweepTileBytes || (!forward_only && half_tile_rows);
+        default: return !forward_only && complex_rows_swept(rows, row_bytes);
     }
+}
+// Rows swept two to a tile by the forward kernel need the ticket, not the records.
+bool forward_needs_ticket_only(SweepClass c, int64_t rows, int64_t row_bytes) {
+    return c != SweepClass::kComplex && rows <= split_max_rows() && sweep_rows_mode() != 0 &&
+           row_bytes == kSweepTileBytes / 2 && rows * row_bytes >= kSweepRowsMinBytes;
 }
 
 // Rows of exactly half a swept tile, starting on the grid: two whole rows per tile of a

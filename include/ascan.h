@@ -232,9 +232,12 @@ ASCAN_API unsigned int ascan_workspace_timeouts(const void* workspace_header_cop
  *
  *   - the array holds ASCAN_STATIC_WORKSPACE_BYTES on every GPU the library is
  *     used on, from the first call on that GPU until the process ends;
- *   - a problem whose table (ascan_workspace_bytes) is larger is refused with
- *     ASCAN_ERR_TOO_LARGE and nothing is launched; problems that are not split
- *     (ascan_workspace_bytes == 0) run the plain kernels and use no table;
+ *   - a problem whose table would be larger is refused with ASCAN_ERR_TOO_LARGE
+ *     and nothing is launched.  The table meant is that of this call's one
+ *     kernel, the identity gate's forward kernel: at most ascan_workspace_bytes,
+ *     and less where only a backward kernel of the shape would be swept.
+ *     Problems whose forward kernel is not swept run the plain kernel and use
+ *     no table;
  *   - all calls on one GPU share that GPU's array (it is cleared by a small
  *     kernel on `stream` at the start of each call): two calls that may run at
  *     the same time on one GPU -- different streams, or graph branches -- race

@@ -101,6 +101,33 @@ def test_static_table_limit_and_unsplit_shapes():
     _abi.check(lib.ascan_forward_split_static(g.data_ptr(), x.data_ptr(), out.data_ptr(), 4, 256, 0, 0, stream))
     torch.cuda.synchronize()
     assert torch.equal(out, want)
+    # a shape of which only the backward kernel would be swept (many complex rows of 64 KiB): ascan_workspace_bytes
+    # reports a table beyond the array's size, but the forward kernel takes none, so the call is not refused
+    rows, T = 24000, 8192
+    assert lib.ascan_workspace_bytes(rows, T, 3) > 4 * 1024 * 1024
+    cg = torch.polar(0.5 + 0.5 * torch.rand(rows, T, device=DEVICE), 6.28 * torch.rand(rows, T, device=DEVICE))
+    cx = torch.randn(rows, T, device=DEVICE, dtype=torch.complex64)
+    cout, cwant = torch.empty_like(cx), torch.empty_like(cx)
+    _abi.check(lib.ascan_forward(cg.data_ptr(), cx.data_ptr(), cwant.data_ptr(), rows, T, 3, 0, stream))
+    _abi.check(lib.ascan_forward_split_static(cg.data_ptr(), cx.data_ptr(), cout.data_ptr(), rows, T, 3, 0, stream))
+    torch.cuda.synchronize()
+    assert torch.equal(torch.view_as_real(cout), torch.view_as_real(cwant))
+    del cg, cx, cout, cwant
+    # rows of half a tile, two to a swept tile: the forward kernel needs the ticket only, whatever the number of rows
+    rows, T = 40000, 8192
+    assert lib.ascan_workspace_bytes(rows, T, 0) > 4 * 1024 * 1024
+    hg, hx = torch.rand(rows, T, device=DEVICE), torch.rand(rows, T, device=DEVICE)
+    hout, hwant = torch.empty_like(hx), torch.empty_like(hx)
+    table = torch.empty(lib.ascan_workspace_bytes(rows, T, 0), dtype=torch.uint8, device=DEVICE)
+    _abi.check(lib.ascan_forward_split(hg.data_ptr(), hx.data_ptr(), hwant.data_ptr(), rows, T, 0, 0, table.data_ptr(),
+                                       table.numel(), stream))
+    _abi.check(lib.ascan_forward_split_static(hg.data_ptr(), hx.data_ptr(), hout.data_ptr(), rows, T, 0, 0, stream))
+    torch.cuda.synchronize()
+    assert torch.equal(hout, hwant)
+    count = ctypes.c_uint(7)
+    _abi.check(lib.ascan_static_workspace_timeouts(ctypes.byref(count), stream))
+    assert count.value == 0
+    del hg, hx, hout, hwant, table
     # validation is that of the other entry points
     assert lib.ascan_forward_split_static(None, x.data_ptr(), out.data_ptr(), 4, 256, 0, 0, stream) == 1
     assert lib.ascan_forward_split_static(g.data_ptr(), x.data_ptr(), out.data_ptr(), 4, 256, 9, 0, stream) == 3
