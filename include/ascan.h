@@ -180,9 +180,12 @@ ASCAN_API int ascan_backward(const void* gates, const void* states, const void* 
  * sequence (warp.cuh:279; scalar.py:98; complex.py:174).
  *
  *   ascan_workspace_bytes  size of the table for a problem, or 0 when no kernel
- *                          would use one (short rows; many complex64 rows): then
- *                          the calls behave exactly like the plain ones and
- *                          ignore the workspace.  Otherwise 128 bytes plus 64
+ *                          would use one (short rows; complex64 rows beyond
+ *                          512 KiB unless they are few): then the calls behave
+ *                          exactly like the plain ones and ignore the workspace.
+ *                          Which kernels of a shape are swept is decided per
+ *                          kernel (of complex64 and of the 16-bit gates with a
+ *                          sigmoid, the backward kernel only).  Otherwise 128 bytes plus 64
  *                          bytes per tile, a few MB at most for tensors of GBs;
  *   workspace              device memory, 64-byte aligned, at least that many
  *                          bytes, not shared with another call that may run at
