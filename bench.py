@@ -358,6 +358,14 @@ def run_sweep(path, steps, warmup):
                             ms = time_call(lambda: torch.autograd.grad(warp_scan(g, x), (g, x), grad_out), steps, warmup,
                                            min_ms)
                         rec["train_one_core_ms"], rec["train_one_core_GBps"] = ms, 8 * nbytes / ms / 1e6
+                        # and with the backward pass run by the calling thread instead of autograd's device thread
+                        torch.autograd.set_multithreading_enabled(False)
+                        try:
+                            ms = time_call(lambda: torch.autograd.grad(warp_scan(g, x), (g, x), grad_out), steps, warmup,
+                                           min_ms)
+                        finally:
+                            torch.autograd.set_multithreading_enabled(True)
+                        rec["train_one_thread_ms"], rec["train_one_thread_GBps"] = ms, 8 * nbytes / ms / 1e6
                     del g, x
                 # forward + backward captured once into a HIP graph and replayed: what a caller reaches who
                 # takes the per-call host cost (Python, autograd, allocation) out of the loop
@@ -441,7 +449,7 @@ def graphed_step(gates, tokens, grad_out, out, d_gates, d_tokens):
     return graph.replay
 
 
-SWEEP_DIRECTIONS = ("forward", "reverse", "backward", "train", "train_one_core", "train_graph")
+SWEEP_DIRECTIONS = ("forward", "reverse", "backward", "train", "train_one_core", "train_one_thread", "train_graph")
 
 
 def write_sweep_csv(records, stem):
@@ -486,16 +494,18 @@ def write_sweep_markdown(records, path, steps, warmup):
                 "allocation included; train (one core) = the same with every thread of the process pinned to one core "
                 "(T <= 2048, where the host cost shows: on these virtual hosts the hand-over between the calling thread "
                 "and autograd's backward thread costs tens of microseconds across cores in some processes, none on one "
-                "core; `taskset -c N` from outside does the same); train (graph) = forward + backward through the C ABI "
+                "core; `taskset -c N` from outside does the same); train (one thread) = the same with "
+                "`torch.autograd.set_multithreading_enabled(False)`, which runs the backward pass on the calling thread "
+                "and takes the hand-over away; train (graph) = forward + backward through the C ABI "
                 "captured once into a HIP graph and replayed, i.e. without the per-call host cost.\n")
         for dt in ("fp32", "bf16"):
             f.write(f"\n## {dt}, shape (8, 1536, T)\n\n| T | forward | reverse | backward | train | train (one core) | "
-                    "train (graph) |\n|---|---|---|---|---|---|---|\n")
+                    "train (one thread) | train (graph) |\n|---|---|---|---|---|---|---|---|\n")
             for rec in records:
                 if rec["dtype"] == dt:
                     f.write(f"| {rec['shape'][2]} | {cell(rec, 'forward')} | {cell(rec, 'reverse')} | "
                             f"{cell(rec, 'backward')} | {cell(rec, 'train')} | {cell(rec, 'train_one_core')} | "
-                            f"{cell(rec, 'train_graph')} |\n")
+                            f"{cell(rec, 'train_one_thread')} | {cell(rec, 'train_graph')} |\n")
         for rec in records:
             if rec["dtype"] == "c64":
                 f.write(f"\n## complex64, shape {tuple(rec['shape'])} (tests/bench_complex.py:79-90 of the reference)\n\n"
