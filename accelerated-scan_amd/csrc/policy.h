@@ -182,11 +182,13 @@ inline int launch_status(hipError_t e) {
 // 32768 72 -> 82, 49152 65 -> 82, 65536 73 -> 82.5, and with rows of any start and
 // length 65533 68 -> 81, 100000 -> 82, 50001 -> 82, 33000 / 36000 70 -> 80, 20000 /
 // 22000 74 -> 78, 17000 (tiles 52 % full) 74 -> 75; a row of half a tile (8192)
-// 75 -> 72, but its backward pass alone gains (want_split).
+// 75 -> 72 in a tile of its own, though its backward pass alone gains (want_split),
+// and 77 -> 80 with two rows to a tile (sweep_rows_per_tile).
 // bf16 T = 32768 72 -> 81, 65536 74 -> 82, 49152 73 -> 78, 100000 / 131071 69 -> 74 /
 // 75, 45000 (tiles 69 % full) 71 -> 72, but 40000 (61 %) 72 -> 70 and 35000 (53 %)
-// 70 -> 61.  complex64 (8,768,65536) 71 -> 70 with 64 KiB forward tiles (which spill)
-// and 64 with 32 KiB ones.  A tile costs a ticket, a look at the table and three
+// 70 -> 61.  complex64 (8,768,65536) 71 -> 70 with both kernels swept (64 KiB forward
+// tiles, which spill; 64 with 32 KiB ones), 73 with the backward kernel alone
+// (complex_rows_swept).  A tile costs a ticket, a look at the table and three
 // barriers, about 2.4 us in which its compute unit requests nothing, whatever its
 // size: all swept kernels of the real dtypes take 64 KiB tiles (4 KiB per wave).
 // ASCAN_SPLIT_MAX_ROWS (0 = never split) and ASCAN_SPLIT_MIN_ROW_BYTES (split every
