@@ -48,15 +48,16 @@ __global__ void __launch_bounds__(64 * kMaxWavesPerBlock)
     __shared__ S stage_all[PACKED ? W * SUB : 1];
     // Split rows: the workgroups take tiles by ticket, in memory order, until none
     // is left; a workgroup only ever waits for tiles whose owners started before it.
-    __shared__ int split_mailbox[2];
+    __shared__ int split_mailbox[4];  // two mailboxes, taken in turn
     __shared__ u32x4_t parked[SPLIT ? 2 * U * 64 : 1];  // wave 0's raw vectors during its walk back
     const unsigned long long split_wait_limit = SPLIT == kSweep ? split->wait_limit : 0ull;  // the longest wait allowed
-    for (bool first_visit = true;; first_visit = false) {
+    int visit_parity = 0;
+    for (bool first_visit = true;; first_visit = false, visit_parity ^= 1) {
     int64_t row;
     int w, slot_base;
     int64_t k_begin = 0, k_end = ntiles;
     if constexpr (SPLIT) {
-        if (!take_split_tile(split, units, ntiles, row, k_begin, split_mailbox)) break;
+        if (!take_split_tile(split, units, ntiles, row, k_begin, split_mailbox + 2 * visit_parity)) break;
         k_end = k_begin + 1;
         int thread = threadIdx.x;
         asm volatile("" : "+v"(thread));  // nothing derived from the wave index is carried from visit to visit

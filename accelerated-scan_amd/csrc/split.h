@@ -133,7 +133,8 @@ __device__ __forceinline__ SplitRecord* split_records(SplitHeader* header) {
 
 // Hands the workgroup its next tile, or returns false when none is left: thread 0
 // draws the ticket, all threads of the workgroup call this together and get the
-// same answer through `mailbox` (two words of LDS).  rows * ntiles is below 2^31.
+// same answer through `mailbox` (two words of LDS; the caller alternates between two mailboxes from
+// call to call).  rows * ntiles is below 2^31.
 //
 // The ticket is drawn here, when the workgroup is ready to start on it, so tiles
 // start in ticket order.  (Drawn a tile step ahead, behind the previous tile's
@@ -163,7 +164,8 @@ __device__ __forceinline__ bool take_split_tile(SplitHeader* header, int64_t row
     __syncthreads();
     const int got_row = __builtin_amdgcn_readfirstlane(mailbox[0]);
     const int got_k = __builtin_amdgcn_readfirstlane(mailbox[1]);
-    __syncthreads();  // the mailbox may be rewritten by the next call
+    // (no second barrier: consecutive calls use alternate mailboxes, and a thread that is two calls
+    // ahead has passed the barrier of the call in between, which every thread reaches after this read)
     if (got_row < 0) return false;
     row = got_row;
     k = got_k;
