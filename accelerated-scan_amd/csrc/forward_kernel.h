@@ -202,9 +202,19 @@ __global__ void __launch_bounds__(64 * kMaxWavesPerBlock)
         // 16-bit storage with a gate non-linearity: eight exponentials and reciprocals per vector and
         // pass make the vector ALU the limit (about 5.4 TB/s for the interpolating gate), so the
         // activated gates and tokens of pass 1 are kept for pass 2; the raw vectors are dead by then.
-        // Everywhere else unpacking again is cheaper than the registers (the split-row kernels would spill).
-        constexpr bool KEEP = Tr::kNarrow && ACT != kGateIdentity && !PACKED && !SPLIT;
-        V gkeep[KEEP ? U : 1][EPV], tkeep[KEEP ? U : 1][EPV];
+        // The swept kernels have fewer registers to spare (wave 0 parks only its raw vectors), and one
+        // workgroup per compute unit hides none of the arithmetic: the mask-free ones keep the gates alone
+        // where the token needs no activation (measured, bf16 / fp16 (8,1536,65536), ms: sigmoid 0.92 / 0.89
+        // -> 0.76 / 0.73, against 0.80 on whole rows; exponential 0.83 / 0.81 -> 0.74 / 0.75), and gates
+        // and tokens at 2 KiB per wave for the normalised exponential gate (1.23 -> 0.94; whole rows 0.81).
+        // Keeping one word per element of the interpolating gate -- the smaller of gate and complement
+        // with the sign of the stored value -- made that kernel 0.96 -> 0.91, whole rows 0.80: not kept.
+        // Everywhere else unpacking again is cheaper than the registers (the kernels would spill).
+        constexpr bool SWEPT_MASK_FREE = SPLIT == kSweep && REGULAR;
+        constexpr bool KEEP =
+            Tr::kNarrow && ACT != kGateIdentity && !PACKED && (!SPLIT || (SWEPT_MASK_FREE && ACT == kGateExpNorm));
+        constexpr bool KEEP_GATES = Tr::kNarrow && SWEPT_MASK_FREE && (ACT == kGateSigmoid || ACT == kGateExp);
+        V gkeep[KEEP || KEEP_GATES ? U : 1][EPV], tkeep[KEEP ? U : 1][EPV];
 #pragma unroll
         for (int j = 0; j < U; ++j) {
             V g[EPV], t[EPV];
@@ -217,6 +227,10 @@ __global__ void __launch_bounds__(64 * kMaxWavesPerBlock)
                     gkeep[j][e] = g[e];
                     tkeep[j][e] = t[e];
                 }
+            }
+            if constexpr (KEEP_GATES) {
+#pragma unroll
+                for (int e = 0; e < EPV; ++e) gkeep[j][e] = g[e];
             }
             if constexpr (PACKED) {
                 const int rel = (int)(sub_base - lo) + vec_offset<U, EPV, REV>(j, lane);
@@ -271,6 +285,11 @@ __global__ void __launch_bounds__(64 * kMaxWavesPerBlock)
                     g[e] = gkeep[j][e];
                     t[e] = tkeep[j][e];
                 }
+            } else if constexpr (KEEP_GATES) {
+                forget_unpacked(traw[j]);
+                Tr::unpack(traw[j], t);
+#pragma unroll
+                for (int e = 0; e < EPV; ++e) g[e] = gkeep[j][e];
             } else {
                 if constexpr (Tr::kNarrow) {
                     forget_unpacked(graw[j]);

@@ -254,12 +254,14 @@ bool too_few_rows(int64_t rows, int64_t ntiles) {
 // `act`: its gate; `forward`: the forward kernel (3 tensors per tile) or the backward one
 // (5 or 6); `mask_free`: the kernel for rows of whole tiles on the grid.  A compute unit
 // holds one swept workgroup, so what a tile costs in arithmetic is not hidden behind another
-// workgroup's loads: the 16-bit forward kernels that evaluate a sigmoid (or the normalised
-// exponential gate's scale) for eight elements per vector lose when swept (bf16
-// (8,1536,65536), ms, whole rows -> swept: sigmoid 0.79 -> 0.92, interpolating gate 0.80 ->
-// 0.97, normalised exponential 0.81 -> 1.20; the plain exponential gains, and so do the fp32
-// kernels of all gates, 72 -> 78-82 % of peak), and so does a forward kernel with 32 KiB
-// tiles (the normalised exponential gate's, fp32: 6.0 -> 5.3 TB/s).  The backward kernels
+// workgroup's loads: the 16-bit forward kernels that form a token from the gate, a second
+// activation for eight elements per vector, lose when swept (bf16 (8,1536,65536), ms, whole
+// rows -> swept: interpolating gate 0.80 -> 0.91, normalised exponential 0.81 -> 0.94), and so
+// does a sigmoid evaluated in both passes (0.80 -> 0.92), as the copies with masking code
+// do; the mask-free kernel keeps the gates of pass 1 and gains (0.80 -> 0.76, fp16
+// 0.80 -> 0.73; T = 32768 0.40 -> 0.39 / 0.37), like the plain exponential and the fp32
+// kernels of all gates (72 -> 78-82 % of peak).  A forward kernel with 32 KiB tiles loses
+// (the normalised exponential gate's, fp32: 6.0 -> 5.3 TB/s).  The backward kernels
 // move five or six tensors per tile, do well with 32 KiB of each, and request the states
 // behind pass 1 so that they travel while the tile looks at the table; swept, the mask-free
 // 16-bit ones of the sigmoid and the interpolating gate gain (bf16 (8,1536,65536) backward
@@ -286,7 +288,7 @@ bool want_split(SweepClass c, int64_t rows, int64_t row_bytes, int64_t tile_byte
         case SweepClass::kNarrow:
             return row_bytes >= kSweepTileBytes && percent_full >= 66 &&
                    (act == kGateIdentity || act == kGateExp ||
-                    (!forward && mask_free && (act == kGateSigmoid || act == kGateSigmoidLerp)));
+                    (mask_free && (act == kGateSigmoid || (!forward && act == kGateSigmoidLerp))));
         default: return !forward && mask_free && complex_rows_swept(rows, row_bytes);
     }
 }

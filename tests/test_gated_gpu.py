@@ -99,7 +99,7 @@ def test_every_small_T(dtype, with_initial):
 @pytest.mark.parametrize("dtype", DTYPES, ids=IDS)
 @pytest.mark.parametrize("with_initial", [False, True], ids=["zero-start", "initial"])
 @pytest.mark.parametrize("rows,T", [(700, 1024), (600, 4096), (3, 16384), (300, 65536), (7, 16392), (5, 4099),
-                                    (2050, 1031), (2, 65536 + 64), (513, 20000), (1024, 3000)])
+                                    (2050, 1031), (2, 65536 + 64), (513, 20000), (1024, 3000), (513, 32768)])
 def test_tile_and_wave_boundaries(dtype, with_initial, rows, T):
     _run_and_compare(rows, T, dtype, seed=rows + T, what="boundaries", with_initial=with_initial)
 
