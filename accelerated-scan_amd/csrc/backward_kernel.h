@@ -93,6 +93,22 @@ __global__ void __launch_bounds__(64 * kMaxWavesPerBlock)
     __shared__ int split_mailbox[4];  // two mailboxes, taken in turn
     __shared__ u32x4_t parked[SPLIT ? NIN * U * 64 : 1];  // wave 0's raw vectors during its walk back
     __shared__ V parked_values[SPLIT ? 4 * U * 64 : 1];  // and its per-lane scan results
+    // 16-bit gates, 16-wave workgroups: what pass 1 made of the stored gates -- the gate and, for a gate with
+    // values, the factor of the values -- waits for pass 2 in LDS, each lane's own words (128 KiB per workgroup),
+    // instead of being evaluated again.  The compute unit holds this one workgroup (its registers allow no
+    // second), nothing else covers its vector ALU time, its registers are taken, and nine tenths of its LDS
+    // were free.  Measured, bf16 (8,1536,65536) backward, ms, swept kernels: sigmoid 1.34 -> 1.24, interpolating
+    // gate 1.58 -> 1.45, exponential 1.26 -> 1.24, normalised exponential 1.72 -> 1.49; fp16 alike.  With
+    // masking code (T = 65533), swept: sigmoid 1.62 -> 1.39, whole rows: 1.53 -> 1.49, interpolating gate
+    // 1.92 -> 1.82, exponential (swept) 1.47 -> 1.36, normalised exponential 1.93 -> 1.79; T = 40000, whole
+    // rows: 0.90 -> 0.89, 1.14 -> 1.10, 0.88 -> 0.89, 1.09 -> 1.08.  The mask-free kernels that own whole rows
+    // (calls without a table) are at their register limit with 4 KiB per wave and lose (sigmoid 1.46 -> 1.50
+    // with 32 bytes of scratch, exponential 1.44 -> 1.47): they evaluate twice as before.
+    constexpr bool KEEP_LDS = Tr::kNarrow && ACT != kGateIdentity && W == kMaxWavesPerBlock && !ROWS && !PACKED &&
+                              (SPLIT == kSweep || !REGULAR || kGateTakesValues<ACT>);
+    constexpr int NKEEP = kGateTakesValues<ACT> ? 2 : 1;
+    typedef float f32x4_t __attribute__((ext_vector_type(4)));
+    __shared__ f32x4_t kept[KEEP_LDS ? W * U * NKEEP * (EPV / 4) * 64 : 1];
     const unsigned long long split_wait_limit = SPLIT == kSweep ? split->wait_limit : 0ull;  // the longest wait allowed
     int visit_parity = 0;
     for (bool first_visit = true;; first_visit = false, visit_parity ^= 1) {
@@ -308,6 +324,17 @@ __global__ void __launch_bounds__(64 * kMaxWavesPerBlock)
             V a[EPV], d[EPV], x[EPV], a_rest[EPV];  // a_rest = 1 - a, interpolating gate only
             Tr::unpack(araw[j], a);
             activate_with_complement<ACT>(a, a_rest);
+            if constexpr (KEEP_LDS) {
+                f32x4_t* mine = kept + (w * U + j) * (NKEEP * (EPV / 4) * 64) + lane;
+#pragma unroll
+                for (int h = 0; h < EPV / 4; ++h) {
+                    mine[h * 64] = f32x4_t{a[4 * h], a[4 * h + 1], a[4 * h + 2], a[4 * h + 3]};
+                    if constexpr (NKEEP == 2) {
+                        mine[(EPV / 4 + h) * 64] =
+                            f32x4_t{a_rest[4 * h], a_rest[4 * h + 1], a_rest[4 * h + 2], a_rest[4 * h + 3]};
+                    }
+                }
+            }
             Tr::unpack(draw[j], d);
             Tr::unpack(xraw[j], x);
             V hi_edge, lo_edge;
@@ -423,8 +450,21 @@ __global__ void __launch_bounds__(64 * kMaxWavesPerBlock)
                 if constexpr (LERP) forget_unpacked(vraw[j]);
             }
             V a[EPV], d[EPV], x[EPV], a_rest[EPV], v[LERP ? EPV : 1];
-            Tr::unpack(araw[j], a);
-            activate_with_complement<ACT>(a, a_rest);
+            if constexpr (KEEP_LDS) {
+                const f32x4_t* mine = kept + (w * U + j) * (NKEEP * (EPV / 4) * 64) + lane;
+#pragma unroll
+                for (int h = 0; h < EPV / 4; ++h) {
+                    const f32x4_t ka = mine[h * 64];
+                    a[4 * h] = ka.x, a[4 * h + 1] = ka.y, a[4 * h + 2] = ka.z, a[4 * h + 3] = ka.w;
+                    if constexpr (NKEEP == 2) {
+                        const f32x4_t kr = mine[(EPV / 4 + h) * 64];
+                        a_rest[4 * h] = kr.x, a_rest[4 * h + 1] = kr.y, a_rest[4 * h + 2] = kr.z, a_rest[4 * h + 3] = kr.w;
+                    }
+                }
+            } else {
+                Tr::unpack(araw[j], a);
+                activate_with_complement<ACT>(a, a_rest);
+            }
             Tr::unpack(draw[j], d);
             Tr::unpack(xraw[j], x);
             if constexpr (LERP) Tr::unpack(vraw[j], v);

@@ -50,6 +50,14 @@ __global__ void __launch_bounds__(64 * kMaxWavesPerBlock)
     // is left; a workgroup only ever waits for tiles whose owners started before it.
     __shared__ int split_mailbox[4];  // two mailboxes, taken in turn
     __shared__ u32x4_t parked[SPLIT ? 2 * U * 64 : 1];  // wave 0's raw vectors during its walk back
+    // 16-bit gates, swept mask-free kernels: one word per element of what pass 1 made of the stored gates waits
+    // for pass 2 in LDS, each lane's own words (128 KiB per workgroup; the compute unit holds this one workgroup
+    // and most of its LDS was free), instead of being evaluated again -- the gate, or for the interpolating gate
+    // the smaller of gate and complement with the sign of the stored value, from which both come back.
+    constexpr bool KEEP_LDS = Tr::kNarrow && SPLIT == kSweep && REGULAR &&
+                              (ACT == kGateSigmoid || ACT == kGateExp || ACT == kGateSigmoidLerp);
+    typedef float f32x4_t __attribute__((ext_vector_type(4)));
+    __shared__ f32x4_t kept[KEEP_LDS ? W * U * (EPV / 4) * 64 : 1];
     const unsigned long long split_wait_limit = SPLIT == kSweep ? split->wait_limit : 0ull;  // the longest wait allowed
     int visit_parity = 0;
     for (bool first_visit = true;; first_visit = false, visit_parity ^= 1) {
@@ -202,35 +210,51 @@ __global__ void __launch_bounds__(64 * kMaxWavesPerBlock)
         // 16-bit storage with a gate non-linearity: eight exponentials and reciprocals per vector and
         // pass make the vector ALU the limit (about 5.4 TB/s for the interpolating gate), so the
         // activated gates and tokens of pass 1 are kept for pass 2; the raw vectors are dead by then.
-        // The swept kernels have fewer registers to spare (wave 0 parks only its raw vectors), and one
-        // workgroup per compute unit hides none of the arithmetic: the mask-free ones keep the gates alone
-        // where the token needs no activation (measured, bf16 / fp16 (8,1536,65536), ms: sigmoid 0.92 / 0.89
-        // -> 0.76 / 0.73, against 0.80 on whole rows; exponential 0.83 / 0.81 -> 0.74 / 0.75), and gates
-        // and tokens at 2 KiB per wave for the normalised exponential gate (1.23 -> 0.94; whole rows 0.81).
-        // Keeping one word per element of the interpolating gate -- the smaller of gate and complement
-        // with the sign of the stored value -- made that kernel 0.96 -> 0.91, whole rows 0.80: not kept.
+        // The swept kernels have no registers for that (wave 0 parks only its raw vectors), and one workgroup
+        // per compute unit hides none of the arithmetic: the mask-free ones keep a word per element in LDS
+        // (KEEP_LDS above; measured, bf16 / fp16 (8,1536,65536), ms: sigmoid 0.92 / 0.89 -> 0.75 / 0.73,
+        // against 0.79 on whole rows, and 0.76 / 0.74 with the gates kept in registers; exponential
+        // 0.83 / 0.81 -> 0.75 / 0.75; interpolating gate 0.96 / 0.98 -> 0.86 / 0.89, whole rows 0.80), except
+        // the normalised exponential gate's, which needs gate and token, has 2 KiB per wave and keeps both
+        // in registers (1.23 -> 0.94, 0.98 through LDS; whole rows 0.81).
         // Everywhere else unpacking again is cheaper than the registers (the kernels would spill).
-        constexpr bool SWEPT_MASK_FREE = SPLIT == kSweep && REGULAR;
-        constexpr bool KEEP =
-            Tr::kNarrow && ACT != kGateIdentity && !PACKED && (!SPLIT || (SWEPT_MASK_FREE && ACT == kGateExpNorm));
-        constexpr bool KEEP_GATES = Tr::kNarrow && SWEPT_MASK_FREE && (ACT == kGateSigmoid || ACT == kGateExp);
-        V gkeep[KEEP || KEEP_GATES ? U : 1][EPV], tkeep[KEEP ? U : 1][EPV];
+        constexpr bool KEEP = Tr::kNarrow && ACT != kGateIdentity && !PACKED &&
+                              (!SPLIT || (SPLIT == kSweep && REGULAR && ACT == kGateExpNorm));
+        V gkeep[KEEP ? U : 1][EPV], tkeep[KEEP ? U : 1][EPV];
 #pragma unroll
         for (int j = 0; j < U; ++j) {
             V g[EPV], t[EPV];
             Tr::unpack(graw[j], g);
             Tr::unpack(traw[j], t);
-            activate_pair<ACT>(g, t);
+            if constexpr (KEEP_LDS) {
+                V word[EPV];
+                if constexpr (ACT == kGateSigmoidLerp) {
+#pragma unroll
+                    for (int e = 0; e < EPV; ++e) {
+                        float gate, complement;
+                        word[e] = sigmoid_pair_kept(g[e], gate, complement);
+                        g[e] = gate;
+                        t[e] = complement * t[e];
+                    }
+                } else {
+                    activate_pair<ACT>(g, t);
+#pragma unroll
+                    for (int e = 0; e < EPV; ++e) word[e] = g[e];
+                }
+                f32x4_t* mine = kept + (w * U + j) * ((EPV / 4) * 64) + lane;
+#pragma unroll
+                for (int h = 0; h < EPV / 4; ++h) {
+                    mine[h * 64] = f32x4_t{word[4 * h], word[4 * h + 1], word[4 * h + 2], word[4 * h + 3]};
+                }
+            } else {
+                activate_pair<ACT>(g, t);
+            }
             if constexpr (KEEP) {
 #pragma unroll
                 for (int e = 0; e < EPV; ++e) {
                     gkeep[j][e] = g[e];
                     tkeep[j][e] = t[e];
                 }
-            }
-            if constexpr (KEEP_GATES) {
-#pragma unroll
-                for (int e = 0; e < EPV; ++e) gkeep[j][e] = g[e];
             }
             if constexpr (PACKED) {
                 const int rel = (int)(sub_base - lo) + vec_offset<U, EPV, REV>(j, lane);
@@ -285,11 +309,24 @@ __global__ void __launch_bounds__(64 * kMaxWavesPerBlock)
                     g[e] = gkeep[j][e];
                     t[e] = tkeep[j][e];
                 }
-            } else if constexpr (KEEP_GATES) {
+            } else if constexpr (KEEP_LDS) {
                 forget_unpacked(traw[j]);
                 Tr::unpack(traw[j], t);
+                const f32x4_t* mine = kept + (w * U + j) * ((EPV / 4) * 64) + lane;
 #pragma unroll
-                for (int e = 0; e < EPV; ++e) g[e] = gkeep[j][e];
+                for (int h = 0; h < EPV / 4; ++h) {
+                    const f32x4_t word = mine[h * 64];
+                    g[4 * h] = word.x, g[4 * h + 1] = word.y, g[4 * h + 2] = word.z, g[4 * h + 3] = word.w;
+                }
+                if constexpr (ACT == kGateSigmoidLerp) {
+#pragma unroll
+                    for (int e = 0; e < EPV; ++e) {
+                        float gate, complement;
+                        sigmoid_pair_from_kept(g[e], gate, complement);
+                        g[e] = gate;
+                        t[e] = complement * t[e];
+                    }
+                }
             } else {
                 if constexpr (Tr::kNarrow) {
                     forget_unpacked(graw[j]);

@@ -61,6 +61,27 @@ __device__ __forceinline__ void sigmoid_pair(float v, float& gate, float& comple
     complement = positive ? small : large;
 }
 
+// The same pair for kernels that keep it from pass 1 to pass 2 as one word per element: the
+// smaller of the two, with the sign of v, is what comes back.  The larger one is formed
+// as 1 - smaller here and in sigmoid_pair_from_kept, so both passes see the same bits
+// (rounding to nearest puts it within 1 ulp of 1 / (1 + t)).
+__device__ __forceinline__ float sigmoid_pair_kept(float v, float& gate, float& complement) {
+    const float t = __builtin_amdgcn_exp2f(__builtin_fabsf(v) * -1.4426950408889634f);
+    const float small = t * __builtin_amdgcn_rcpf(1.0f + t);
+    const float large = 1.0f - small;
+    const bool positive = v >= 0.0f;
+    gate = positive ? large : small;
+    complement = positive ? small : large;
+    return positive ? small : -small;
+}
+__device__ __forceinline__ void sigmoid_pair_from_kept(float kept, float& gate, float& complement) {
+    const float small = __builtin_fabsf(kept);
+    const float large = 1.0f - small;
+    const bool positive = f2i(kept) >= 0;  // the sign bit, so that a kept -0 is the negative side
+    gate = positive ? large : small;
+    complement = positive ? small : large;
+}
+
 // exp(v) and sqrt(1 - exp(2 v)) for v <= 0 (0 for v > 0).  1 - exp(w), w = 2 v, loses
 // its leading digits to cancellation as w approaches 0, where the gates of long
 // memories live; for w > -1/16 it is summed as -w (1 + w/2 + w^2/6 + w^3/24 + w^4/120)

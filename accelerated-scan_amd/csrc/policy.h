@@ -256,18 +256,20 @@ bool too_few_rows(int64_t rows, int64_t ntiles) {
 // holds one swept workgroup, so what a tile costs in arithmetic is not hidden behind another
 // workgroup's loads: the 16-bit forward kernels that form a token from the gate, a second
 // activation for eight elements per vector, lose when swept (bf16 (8,1536,65536), ms, whole
-// rows -> swept: interpolating gate 0.80 -> 0.91, normalised exponential 0.81 -> 0.94), and so
-// does a sigmoid evaluated in both passes (0.80 -> 0.92), as the copies with masking code
-// do; the mask-free kernel keeps the gates of pass 1 and gains (0.80 -> 0.76, fp16
-// 0.80 -> 0.73; T = 32768 0.40 -> 0.39 / 0.37), like the plain exponential and the fp32
+// rows -> swept: interpolating gate 0.80 -> 0.86, normalised exponential 0.81 -> 0.94), and so
+// does a sigmoid evaluated in both passes (0.79 -> 0.92), as the copies with masking code
+// do; the mask-free kernel keeps the gates of pass 1 in LDS and gains (0.79 -> 0.75, fp16
+// 0.79 -> 0.73; T = 32768 0.40 -> 0.39 / 0.37), like the plain exponential and the fp32
 // kernels of all gates (72 -> 78-82 % of peak).  A forward kernel with 32 KiB tiles loses
 // (the normalised exponential gate's, fp32: 6.0 -> 5.3 TB/s).  The backward kernels
-// move five or six tensors per tile, do well with 32 KiB of each, and request the states
-// behind pass 1 so that they travel while the tile looks at the table; swept, the mask-free
-// 16-bit ones of the sigmoid and the interpolating gate gain (bf16 (8,1536,65536) backward
-// 1.46 -> 1.33 and 1.73 -> 1.59 ms, T = 32768 0.79 -> 0.71 and 0.93 -> 0.79, fp16 alike; the
-// normalised exponential gate's 1.72 -> 1.72), their copies with masking code do not
-// (T = 65533: sigmoid 1.53 -> 1.63, interpolating gate 1.92 -> 1.86).
+// move five or six tensors per tile, do well with 32 KiB of each, request the states behind
+// pass 1 so that they travel while the tile looks at the table, and keep the activated gates
+// of pass 1 in LDS (backward_kernel.h).  Swept, the mask-free 16-bit ones gain (bf16
+// (8,1536,65536) backward, ms, whole rows -> swept: sigmoid 1.46 -> 1.24, interpolating gate
+// 1.73 -> 1.45, normalised exponential 1.72 -> 1.49; T = 32768 0.79 -> 0.63, 0.93 -> 0.74,
+// 0.90 -> 0.75; fp16 alike).  With masking code (T = 65533) the sigmoid's gains, 1.49 -> 1.39,
+// the two with values do not: interpolating gate 1.82 -> 1.85, normalised exponential
+// 1.79 -> 1.82.
 bool want_split(SweepClass c, int64_t rows, int64_t row_bytes, int64_t tile_bytes, int64_t ntiles, int act, bool forward,
                 bool mask_free) {
     if (rows > split_max_rows()) return false;
@@ -287,8 +289,8 @@ bool want_split(SweepClass c, int64_t rows, int64_t row_bytes, int64_t tile_byte
         case SweepClass::kF32: return percent_full >= (forward ? (ntiles == 1 ? 80 : 55) : 50);
         case SweepClass::kNarrow:
             return row_bytes >= kSweepTileBytes && percent_full >= 66 &&
-                   (act == kGateIdentity || act == kGateExp ||
-                    (mask_free && (act == kGateSigmoid || (!forward && act == kGateSigmoidLerp))));
+                   (act == kGateIdentity || act == kGateExp || (act == kGateSigmoid && (mask_free || !forward)) ||
+                    (gate_takes_values(act) && mask_free && !forward));
         default: return !forward && mask_free && complex_rows_swept(rows, row_bytes);
     }
 }
