@@ -104,8 +104,14 @@ __global__ void __launch_bounds__(64 * kMaxWavesPerBlock)
     // rows: 0.90 -> 0.89, 1.14 -> 1.10, 0.88 -> 0.89, 1.09 -> 1.08.  The mask-free kernels that own whole rows
     // (calls without a table) are at their register limit with 4 KiB per wave and lose (sigmoid 1.46 -> 1.50
     // with 32 bytes of scratch, exponential 1.44 -> 1.47): they evaluate twice as before.
-    constexpr bool KEEP_LDS = Tr::kNarrow && ACT != kGateIdentity && W == kMaxWavesPerBlock && !ROWS && !PACKED &&
-                              (SPLIT == kSweep || !REGULAR || kGateTakesValues<ACT>);
+    // The fp32 kernels have half the arithmetic per byte and gain or lose a per cent, swept and mask-free
+    // ((8,1536,T), T = 65536 / 32768, ms: sigmoid 2.49 -> 2.46 / 1.24 -> 1.25, exponential alike, interpolating
+    // gate 2.91 -> 2.92 / 1.44 -> 1.45): only the normalised exponential gate's, with a series and a root in
+    // its factor, keeps them (2.96 -> 2.93 / 1.46 -> 1.46, T = 49152 2.22 -> 2.19).
+    constexpr bool KEEP_LDS =
+        ACT != kGateIdentity && W == kMaxWavesPerBlock && !ROWS && !PACKED &&
+        (Tr::kNarrow ? SPLIT == kSweep || !REGULAR || kGateTakesValues<ACT>
+                     : ACT == kGateExpNorm && SPLIT == kSweep && REGULAR);
     constexpr int NKEEP = kGateTakesValues<ACT> ? 2 : 1;
     typedef float f32x4_t __attribute__((ext_vector_type(4)));
     __shared__ f32x4_t kept[KEEP_LDS ? W * U * NKEEP * (EPV / 4) * 64 : 1];

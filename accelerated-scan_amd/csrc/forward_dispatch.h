@@ -28,7 +28,7 @@ hipError_t launch_forward_split(const void* gates, const void* tokens, void* out
                                 hipStream_t stream) {
     using S = typename Tr::S;
     using TokS = typename Tr::TokS;
-    constexpr int U = forward_split_blocks<ACT>(REGULAR ? SplitTuning<Tr>::U : SplitTuning<Tr>::UG);
+    constexpr int U = forward_split_blocks<Tr, ACT, REGULAR>(REGULAR ? SplitTuning<Tr>::U : SplitTuning<Tr>::UG);
     auto kernel = scan_forward_kernel<Tr, kSplitWaves, U, REV, true, REGULAR, MODE, ACT, false>;
     const unsigned resident = resident_workgroups(kernel, 64 * kSplitWaves, MODE == kSweepRows ? 1 : kMaxWavesPerBlock);
     if (resident == 0) return hipErrorInvalidConfiguration;
@@ -99,8 +99,8 @@ int forward_typed(const void* gates, const void* tokens, void* out, const void* 
         return launch_status(err);
     }
     if (same_lead && ws.ptr != nullptr) {
-        const int64_t SUBS = (int64_t)forward_split_blocks_of(act, SplitTuning<Tr>::U) * 64 * Tr::EPV;
-        const int64_t SUBSG = (int64_t)forward_split_blocks_of(act, SplitTuning<Tr>::UG) * 64 * Tr::EPV;
+        const int64_t SUBS = (int64_t)forward_split_blocks_of<Tr>(act, SplitTuning<Tr>::U, true) * 64 * Tr::EPV;
+        const int64_t SUBSG = (int64_t)forward_split_blocks_of<Tr>(act, SplitTuning<Tr>::UG, false) * 64 * Tr::EPV;
         if constexpr (kSweepClass<Tr> != SweepClass::kComplex) {
             // rows of half a tile: two whole rows per swept tile
             const int per_tile = lead == 0 ? sweep_rows_per_tile(kSweepClass<Tr>, rows, T, kElem, SUBS, act) : 0;

@@ -50,14 +50,21 @@ __global__ void __launch_bounds__(64 * kMaxWavesPerBlock)
     // is left; a workgroup only ever waits for tiles whose owners started before it.
     __shared__ int split_mailbox[4];  // two mailboxes, taken in turn
     __shared__ u32x4_t parked[SPLIT ? 2 * U * 64 : 1];  // wave 0's raw vectors during its walk back
-    // 16-bit gates, swept mask-free kernels: one word per element of what pass 1 made of the stored gates waits
-    // for pass 2 in LDS, each lane's own words (128 KiB per workgroup; the compute unit holds this one workgroup
-    // and most of its LDS was free), instead of being evaluated again -- the gate, or for the interpolating gate
-    // the smaller of gate and complement with the sign of the stored value, from which both come back.
-    constexpr bool KEEP_LDS = Tr::kNarrow && SPLIT == kSweep && REGULAR &&
-                              (ACT == kGateSigmoid || ACT == kGateExp || ACT == kGateSigmoidLerp);
+    // Gates with a non-linearity, swept mask-free kernels: what pass 1 made of the stored values waits for pass 2
+    // in LDS, each lane's own words (up to 128 KiB per workgroup; the compute unit holds this one workgroup and
+    // most of its LDS was free), instead of being evaluated again.  16-bit storage has room for one word per
+    // element: the gate, or for the interpolating gate the smaller of gate and complement with the sign of the
+    // stored value, from which both come back.  fp32 storage has room for gate and token (KEEP_BOTH), which also
+    // frees the registers of the raw vectors, so the normalised exponential gate's kernel takes 4 KiB per wave
+    // like the others (forward_split_blocks): (8,1536,T) fp32 forward, ms, T = 65536 / 49152: 1.60 -> 1.50,
+    // 1.35 -> 1.12; interpolating gate 1.52 -> 1.48, sigmoid 1.51 -> 1.49, exponential 1.49 -> 1.48.
+    constexpr bool kReal = Tr::kNarrow || std::is_same<S, float>::value;
+    constexpr bool KEEP_BOTH = std::is_same<S, float>::value && kGateTakesValues<ACT> && SPLIT != kWholeRows && REGULAR;
+    constexpr bool KEEP_LDS = KEEP_BOTH || (kReal && SPLIT != kWholeRows && REGULAR &&
+                                            (ACT == kGateSigmoid || ACT == kGateExp || ACT == kGateSigmoidLerp));
+    constexpr int NKEEP = KEEP_BOTH ? 2 : 1;
     typedef float f32x4_t __attribute__((ext_vector_type(4)));
-    __shared__ f32x4_t kept[KEEP_LDS ? W * U * (EPV / 4) * 64 : 1];
+    __shared__ f32x4_t kept[KEEP_LDS ? W * U * NKEEP * (EPV / 4) * 64 : 1];
     const unsigned long long split_wait_limit = SPLIT == kSweep ? split->wait_limit : 0ull;  // the longest wait allowed
     int visit_parity = 0;
     for (bool first_visit = true;; first_visit = false, visit_parity ^= 1) {
@@ -219,7 +226,7 @@ __global__ void __launch_bounds__(64 * kMaxWavesPerBlock)
         // in registers (1.23 -> 0.94, 0.98 through LDS; whole rows 0.81).
         // Everywhere else unpacking again is cheaper than the registers (the kernels would spill).
         constexpr bool KEEP = Tr::kNarrow && ACT != kGateIdentity && !PACKED &&
-                              (!SPLIT || (SPLIT == kSweep && REGULAR && ACT == kGateExpNorm));
+                              (!SPLIT || (SPLIT == kSweep && REGULAR && ACT == kGateExpNorm && !KEEP_LDS));
         V gkeep[KEEP ? U : 1][EPV], tkeep[KEEP ? U : 1][EPV];
 #pragma unroll
         for (int j = 0; j < U; ++j) {
@@ -228,7 +235,7 @@ __global__ void __launch_bounds__(64 * kMaxWavesPerBlock)
             Tr::unpack(traw[j], t);
             if constexpr (KEEP_LDS) {
                 V word[EPV];
-                if constexpr (ACT == kGateSigmoidLerp) {
+                if constexpr (ACT == kGateSigmoidLerp && !KEEP_BOTH) {
 #pragma unroll
                     for (int e = 0; e < EPV; ++e) {
                         float gate, complement;
@@ -241,10 +248,13 @@ __global__ void __launch_bounds__(64 * kMaxWavesPerBlock)
 #pragma unroll
                     for (int e = 0; e < EPV; ++e) word[e] = g[e];
                 }
-                f32x4_t* mine = kept + (w * U + j) * ((EPV / 4) * 64) + lane;
+                f32x4_t* mine = kept + (wave_in_tile * U + j) * (NKEEP * (EPV / 4) * 64) + lane;
 #pragma unroll
                 for (int h = 0; h < EPV / 4; ++h) {
                     mine[h * 64] = f32x4_t{word[4 * h], word[4 * h + 1], word[4 * h + 2], word[4 * h + 3]};
+                    if constexpr (KEEP_BOTH) {
+                        mine[(EPV / 4 + h) * 64] = f32x4_t{t[4 * h], t[4 * h + 1], t[4 * h + 2], t[4 * h + 3]};
+                    }
                 }
             } else {
                 activate_pair<ACT>(g, t);
@@ -310,15 +320,21 @@ __global__ void __launch_bounds__(64 * kMaxWavesPerBlock)
                     t[e] = tkeep[j][e];
                 }
             } else if constexpr (KEEP_LDS) {
-                forget_unpacked(traw[j]);
-                Tr::unpack(traw[j], t);
-                const f32x4_t* mine = kept + (w * U + j) * ((EPV / 4) * 64) + lane;
+                if constexpr (!KEEP_BOTH) {
+                    forget_unpacked(traw[j]);
+                    Tr::unpack(traw[j], t);
+                }
+                const f32x4_t* mine = kept + (wave_in_tile * U + j) * (NKEEP * (EPV / 4) * 64) + lane;
 #pragma unroll
                 for (int h = 0; h < EPV / 4; ++h) {
                     const f32x4_t word = mine[h * 64];
                     g[4 * h] = word.x, g[4 * h + 1] = word.y, g[4 * h + 2] = word.z, g[4 * h + 3] = word.w;
+                    if constexpr (KEEP_BOTH) {
+                        const f32x4_t tok = mine[(EPV / 4 + h) * 64];
+                        t[4 * h] = tok.x, t[4 * h + 1] = tok.y, t[4 * h + 2] = tok.z, t[4 * h + 3] = tok.w;
+                    }
                 }
-                if constexpr (ACT == kGateSigmoidLerp) {
+                if constexpr (ACT == kGateSigmoidLerp && !KEEP_BOTH) {
 #pragma unroll
                     for (int e = 0; e < EPV; ++e) {
                         float gate, complement;

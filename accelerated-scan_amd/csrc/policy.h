@@ -228,6 +228,7 @@ int sweep_rows_mode() {
     return v;
 }
 constexpr int64_t kSweepRowsMinBytes = 256ll << 20;  // of one tensor
+constexpr int64_t kShortRowsSweptMinBytes = 128ll << 20;  // of one tensor (want_split)
 template <class Tr>
 constexpr SweepClass kSweepClass = Tr::kNarrow ? SweepClass::kNarrow
                                                : (std::is_same<typename Tr::V, float>::value ? SweepClass::kF32
@@ -261,7 +262,7 @@ bool too_few_rows(int64_t rows, int64_t ntiles) {
 // do; the mask-free kernel keeps the gates of pass 1 in LDS and gains (0.79 -> 0.75, fp16
 // 0.79 -> 0.73; T = 32768 0.40 -> 0.39 / 0.37), like the plain exponential and the fp32
 // kernels of all gates (72 -> 78-82 % of peak).  A forward kernel with 32 KiB tiles loses
-// (the normalised exponential gate's, fp32: 6.0 -> 5.3 TB/s).  The backward kernels
+// (the normalised exponential gate's with masking code, fp32: 6.0 -> 5.3 TB/s).  The backward kernels
 // move five or six tensors per tile, do well with 32 KiB of each, request the states behind
 // pass 1 so that they travel while the tile looks at the table, and keep the activated gates
 // of pass 1 in LDS (backward_kernel.h).  Swept, the mask-free 16-bit ones gain (bf16
@@ -276,7 +277,15 @@ bool want_split(SweepClass c, int64_t rows, int64_t row_bytes, int64_t tile_byte
     if (too_few_rows(rows, ntiles)) return true;
     if (split_forced_min_row_bytes() > 0) return row_bytes >= split_forced_min_row_bytes();
     if (forward && tile_bytes < kSweepTileBytes) return false;
-    if (tile_bytes < kSweepTileBytes && row_bytes < kSweepTileBytes) return false;
+    // 32 KiB tiles (the backward kernels of the gates with values) on rows shorter than 64 KiB: one workgroup
+    // per row does badly there (fp32 interpolating gate, (8,1536,T) backward, ms, whole rows -> swept:
+    // T = 8192 0.41 -> 0.37, 10000 0.52 -> 0.50, 12288 0.62 -> 0.58, 14000 0.74 -> 0.64; (16,1536,8192)
+    // 0.88 -> 0.74; bf16 (8,1536,16384) 0.41 -> 0.37), but a sweep needs a launch worth its start:
+    // (4,1536,8192) 0.203 -> 0.192, (2,1536,8192) 0.102 -> 0.103, (1,1536,8192) 0.052 -> 0.058.
+    if (tile_bytes < kSweepTileBytes && row_bytes < kSweepTileBytes &&
+        (row_bytes < tile_bytes || rows * row_bytes < kShortRowsSweptMinBytes)) {
+        return false;
+    }
     // How full the row's tiles are.  The remainder tile costs little (it is the first of its row in scan
     // order and its empty sub-tiles are skipped) but not nothing, and a row shorter than a tile leaves
     // part of its only tile's workgroup idle.  Measured, fp32 (8,1536,T), TB/s whole rows -> swept:
@@ -288,7 +297,7 @@ bool want_split(SweepClass c, int64_t rows, int64_t row_bytes, int64_t tile_byte
     switch (c) {
         case SweepClass::kF32: return percent_full >= (forward ? (ntiles == 1 ? 80 : 55) : 50);
         case SweepClass::kNarrow:
-            return row_bytes >= kSweepTileBytes && percent_full >= 66 &&
+            return row_bytes >= tile_bytes && percent_full >= 66 &&
                    (act == kGateIdentity || act == kGateExp || (act == kGateSigmoid && (mask_free || !forward)) ||
                     (gate_takes_values(act) && mask_free && !forward));
         default: return !forward && mask_free && complex_rows_swept(rows, row_bytes);
@@ -492,12 +501,19 @@ constexpr int backward_blocks(int blocks) {
 inline int backward_blocks_of(int act, int blocks) { return gate_takes_values(act) && blocks > 2 ? 2 : blocks; }
 
 // The split-row forward kernel of the normalised exponential gate (two activations
-// per element next to the look-back's registers) takes 2 KiB per wave and tile as well.
-template <int ACT>
+// per element next to the look-back's registers) takes 2 KiB per wave and tile as well --
+// except the mask-free fp32 one, which keeps gate and token of pass 1 in LDS and needs
+// no registers for a second evaluation (79 against 113).
+template <class Tr, int ACT, bool REGULAR>
 constexpr int forward_split_blocks(int blocks) {
-    return ACT == kGateExpNorm && blocks > 2 ? 2 : blocks;
+    constexpr bool kept_in_lds = REGULAR && std::is_same<typename Tr::S, float>::value;
+    return ACT == kGateExpNorm && !kept_in_lds && blocks > 2 ? 2 : blocks;
 }
-inline int forward_split_blocks_of(int act, int blocks) { return act == kGateExpNorm && blocks > 2 ? 2 : blocks; }
+template <class Tr>
+inline int forward_split_blocks_of(int act, int blocks, bool regular) {
+    const bool kept_in_lds = regular && std::is_same<typename Tr::S, float>::value;
+    return act == kGateExpNorm && !kept_in_lds && blocks > 2 ? 2 : blocks;
+}
 
 }  // namespace
 }  // namespace ascan

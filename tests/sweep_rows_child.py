@@ -72,8 +72,8 @@ def main():
                     close(what + " d_gates", dg, t_dg, dtype)
                     close(what + " d_initial", ds, t_ds, dtype)
                     checked += 1
-    # the gates with a non-linearity, fp32: the interpolating gate's backward kernel and the normalised
-    # exponential gate's forward kernel take 2 KiB per wave, so their rows are half as long per wave
+    # the gates with a non-linearity, fp32: the backward kernels of the two gates with values take 2 KiB per
+    # wave, so their rows are half as long per wave
     for gate, fwd, bwd, with_values in (
             (_abi.GATE_SIGMOID, seqscan.forward_sigmoid, seqscan.backward_sigmoid, False),
             (_abi.GATE_EXP, seqscan.forward_exp, seqscan.backward_exp, False),
@@ -92,7 +92,7 @@ def main():
             ds = torch.empty_like(s)
             tables = [torch.zeros(4096, dtype=torch.uint8, device=DEVICE) for _ in range(2)]
             what = f"gate {gate} rows={rows} T={T}"
-            per_wave = (512 if gate == _abi.GATE_EXP_NORM else 1024, 512 if with_values else 1024)  # forward, backward
+            per_wave = (1024, 512 if with_values else 1024)  # forward, backward
             shared = [T // n <= 8 for n in per_wave]  # a row on at most half a tile's waves: rows share tiles
             _abi.forward_gated(zg, x, out, gate, workspace=tables[0], initial=s)
             if with_values:

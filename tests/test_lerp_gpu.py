@@ -122,6 +122,18 @@ def test_split_rows(dtype, rows, T):
     _run_and_compare(rows, T, dtype, seed=rows, what="split", with_initial=True)
 
 
+@pytest.mark.parametrize("dtype,rows,T", [(torch.float32, 4096, 8192), (torch.float32, 4100, 10000),
+                                          (torch.bfloat16, 8192, 16384)],
+                         ids=["fp32-4096x8192", "fp32-4100x10000", "bf16-8192x16384"])
+def test_short_rows_of_a_large_launch_are_swept_backward(dtype, rows, T):
+    """Rows of 32 to 64 KiB in tensors of 128 MiB and more (256 MiB in 16-bit storage): the backward kernel,
+    whose tiles are 32 KiB, takes them by ticket instead of one workgroup per row."""
+    from accelerated_scan import _abi
+
+    assert _abi.load().ascan_workspace_bytes(rows, T, _abi.dtype_code(dtype)) > 0
+    _run_and_compare(rows, T, dtype, seed=rows + T, what="short rows swept", with_initial=True)
+
+
 def _random_cases(n, seed, n_dtypes):
     """Seeded random (dtype, rows, T, offsets): short rows in groups, rows of every
     tile count, few long rows; equal offsets for all tensors in 7 of 10 cases."""
