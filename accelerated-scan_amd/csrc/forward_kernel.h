@@ -63,6 +63,11 @@ __global__ void __launch_bounds__(64 * kMaxWavesPerBlock)
     constexpr bool KEEP_LDS = KEEP_BOTH || (kReal && SPLIT != kWholeRows && REGULAR &&
                                             (ACT == kGateSigmoid || ACT == kGateExp || ACT == kGateSigmoidLerp));
     constexpr int NKEEP = KEEP_BOTH ? 2 : 1;
+    // complex64, swept mask-free kernel: every wave's raw vectors wait for pass 2 in LDS (128 KiB), not only
+    // wave 0's during its look at the table; that is what lets the kernel take 4 KiB per wave (128 registers,
+    // no scratch; (8,768,65536) forward swept 2.03 ms with 2 KiB per wave, 1.59 like this, 1.64 on whole rows).
+    constexpr bool STAGE_LDS = !kReal && SPLIT == kSweep && REGULAR;
+    __shared__ u32x4_t staged[STAGE_LDS ? W * U * 2 * 64 : 1];
     typedef float f32x4_t __attribute__((ext_vector_type(4)));
     __shared__ f32x4_t kept[KEEP_LDS ? W * U * NKEEP * (EPV / 4) * 64 : 1];
     const unsigned long long split_wait_limit = SPLIT == kSweep ? split->wait_limit : 0ull;  // the longest wait allowed
@@ -285,6 +290,10 @@ __global__ void __launch_bounds__(64 * kMaxWavesPerBlock)
             totX[j] = read_lane<63>(X);
             exA[j] = shift_up1(A, vone<V>());
             exX[j] = shift_up1(X, vzero<V>());
+            if constexpr (STAGE_LDS) {
+                staged[((wave_in_tile * U + j) * 2) * 64 + lane] = graw[j];
+                staged[((wave_in_tile * U + j) * 2 + 1) * 64 + lane] = traw[j];
+            }
         }
 
         V c;
@@ -292,17 +301,21 @@ __global__ void __launch_bounds__(64 * kMaxWavesPerBlock)
             hand_over(
                 totA, totX, c, k, lane,
                 [&] {
+                    if constexpr (!STAGE_LDS) {
 #pragma unroll
-                    for (int j = 0; j < U; ++j) {
-                        parked[(2 * j) * 64 + lane] = graw[j];
-                        parked[(2 * j + 1) * 64 + lane] = traw[j];
+                        for (int j = 0; j < U; ++j) {
+                            parked[(2 * j) * 64 + lane] = graw[j];
+                            parked[(2 * j + 1) * 64 + lane] = traw[j];
+                        }
                     }
                 },
                 [&] {
+                    if constexpr (!STAGE_LDS) {
 #pragma unroll
-                    for (int j = 0; j < U; ++j) {
-                        graw[j] = parked[(2 * j) * 64 + lane];
-                        traw[j] = parked[(2 * j + 1) * 64 + lane];
+                        for (int j = 0; j < U; ++j) {
+                            graw[j] = parked[(2 * j) * 64 + lane];
+                            traw[j] = parked[(2 * j + 1) * 64 + lane];
+                        }
                     }
                 });
         } else {
@@ -344,6 +357,10 @@ __global__ void __launch_bounds__(64 * kMaxWavesPerBlock)
                     }
                 }
             } else {
+                if constexpr (STAGE_LDS) {
+                    graw[j] = staged[((wave_in_tile * U + j) * 2) * 64 + lane];
+                    traw[j] = staged[((wave_in_tile * U + j) * 2 + 1) * 64 + lane];
+                }
                 if constexpr (Tr::kNarrow) {
                     forget_unpacked(graw[j]);
                     forget_unpacked(traw[j]);

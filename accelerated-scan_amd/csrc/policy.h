@@ -37,7 +37,11 @@ template <> struct Tuning<TraitsC64RealTokens> : Tuning<TraitsC64> {};
 // general).  A swept tile has a fixed cost (ticket, look-back, barriers), so the real
 // dtypes take 4 KiB per wave in every swept kernel, the ones with masking code included
 // (which fit their registers: wave 0 parks its vectors in LDS during the look-back, and a
-// sub-tile that holds nothing of the row is skipped); the complex kernels keep 2 KiB.
+// sub-tile that holds nothing of the row is skipped); the complex kernels keep 2 KiB, except
+// the mask-free forward kernel, whose raw vectors all wait for pass 2 in LDS (forward_kernel.h;
+// the backward kernel with its gate and gradient vectors there and 4 KiB per wave spills 48
+// bytes and is no faster: (8,768,65536) 2.74 -> 2.71 ms, (8,768,32768) 1.31 -> 1.35,
+// (4,1024,8192) 0.228 -> 0.241).
 // (8 KiB per wave in the fp32 forward kernel, half as many tiles: 6.35-6.41 TB/s at
 // (8,1536,65536) against 6.5-6.56, and 40 bytes of scratch.)
 template <class Tr> struct SplitTuning {
@@ -46,7 +50,7 @@ template <class Tr> struct SplitTuning {
 template <> struct SplitTuning<TraitsF32> { static constexpr int U = 4, UG = 4, UB = 4, UBG = 4; };
 template <> struct SplitTuning<TraitsBF16> { static constexpr int U = 4, UG = 4, UB = 4, UBG = 4; };
 template <> struct SplitTuning<TraitsF16> { static constexpr int U = 4, UG = 4, UB = 4, UBG = 4; };
-template <> struct SplitTuning<TraitsC64> { static constexpr int U = 2, UG = 2, UB = 2, UBG = 2; };
+template <> struct SplitTuning<TraitsC64> { static constexpr int U = 4, UG = 2, UB = 2, UBG = 2; };
 template <> struct SplitTuning<TraitsC64RealTokens> : SplitTuning<TraitsC64> {};
 
 // Launch geometry: W waves per row, R rows per workgroup (W*R <= 16).
@@ -234,8 +238,11 @@ constexpr SweepClass kSweepClass = Tr::kNarrow ? SweepClass::kNarrow
                                                : (std::is_same<typename Tr::V, float>::value ? SweepClass::kF32
                                                                                              : SweepClass::kComplex);
 
-// complex64: many rows.  The forward kernel loses when swept whatever the shape (32 KiB tiles, twice
-// the arithmetic per byte: (8,768,65536) 1.65 -> 2.05 ms).  The mask-free backward kernel, which
+// complex64: many rows.  The forward kernel with masking code loses when swept whatever the shape (32 KiB
+// tiles, twice the arithmetic per byte: (8,768,65536) 1.65 -> 2.05 ms); the mask-free one, with 64 KiB tiles
+// and its raw vectors in LDS between the passes, gains a little on rows of two to eight tiles ((8,768,T),
+// T = 65536 / 32768 / 16384: 1.64 -> 1.59, 0.81 -> 0.78, 0.405 -> 0.400; one tile, (4,1024,8192),
+// 0.150 -> 0.154; rows of 1 MiB 3.30 -> 3.33, (1,512,131072) 0.28 -> 0.30).  The mask-free backward kernel, which
 // requests the states behind pass 1, gains on rows of 64 to 512 KiB when there are more than two per
 // compute unit: (8,768,65536) 2.89 -> 2.73 ms, (8,768,32768) 1.41 -> 1.31, (4,1024,8192) 0.235 -> 0.219,
 // (1,2048,32768) 0.476 -> 0.444, (1,512,32768) 0.129 -> 0.123; rows of 1 MiB are level ((1,1024,131072)
@@ -300,7 +307,8 @@ bool want_split(SweepClass c, int64_t rows, int64_t row_bytes, int64_t tile_byte
             return row_bytes >= tile_bytes && percent_full >= 66 &&
                    (act == kGateIdentity || act == kGateExp || (act == kGateSigmoid && (mask_free || !forward)) ||
                     (gate_takes_values(act) && mask_free && !forward));
-        default: return !forward && mask_free && complex_rows_swept(rows, row_bytes);
+        default:
+            return mask_free && complex_rows_swept(rows, row_bytes) && (!forward || row_bytes >= 2 * kSweepTileBytes);
     }
 }
 
