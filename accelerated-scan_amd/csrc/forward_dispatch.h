@@ -30,7 +30,10 @@ hipError_t launch_forward_split(const void* gates, const void* tokens, void* out
     using TokS = typename Tr::TokS;
     constexpr int U = forward_split_blocks<Tr, ACT, REGULAR>(REGULAR ? SplitTuning<Tr>::U : SplitTuning<Tr>::UG);
     auto kernel = scan_forward_kernel<Tr, kSplitWaves, U, REV, true, REGULAR, MODE, ACT, false>;
-    const unsigned resident = resident_workgroups(kernel, 64 * kSplitWaves, MODE == kSweepRows ? 1 : kMaxWavesPerBlock);
+    // one workgroup per compute unit: the mask-free kernels would fit twice since their waves fold the tile's
+    // totals in one row of lanes (63-75 registers), and run no faster that way (fp32 / bf16 (8,1536,65536)
+    // 1.483 / 0.735 ms with two, 1.480 / 0.732 with one)
+    const unsigned resident = resident_workgroups(kernel, 64 * kSplitWaves, 1);
     if (resident == 0) return hipErrorInvalidConfiguration;
     const bool whole_rows = MODE == kSweepRows;
     const hipError_t e = reset_split_table(ws, whole_rows ? 0 : rows, ntiles, stream);

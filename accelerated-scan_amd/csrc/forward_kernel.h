@@ -39,7 +39,7 @@ __global__ void __launch_bounds__(64 * kMaxWavesPerBlock)
     const int64_t len = PACKED ? (rows - first_row < group ? rows - first_row : (int64_t)group) * T : T;
     const int64_t longest = PACKED ? (int64_t)group * T : T;
     // rows start at the same misalignment when their length is a multiple of the grid spacing
-    const int head = REGULAR ? 0 : (ALIGNED ? (longest % G == 0 ? row_lead<Tr>(gates, G) : G - 1) : 0);
+    const int head = REGULAR ? 0 : (ALIGNED ? ((longest & (G - 1)) == 0 ? row_lead<Tr>(gates, G) : G - 1) : 0);
     const int64_t ntiles = tiles_per_row(longest, TILE, head);  // 1 when a tile holds several rows
     // Several rows per tile: a row takes as many waves as it has sub-tiles, the tile as many rows as fit.
     const int row_waves = ROWS ? (int)tiles_per_row(longest, SUB, head) : W;
@@ -68,7 +68,6 @@ __global__ void __launch_bounds__(64 * kMaxWavesPerBlock)
     // no scratch; (8,768,65536) forward swept 2.03 ms with 2 KiB per wave, 1.59 like this, 1.64 on whole rows).
     constexpr bool STAGE_LDS = !kReal && SPLIT == kSweep && REGULAR;
     __shared__ u32x4_t staged[STAGE_LDS ? W * U * 2 * 64 : 1];
-    typedef float f32x4_t __attribute__((ext_vector_type(4)));
     __shared__ f32x4_t kept[KEEP_LDS ? W * U * NKEEP * (EPV / 4) * 64 : 1];
     const unsigned long long split_wait_limit = SPLIT == kSweep ? split->wait_limit : 0ull;  // the longest wait allowed
     int visit_parity = 0;
@@ -113,7 +112,7 @@ __global__ void __launch_bounds__(64 * kMaxWavesPerBlock)
     // fp32 (8,1536,65533), five tiles per row: forward 1.72 ms with the remainder last, 1.50 ms first).
     // A scan that runs down the addresses has it first as things are; one that runs up is addressed
     // from further below instead, so that its last tile ends on the grid boundary above the row.
-    if constexpr (SPLIT == kSweep && !REV && ALIGNED && !REGULAR) lo += ntiles * TILE - (lo + len + G - 1) / G * G;
+    if constexpr (SPLIT == kSweep && !REV && ALIGNED && !REGULAR) lo += ntiles * TILE - ((lo + len + G - 1) & ~(int64_t)(G - 1));  // G is a power of two
     const int64_t hi = lo + len;
     const S* __restrict__ grow = gates + row * T - lo;
     const typename Tr::TokS* __restrict__ trow = tokens + row * T - lo;
@@ -137,7 +136,7 @@ __global__ void __launch_bounds__(64 * kMaxWavesPerBlock)
         if constexpr (ROWS) {
             exchange_carries_rows<V, W, U>(totA, totX, c, slots, wave_in_tile, lane, wave_in_tile - w, row_start);
         } else {
-            exchange_carries_split<V, W, U>(totA, totX, c, slots, w, lane, split, split_wait_limit,
+            exchange_carries_split<V, W, U, true>(totA, totX, c, slots, w, lane, split, split_wait_limit,
                                             split_records(split) + row * ntiles, k, ntiles, row_start, set_aside,
                                             take_back);
         }

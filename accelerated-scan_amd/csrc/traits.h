@@ -15,6 +15,7 @@ namespace {
 // ---------------------------------------------------------------------------
 typedef unsigned int u32x4_t __attribute__((ext_vector_type(4)));  // one 16-byte vector
 typedef unsigned int u32x2_t __attribute__((ext_vector_type(2)));
+typedef float f32x4_t __attribute__((ext_vector_type(4)));  // four words of LDS at a time
 typedef float floatx2_t __attribute__((ext_vector_type(2)));
 typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
 typedef _Float16 halfx2_t __attribute__((ext_vector_type(2)));

@@ -147,6 +147,17 @@ __device__ __forceinline__ V shift_down1(V v, V edge) {
     return dpp_move<kWaveShl1, 0xF>(edge, v);
 }
 
+// v of lane `lane`, a wave-uniform index held in a scalar register.
+__device__ __forceinline__ float read_lane_at(float v, int lane) {
+    return i2f(__builtin_amdgcn_readlane(f2i(v), lane));
+}
+__device__ __forceinline__ cfloat read_lane_at(cfloat v, int lane) {
+    cfloat r;
+    r.re = read_lane_at(v.re, lane);
+    r.im = read_lane_at(v.im, lane);
+    return r;
+}
+
 template <int LANE>
 __device__ __forceinline__ float read_lane(float v) {
     return i2f(__builtin_amdgcn_readlane(f2i(v), LANE));
