@@ -76,7 +76,10 @@ __global__ void __launch_bounds__(64 * kMaxWavesPerBlock)
     int w, slot_base;
     int64_t k_begin = 0, k_end = ntiles;
     if constexpr (SPLIT) {
-        if (!take_split_tile(split, units, ntiles, row, k_begin, split_mailbox + 2 * visit_parity)) break;
+        if (!take_split_tile(split, units, ntiles, row, k_begin, split_mailbox + 2 * visit_parity,
+                             SPLIT == kSweep ? band_rows(ntiles) : 0)) {
+            break;
+        }
         k_end = k_begin + 1;
         int thread = threadIdx.x;
         asm volatile("" : "+v"(thread));  // nothing derived from the wave index is carried from visit to visit

@@ -27,6 +27,20 @@ namespace {
 // A ticket is drawn when the workgroup is ready for the tile, never ahead: a
 // tile held back by its owner's previous tile stalls every later tile of the row.
 //
+// Long rows.  In memory order the tiles in flight at one time -- one per compute
+// unit -- are a few whole rows when rows are long, so a tile has up to 63 earlier
+// tiles of its window in flight beside it and waits for the slowest of them.  The
+// forward kernel therefore hands out rows of 16 tiles and more in bands (band_rows
+// below): ticket n of a band of R rows is tile n / R of the band's row n % R, so the
+// tiles in flight are 256 / R consecutive tiles of each of R rows, and a tile waits
+// for a handful.  A tile's earlier tiles still hold smaller tickets.  Measured, fp32
+// forward, 3.2 GB per tensor, ms, memory order -> bands: 16 tiles per row 1.567 ->
+// 1.53 (R = 64; 1.59-1.84 with R = 32), 32 tiles 1.62 -> 1.51 (R = 32; 1.52 with
+// 64), 64 tiles 1.68 -> 1.54 (1.58 with 64, 1.60 with 128), 128 tiles 1.576 -> 1.52,
+// bf16 64 tiles 1.73 -> 1.55.  The backward kernel, with five tensors per tile,
+// prefers memory order: R = 32 / 64, 16 tiles 2.49 -> 2.9 / 2.61, 64 tiles 2.65 ->
+// 2.62 / 2.72, 128 tiles 2.57 -> 2.63 / 2.69.
+//
 // Because tickets are taken in order, a tile is only ever waited for by
 // workgroups that started after its owner did: progress never depends on a
 // workgroup that has not been dispatched yet, whatever else is running on the
@@ -65,6 +79,9 @@ static_assert(sizeof(SplitTicket) == 64, "ticket line is 64 bytes");
 constexpr int kWholeRows = 0;  // a workgroup owns its rows from start to end
 constexpr int kSweep = 1;      // tiles of all rows by ticket, in memory order; a row's tiles hand their state on
 constexpr int kSweepRows = 2;  // the same for rows of at most half a tile: a tile holds several whole rows
+
+// Rows per band for rows of `ntiles` tiles in the forward kernel; 0 = memory order.
+__device__ __forceinline__ int band_rows(int64_t ntiles) { return ntiles >= 32 ? 32 : (ntiles >= 16 ? 64 : 0); }
 
 constexpr unsigned long long kWaitStepCap = 1000;  // 10 us in 100 MHz ticks
 constexpr int kSplitWindow = 64;                   // tiles per look-back window: one per lane
@@ -134,7 +151,7 @@ __device__ __forceinline__ SplitRecord* split_records(SplitHeader* header) {
 // Hands the workgroup its next tile, or returns false when none is left: thread 0
 // draws the ticket, all threads of the workgroup call this together and get the
 // same answer through `mailbox` (two words of LDS; the caller alternates between two mailboxes from
-// call to call).  rows * ntiles is below 2^31.
+// call to call).  rows * ntiles is below 2^31.  `band`: rows per band, 0 for memory order.
 //
 // The ticket is drawn here, when the workgroup is ready to start on it, so tiles
 // start in ticket order.  (Drawn a tile step ahead, behind the previous tile's
@@ -148,15 +165,24 @@ __device__ __forceinline__ SplitRecord* split_records(SplitHeader* header) {
 // at the far end of the loop body was compiled into a loop in which thread 0 left
 // for its draw while the other lanes went on to read the mailbox it had yet to fill.
 __device__ __forceinline__ bool take_split_tile(SplitHeader* header, int64_t rows, int64_t ntiles, int64_t& row,
-                                                int64_t& k, int* mailbox) {
+                                                int64_t& k, int* mailbox, int band = 0) {
     if (threadIdx.x == 0) {
         const unsigned long long ticket = __hip_atomic_fetch_add(&split_ticket(header)->next, 1ull, __ATOMIC_RELAXED,
                                                                  __HIP_MEMORY_SCOPE_AGENT);
         int got_row = -1, got_k = -1;
         if (ticket < (unsigned long long)(rows * ntiles)) {
             const unsigned n = (unsigned)ticket, per_row = (unsigned)ntiles;
-            got_row = (int)(n / per_row);
-            got_k = (int)(n - (unsigned)got_row * per_row);
+            if (band > 0) {
+                const unsigned band_tiles = (unsigned)band * per_row;
+                const unsigned b = n / band_tiles, i = n - b * band_tiles;
+                const unsigned left = (unsigned)rows - b * (unsigned)band;  // the last band may hold fewer rows
+                const unsigned in_band = left < (unsigned)band ? left : (unsigned)band;
+                got_k = (int)(i / in_band);
+                got_row = (int)(b * (unsigned)band + (i - (unsigned)got_k * in_band));
+            } else {
+                got_row = (int)(n / per_row);
+                got_k = (int)(n - (unsigned)got_row * per_row);
+            }
         }
         mailbox[0] = got_row;
         mailbox[1] = got_k;

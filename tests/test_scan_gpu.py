@@ -824,10 +824,13 @@ def test_linearity_and_concatenation():
 # Split rows: few rows, long sequences, several workgroups per row
 # ---------------------------------------------------------------------------
 @pytest.mark.parametrize("dtype", ALL_DTYPES, ids=ALL_IDS)
-@pytest.mark.parametrize("rows,T", [(1, 1 << 20), (3, 300000), (64, 65536), (128, 65536 + 8), (5, 99999), (2, 16384 * 3)])
+@pytest.mark.parametrize("rows,T", [(1, 1 << 20), (3, 300000), (64, 65536), (128, 65536 + 8), (5, 99999), (2, 16384 * 3),
+                                    (70, 1 << 18), (100, 1 << 19), (33, (1 << 19) + 100)],
+                         ids=lambda v: str(v))
 def test_split_rows(dtype, rows, T):
     """The table-passing kernels (one workgroup per tile) against the fp64 loops,
-    and no wait may have run out."""
+    and no wait may have run out.  The last three shapes have rows of 16 tiles and more, which the
+    forward kernel hands out in bands of 64 or 32 rows (the last band partly filled)."""
     from accelerated_scan import _abi
 
     lib = _abi.load()
