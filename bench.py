@@ -52,8 +52,8 @@ HBM_PEAK_GBPS = 8000.0  # MI355X HBM3E, published peak
 # this script, so the figure is carried over from those runs, not measured in
 # the run that prints it; `traffic_source` in the output says so.
 MEASURED_TRAFFIC_BYTES = {
-    ((8, 1536, 65536), "fp32"): 16134381698,  # FETCH_SIZE 4 729 419, WRITE_SIZE 6 297 745 KiB per dispatch
-    ((8, 1536, 65536), "bf16"): 8070470125,   # FETCH_SIZE 2 366 184, WRITE_SIZE 3 149 131
+    ((8, 1536, 65536), "fp32"): 16134601632,  # FETCH_SIZE 4 729 483, WRITE_SIZE 6 297 835 KiB per dispatch
+    ((8, 1536, 65536), "bf16"): 8070736352,   # FETCH_SIZE 2 366 349, WRITE_SIZE 3 149 061
 }
 TRAFFIC_SOURCE = {
     ((8, 1536, 65536), "fp32"): "profiles/scan_f32_8x1536x65536_fwd_bwd.md (rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE); "
