@@ -240,17 +240,17 @@ constexpr SweepClass kSweepClass = Tr::kNarrow ? SweepClass::kNarrow
 
 // complex64: many rows.  The forward kernel with masking code loses when swept whatever the shape (32 KiB
 // tiles, twice the arithmetic per byte: (8,768,65536) 1.65 -> 2.05 ms); the mask-free one, with 64 KiB tiles
-// and its raw vectors in LDS between the passes, gains a little on rows of two to eight tiles ((8,768,T),
+// and its raw vectors in LDS between the passes, gains on rows of two tiles and more ((8,768,T),
 // T = 65536 / 32768 / 16384: 1.64 -> 1.59, 0.81 -> 0.78, 0.405 -> 0.400; one tile, (4,1024,8192),
-// 0.150 -> 0.154; rows of 1 MiB 3.30 -> 3.33, (1,512,131072) 0.28 -> 0.30).  The mask-free backward kernel, which
-// requests the states behind pass 1, gains on rows of 64 to 512 KiB when there are more than two per
-// compute unit: (8,768,65536) 2.89 -> 2.73 ms, (8,768,32768) 1.41 -> 1.31, (4,1024,8192) 0.235 -> 0.219,
-// (1,2048,32768) 0.476 -> 0.444, (1,512,32768) 0.129 -> 0.123; rows of 1 MiB are level ((1,1024,131072)
-// 0.955 -> 0.966), 256 rows lose (0.124 -> 0.130) and so does the kernel with masking code
-// ((8,768,65533) 2.94 -> 3.18).
-bool complex_rows_swept(int64_t rows, int64_t row_bytes) {
-    return rows >= 512 && row_bytes >= kSweepTileBytes && row_bytes <= 8 * kSweepTileBytes;
-}
+// 0.150 -> 0.154).  The mask-free backward kernel, which requests the states behind pass 1, gains on rows
+// of one tile and more when there are more than two per compute unit: (8,768,65536) 2.89 -> 2.73 ms,
+// (8,768,32768) 1.41 -> 1.31, (4,1024,8192) 0.235 -> 0.219, (1,2048,32768) 0.476 -> 0.444, (1,512,32768)
+// 0.129 -> 0.123; 256 rows lose (0.124 -> 0.130) and so does the kernel with masking code ((8,768,65533)
+// 2.94 -> 3.18).  Rows of 1 MiB and more were level when every lane walked the tile's wave totals and the
+// forward kernel took all rows in memory order; now they gain too, forward + backward, % of peak:
+// (2,1536,131072) 71.1 -> 73.3, (1,1536,262144) 68.7 -> 72.3, (1,768,524288) 67.3 -> 72.4, (1,600,1048576)
+// 62 -> 73, (1,512,131072) 70.5 -> 71.8, (1,1024,131072) 71.2 -> 73.0.
+bool complex_rows_swept(int64_t rows, int64_t row_bytes) { return rows >= 512 && row_bytes >= kSweepTileBytes; }
 
 // Too few rows to occupy the compute units with one workgroup each: with up to 64
 // rows two tiles per row already pay; up to 128, four.

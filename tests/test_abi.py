@@ -108,20 +108,20 @@ def test_workspace_sizing_and_split_entry_validation():
     lib = _abi.load()
     buf = ctypes.create_string_buffer(256)
     p = ctypes.addressof(buf)
-    # short rows, very long complex rows in plenty, and a complex row per compute unit: the plain kernels are the right choice
+    # short rows, and a complex row per compute unit: the plain kernels are the right choice
     assert lib.ascan_workspace_bytes(12288, 4096, 0) == 0
     assert lib.ascan_workspace_bytes(4096, 16384, 1) == 0
     assert lib.ascan_workspace_bytes(12288, 12288, 1) == 0
     assert lib.ascan_workspace_bytes(4, 4096, 0) == 0
-    assert lib.ascan_workspace_bytes(6144, 262144, 3) == 0
     assert lib.ascan_workspace_bytes(256, 65536, 3) == 0
     # long rows in a real dtype are swept in memory order, however many there are (fp32 from 32 KiB on:
     # the backward kernel gains from half-full 64 KiB tiles; 16-bit from 64 KiB on)
     assert lib.ascan_workspace_bytes(12288, 65536, 0) == 128 + 12288 * (65536 // 8192 + 1) * 64
     assert lib.ascan_workspace_bytes(12288, 8192, 0) > 0
     assert lib.ascan_workspace_bytes(12288, 32768, 1) > 0
-    # many complex rows of 64 to 512 KiB: the backward kernel is swept
+    # many complex rows of 64 KiB and more: the backward kernel is swept, and the forward kernel from two tiles on
     assert lib.ascan_workspace_bytes(6144, 65536, 3) == 128 + 6144 * (65536 // 4096 + 1) * 64
+    assert lib.ascan_workspace_bytes(6144, 262144, 3) == 128 + 6144 * (262144 // 4096 + 1) * 64
     assert lib.ascan_workspace_bytes(4096, 8192, 4) > 0
     # 16-bit rows of exactly half a tile, two to a swept tile, once the tensors reach 256 MiB
     assert lib.ascan_workspace_bytes(12288, 16384, 1) > 0

@@ -882,11 +882,12 @@ def test_sweep_of_many_long_rows(dtype, rows, T):
 
 
 @pytest.mark.parametrize("dtype", [torch.complex64, C64_REAL_TOKENS], ids=["c64", "c64-real-tokens"])
-@pytest.mark.parametrize("rows,T", [(600, 8192), (513, 32768), (700, 12288)])
+@pytest.mark.parametrize("rows,T", [(600, 8192), (513, 32768), (700, 12288), (520, 1 << 17)])
 def test_sweep_of_many_complex_rows(dtype, rows, T):
-    """Complex rows of 64 to 512 KiB, 512 of them and more: the forward kernel keeps one workgroup per
-    row, the mask-free backward kernel is swept by ticket (32 KiB tiles, states requested after its
-    first pass).  Both scan directions against the fp64 loops; no wait may have run out."""
+    """Complex rows of 64 KiB and more, 512 of them and more: the mask-free backward kernel is swept by
+    ticket (32 KiB tiles, states requested after its first pass), and so is the mask-free forward kernel
+    from two 64 KiB tiles per row on (in bands of rows from 16 tiles on: the last shape).  Both scan
+    directions against the fp64 loops; no wait may have run out."""
     from accelerated_scan import _abi
 
     lib = _abi.load()
