@@ -296,13 +296,14 @@ bool want_split(SweepClass c, int64_t rows, int64_t row_bytes, int64_t tile_byte
     // How full the row's tiles are.  The remainder tile costs little (it is the first of its row in scan
     // order and its empty sub-tiles are skipped) but not nothing, and a row shorter than a tile leaves
     // part of its only tile's workgroup idle.  Measured, fp32 (8,1536,T), TB/s whole rows -> swept:
-    // forward T = 8192 6.1 -> 5.0, 12000 6.1 -> 5.8, 14000 6.1 -> 6.2, 17000 5.9 -> 5.6, 20000 5.9 -> 6.2;
+    // forward T = 8192 6.1 -> 5.0, 10000 5.86 -> 5.77, 12000 6.08 -> 6.24, 13000 6.08 -> 6.26, 14000 6.1 -> 6.2,
+    // 17000 6.0 -> 5.9, 20000 5.9 -> 6.2;
     // backward (320 KiB per full tile rather than 192) 8192 6.0 -> 6.2, 10000 6.1 -> 6.3, 12000 6.0 -> 6.4,
     // 17000 5.9 -> 6.3; bf16 35000 (53 %) 70 -> 61 % of peak, 40000 (61 %) 72 -> 70, 45000 (69 %) 71 -> 72,
     // 24000 and 16384 (one tile, 73 and 50 % full) 71 -> 69 and 78 -> 63.
     const int64_t percent_full = row_bytes * 100 / (ntiles * tile_bytes);
     switch (c) {
-        case SweepClass::kF32: return percent_full >= (forward ? (ntiles == 1 ? 80 : 55) : 50);
+        case SweepClass::kF32: return percent_full >= (forward ? (ntiles == 1 ? 73 : 55) : 50);
         case SweepClass::kNarrow:
             return row_bytes >= tile_bytes && percent_full >= 66 &&
                    (act == kGateIdentity || act == kGateExp || (act == kGateSigmoid && (mask_free || !forward)) ||
